@@ -1,0 +1,185 @@
+/*
+ * C ABI of libkerops_hip.so -- hand-written gfx950 (MI355X) kernels for the
+ * channels-last 3D depthwise-conv path of neuro-ml/kerops.
+ *
+ * The reference has no FFI: its boundary is the launch of a Triton kernel from
+ * a Python op (`kernel[grid](tensors..., ints..., constexprs..., num_warps=)`).
+ * Each entry point below replaces one such launch site (cited per function,
+ * paths relative to the reference tree) together with the torch glue around it
+ * (per-sample launch loops, zero-filled partial buffers, torch.sum reductions).
+ *
+ * Conventions
+ *  - Activations are dense [N][H][W][D][C] fp16 arrays: the memory of a torch
+ *    (N, C, H, W, D) tensor in channels_last_3d.  H, W, D are the reference's axis
+ *    names in torch-shape order; D is the innermost spatial axis.
+ *  - Every pointer is a device pointer, 16-byte aligned.  C is a power of two.
+ *  - The caller owns every buffer, including the workspace whose size the
+ *    matching *_workspace_bytes function returns.  The library allocates nothing
+ *    and keeps no device state; workspaces need not be zeroed.
+ *  - All work is enqueued on `stream` (a hipStream_t, NULL = default stream); no
+ *    entry point synchronises with the host.
+ *  - Return value: KEROPS_OK or a negative KEROPS_E_* code; the text of the last
+ *    failure on the calling thread is available from kerops_last_error_string().
+ *    Nothing throws.
+ *  - Trailing `tile_*`, `h_chunk` and `blocks` arguments are launch-shape knobs;
+ *    0 selects the built-in choice for gfx950.
+ */
+#ifndef KEROPS_HIP_H
+#define KEROPS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KEROPS_OK 0
+#define KEROPS_E_BADARG (-1)        /* null/misaligned pointer, non-positive size, bad knob */
+#define KEROPS_E_UNSUPPORTED_C (-2) /* channel count the kernel family does not cover */
+#define KEROPS_E_WORKSPACE (-3)     /* workspace missing or smaller than *_workspace_bytes */
+#define KEROPS_E_LAUNCH (-4)        /* HIP reported a launch error */
+
+#define KEROPS_DTYPE_F16 0
+#define KEROPS_DTYPE_F32 1
+
+int kerops_hip_version(void);
+const char* kerops_last_error_string(void);
+
+/* Depthwise 3x3x3 cross-correlation, zero padding 1, stride 1, no bias, fp32
+ * accumulation of all 27 taps, one RNE rounding to fp16:
+ *   y[n,h,w,d,c] = sum_{kh,kw,kd} x[n,h+kh-1,w+kw-1,d+kd-1,c] * wt[kh,kw,kd,c]
+ * wt is [3][3][3][C] fp16.  C in {8,16,32,64,128}.
+ * Replaces the `_DWConv_cl3d_impl[grid](...)` launch and its per-sample Python
+ * loop: kerops/ops/conv/dwconv.py:47-61 (kernel kerops/kernels/dw_conv.py:6-142). */
+int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W, int32_t D,
+                          int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk, void* stream);
+
+/* Depthwise weight gradient, fp32 end to end:
+ *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]
+ * gw is [3][3][3][C] fp32.  Deterministic: per-workgroup partials go to the
+ * workspace and a second kernel adds them in a fixed order.
+ * Replaces the zero-filled partial buffer, the `_DWConv_wgrad_cl3d_impl[grid](...)`
+ * launches and the trailing `grad_w.sum(dim=(0, 1))`:
+ * kerops/ops/conv/dwconv_wgrad.py:54-77 (kernel kerops/kernels/dw_conv.py:147-287). */
+int64_t kerops_dwconv_wgrad_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w,
+                                            int32_t tile_d, int32_t h_chunk);
+int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* workspace, int64_t workspace_bytes,
+                            int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d,
+                            int32_t h_chunk, void* stream);
+
+/* Per-channel mean and mean of squares over M = numel / C voxels, fp32.
+ * Replaces the zero-fill of mean/sqmean and the `_Stats_cl3d_impl[(grid,)](...)`
+ * launch: kerops/ops/stats.py:27-31 (kernel kerops/kernels/stats.py:6-23).
+ * Two-pass and deterministic instead of float atomics. */
+int64_t kerops_stats_workspace_bytes(int64_t M, int32_t C, int32_t blocks);
+int kerops_stats_f16(const void* x, float* mean, float* sqmean, int64_t M, int32_t C, void* workspace,
+                     int64_t workspace_bytes, int32_t blocks, void* stream);
+
+/* dx = 2*x*sqmean_grad[c]/M + mean_grad[c]/M, fp16.
+ * Replaces `_Stats_cl3d_backward_impl[(grid,)](...)`: kerops/ops/stats.py:52-63
+ * (kernel kerops/kernels/stats.py:26-51). */
+int kerops_stats_bwd_f16(const void* x, const float* mean_grad, const float* sqmean_grad, void* dx, int64_t M,
+                         int32_t C, int32_t blocks, void* stream);
+
+/* z = fp16(x + y) and the per-channel mean / mean of squares of z.
+ * Replaces `_AddStats_cl3d_impl[(grid,)](...)`: kerops/ops/addition.py:35-48
+ * (kernel kerops/kernels/addition.py:6-37).  z may alias x (the inplace mode).
+ * Workspace as for kerops_stats_f16. */
+int kerops_add_stats_f16(const void* x, const void* y, void* z, float* mean, float* sqmean, int64_t M, int32_t C,
+                         void* workspace, int64_t workspace_bytes, int32_t blocks, void* stream);
+
+/* out = fp16(add_grad + 2*add_result*sqmean_grad[c]/M + mean_grad[c]/M).
+ * Replaces `_AddStats_cl3d_backward_impl[(grid,)](...)`: kerops/ops/addition.py:75-88
+ * (kernel kerops/kernels/addition.py:41-75). */
+int kerops_add_stats_bwd_f16(const void* add_grad, const float* mean_grad, const float* sqmean_grad,
+                             const void* add_result, void* out, int64_t M, int32_t C, int32_t blocks, void* stream);
+
+/* y = fp16(max(float(x) * wv[c] + bv[c], 0)); wv, bv are fp32 [C].
+ * Replaces `_ApplyBNReLU_cl3d_impl[(grid,)](...)`: kerops/ops/bnrelu.py:30-41
+ * (kernel kerops/kernels/bnrelu.py:6-31). */
+int kerops_bnrelu_fwd_f16(const void* x, const float* wv, const float* bv, void* y, int64_t M, int32_t C,
+                          int32_t blocks, void* stream);
+
+/* keep = (x*wv[c] > -bv[c]); g' = g*keep; dx = fp16(wv[c]*g'); dW[c] = sum x*g';
+ * dB[c] = sum g' (fp32, deterministic two-pass).
+ * Replaces the zero-fill of the two gradients and
+ * `_ApplyBNReLU_cl3d_backward_impl[(grid,)](...)`: kerops/ops/bnrelu.py:64-82
+ * (kernel kerops/kernels/bnrelu.py:35-71).  Workspace as for kerops_stats_f16. */
+int kerops_bnrelu_bwd_f16(const void* x, const float* wv, const float* bv, const void* g, void* dx, float* dW,
+                          float* dB, int64_t M, int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks,
+                          void* stream);
+
+/* 2x2x2 stride-2 average pool with ceil_mode (edge windows divide by the number
+ * of existing voxels), y dense [N][ceil(H/2)][ceil(W/2)][ceil(D/2)][C] fp16, plus
+ * mean / mean of squares of the fp32 pooled values.
+ * Replaces the zero-fill of mean/sqmean and
+ * `_AvgPoolCeilStats_cl3d_impl[(N, H/2, W/2)](...)`: kerops/ops/avgpool.py:33-60
+ * (kernel kerops/kernels/avgpool.py:6-93). */
+int64_t kerops_avgpool_ceil_stats_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
+                                                  int32_t blocks);
+int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H, int32_t W,
+                                  int32_t D, int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks,
+                                  void* stream);
+
+/* dx[every existing voxel of a window] =
+ *   fp16((inpgrad + meangrad[c]/Mo + 2*output*sqmeangrad[c]/Mo) / count),
+ * Mo = N*ceil(H/2)*ceil(W/2)*ceil(D/2); (N,H,W,D) is the shape of dx.
+ * Replaces the zero-filled outgrad and
+ * `_AvgPoolCeilStats_cl3d_backward_impl[(N, H/2, W/2)](...)`:
+ * kerops/ops/avgpool.py:93-122 (kernel kerops/kernels/avgpool.py:97-185). */
+int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad, const float* sqmeangrad,
+                                      const void* output, void* dx, int32_t N, int32_t H, int32_t W, int32_t D,
+                                      int32_t C, int32_t blocks, void* stream);
+
+/* u8 = (uint8)(((clip(float(x), -window, window) + window) / (2*window)) * 255),
+ * each step one IEEE fp32 operation, conversion by truncation.  dtype is the
+ * KEROPS_DTYPE_* tag of x.  Flat over numel elements.
+ * Replaces `_QuantUint8Window_impl[(numblocks,)](...)`:
+ * kerops/ops/quantization.py:19 (kernel kerops/kernels/quantization.py:6-27). */
+int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int64_t numel, float window, int32_t blocks,
+                           void* stream);
+
+/* out = float(u8) * (2*window/255) - window (scale formed once in fp32; one
+ * multiply, one subtract), stored as dtype.
+ * Replaces `_DequantUint8Window_impl[(numblocks,)](...)`:
+ * kerops/ops/quantization.py:34 (kernel kerops/kernels/quantization.py:31-49). */
+int kerops_dequant_u8_window(const void* q, void* out, int32_t dtype, int64_t numel, float window, int32_t blocks,
+                             void* stream);
+
+/* max |y| over numel fp16 values, written to *absmax (device fp32).  No reference
+ * counterpart: first pass of the symmetric int8 quantiser of the fused-block
+ * configuration.  Workspace: kerops_absmax_workspace_bytes(blocks). */
+int64_t kerops_absmax_workspace_bytes(int32_t blocks);
+int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, void* workspace, int64_t workspace_bytes,
+                      int32_t blocks, void* stream);
+
+/* q = clamp(rint_half_even(float(y) / (absmax/127)), -127, 127) as int8, with
+ * absmax read from device memory; absmax == 0 gives q = 0.  No reference
+ * counterpart: second pass of the symmetric int8 quantiser. */
+int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t numel, int32_t blocks, void* stream);
+
+/* Pointwise (1x1x1) channel mixing on MFMA:
+ *   out[v, co] = fp16(sum_ci act(x[v, ci]) * Wm[ci, co]) (+ add[v, co], fp16 add)
+ * x dense [V][Cin] fp16, Wm [Cin][Cout] fp16, add/out dense [V][Cout] fp16;
+ * act = ReLU when relu_in != 0; add may be NULL.  Cin, Cout in {16,32,64,128}.
+ * Replaces `_ReLULinearAdd[(grid,)](...)`: kerops/ops/linear/relu_linear_add.py:46-50
+ * (kernel kerops/kernels/linear.py:6-45). */
+int kerops_pointwise_f16(const void* x, const void* Wm, const void* add, void* out, int64_t V, int32_t Cin,
+                         int32_t Cout, int32_t relu_in, void* stream);
+
+/* Fused depthwise-separable block (no single reference counterpart; composition
+ * of DWConv, a folded inference BN, ReLU and the pointwise GEMM above):
+ *   t = fp16(relu(dwconv(x, wt) * scale[c] + shift[c]));  y = fp16(t @ Wm)
+ * and the running max |y| written to *absmax (device fp32) for the int8 pass.
+ * x [N][H][W][D][Cin], y [N][H][W][D][Cout].  Cin = 64, Cout = 128 built in.
+ * Workspace: kerops_dwsep_block_workspace_bytes(...). */
+int64_t kerops_dwsep_block_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t Cin, int32_t Cout);
+int kerops_dwsep_block_f16(const void* x, const void* wt, const float* scale, const float* shift, const void* Wm,
+                           void* y, float* absmax, int32_t N, int32_t H, int32_t W, int32_t D, int32_t Cin,
+                           int32_t Cout, void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* KEROPS_HIP_H */

@@ -1,0 +1,221 @@
+// 2x2x2 stride-2 ceil-mode average pool with per-channel statistics of the pooled
+// values, and its backward, on [N][H][W][D][C] fp16 (gfx950).
+//
+// One thread produces one chunk of V = min(8, C) channels of one pooled voxel: it reads
+// the (up to) eight input chunks of the window as 16-byte accesses, adds the D pair first
+// and then the four (h, w) rows in the order (0,0) (0,1) (1,0) (1,1), divides by the number
+// of voxels that exist in the window and stores the RNE-rounded fp16 chunk.  Consecutive
+// lanes take consecutive (d_out, channel-group) chunks, so the two D-taps of a wavefront
+// together cover contiguous input memory.  The statistics use the unrounded fp32 pooled
+// values and the same deterministic two-pass reduction as the other per-channel sums.
+#include "common.hpp"
+
+namespace kerops {
+
+struct PoolDims {
+    int N, H, W, D, Ho, Wo, Do, C, CG;
+};
+
+template <int V>
+__global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_t* __restrict__ x,
+                                                                     half_t* __restrict__ y, float* __restrict__ ws,
+                                                                     const PoolDims p, int64_t nchunks)
+{
+    typedef typename HVec<V>::type hv;
+    __shared__ float red[kStreamWaves * 2 * 64 * V];
+    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
+    float acc[2][V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[0][j] = acc[1][j] = 0.0f;
+    const int64_t sD = p.CG, sW = (int64_t)p.D * p.CG, sH = (int64_t)p.W * sW, sN = (int64_t)p.H * sH;  // in chunks
+
+    for (int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x; i < nchunks; i += T) {
+        int64_t r = i;
+        const int cg = (int)(r % p.CG);
+        r /= p.CG;
+        const int dO = (int)(r % p.Do);
+        r /= p.Do;
+        const int wO = (int)(r % p.Wo);
+        r /= p.Wo;
+        const int hO = (int)(r % p.Ho);
+        const int n = (int)(r / p.Ho);
+        const bool h1 = 2 * hO + 1 < p.H, w1 = 2 * wO + 1 < p.W, d1 = 2 * dO + 1 < p.D;
+        const int64_t base = n * sN + (2 * hO) * sH + (2 * wO) * sW + (2 * dO) * sD + cg;
+        hv v[2][2][2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
+                    hv t;
+#pragma unroll
+                    for (int j = 0; j < V; ++j) t[j] = (half_t)0;
+                    if (ok) t = ld<V>(x, base + a * sH + b * sW + e * sD);
+                    v[a][b][e] = t;
+                }
+        const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
+        hv o;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            float s = 0.0f;
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) s += (float)v[a][b][0][j] + (float)v[a][b][1][j];
+            const float m = __fdiv_rn(s, cnt);
+            o[j] = (half_t)m;
+            acc[0][j] += m;
+            acc[1][j] = __builtin_fmaf(m, m, acc[1][j]);
+        }
+        st<V>(y, i, o);
+    }
+    block_channel_partials<2, V>(acc, p.CG, red, ws + (int64_t)blockIdx.x * 2 * p.CG * V);
+}
+
+template <int V>
+__global__ __launch_bounds__(kStreamThreads) void avgpool_bwd_kernel(const half_t* __restrict__ inpgrad,
+                                                                     const float* __restrict__ meangrad,
+                                                                     const float* __restrict__ sqmeangrad,
+                                                                     const half_t* __restrict__ output,
+                                                                     half_t* __restrict__ dx, const PoolDims p,
+                                                                     int64_t nchunks, float fMo)
+{
+    typedef typename HVec<V>::type hv;
+    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
+    const int64_t sD = p.CG, sW = (int64_t)p.D * p.CG, sH = (int64_t)p.W * sW, sN = (int64_t)p.H * sH;
+    int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
+    const int cg0 = (int)(i % p.CG);
+    float mg[V], sg[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        mg[j] = __fdiv_rn(meangrad[cg0 * V + j], fMo);
+        sg[j] = sqmeangrad[cg0 * V + j];
+    }
+    for (; i < nchunks; i += T) {
+        int64_t r = i / p.CG;
+        const int dO = (int)(r % p.Do);
+        r /= p.Do;
+        const int wO = (int)(r % p.Wo);
+        r /= p.Wo;
+        const int hO = (int)(r % p.Ho);
+        const int n = (int)(r / p.Ho);
+        const bool h1 = 2 * hO + 1 < p.H, w1 = 2 * wO + 1 < p.W, d1 = 2 * dO + 1 < p.D;
+        const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
+        const hv g = ld<V>(inpgrad, i), o = ld<V>(output, i);
+        hv res;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const float s = __fdiv_rn(__fmul_rn(__fmul_rn(2.0f, (float)o[j]), sg[j]), fMo);
+            const float t = __fadd_rn(__fadd_rn((float)g[j], mg[j]), s);
+            res[j] = (half_t)__fdiv_rn(t, cnt);
+        }
+        const int64_t base = n * sN + (2 * hO) * sH + (2 * wO) * sW + (2 * dO) * sD + cg0;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
+                    if (ok) st<V>(dx, base + a * sH + b * sW + e * sD, res);
+                }
+    }
+}
+
+static int pool_plan(const char* op, int N, int H, int W, int D, int C, int* blocks, PoolDims* p, int64_t* nchunks,
+                     int64_t* need)
+{
+    if (N <= 0 || H <= 0 || W <= 0 || D <= 0 || C <= 0 || !is_pow2(C)) {
+        set_error("%s: extents must be positive and C a power of two", op);
+        return KEROPS_E_BADARG;
+    }
+    if (C > kMaxReduceChannels) {
+        set_error("%s: built for C <= %d (got %d)", op, kMaxReduceChannels, C);
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    const int V = C >= 8 ? 8 : C;
+    p->N = N;
+    p->H = H;
+    p->W = W;
+    p->D = D;
+    p->Ho = (H + 1) / 2;
+    p->Wo = (W + 1) / 2;
+    p->Do = (D + 1) / 2;
+    p->C = C;
+    p->CG = C / V;
+    *nchunks = (int64_t)N * p->Ho * p->Wo * p->Do * p->CG;
+    if (*blocks <= 0) *blocks = stream_blocks_default(*nchunks);
+    if (*blocks > 65536) {
+        set_error("%s: blocks must be <= 65536", op);
+        return KEROPS_E_BADARG;
+    }
+    *need = (int64_t)(*blocks) * 2 * C * (int64_t)sizeof(float);
+    return KEROPS_OK;
+}
+
+}  // namespace kerops
+
+using namespace kerops;
+
+extern "C" int64_t kerops_avgpool_ceil_stats_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
+                                                             int32_t blocks)
+{
+    PoolDims p;
+    int64_t nchunks = 0, need = 0;
+    int rc = pool_plan("avgpool_ceil_stats", N, H, W, D, C, &blocks, &p, &nchunks, &need);
+    return rc != KEROPS_OK ? rc : need;
+}
+
+extern "C" int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H,
+                                             int32_t W, int32_t D, int32_t C, void* workspace,
+                                             int64_t workspace_bytes, int32_t blocks, void* stream)
+{
+    PoolDims p;
+    int64_t nchunks = 0, need = 0;
+    int rc = pool_plan("avgpool_ceil_stats", N, H, W, D, C, &blocks, &p, &nchunks, &need);
+    if (rc != KEROPS_OK) return rc;
+    if (!x || !y || !mean || !sqmean || !aligned16(x) || !aligned16(y)) {
+        set_error("avgpool_ceil_stats: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
+        set_error("avgpool_ceil_stats: workspace of %lld bytes required, %lld given", (long long)need,
+                  (long long)workspace_bytes);
+        return KEROPS_E_WORKSPACE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    float* ws = (float*)workspace;
+    KEROPS_DISPATCH_V(C, {
+        hipLaunchKernelGGL((avgpool_fwd_kernel<V>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x,
+                           (half_t*)y, ws, p, nchunks);
+    });
+    rc = check_launch("avgpool_ceil_stats");
+    if (rc != KEROPS_OK) return rc;
+    const double Mo = (double)N * p.Ho * p.Wo * p.Do;
+    launch_reduce_rows(ws, blocks, 2 * C, mean, sqmean, C, 1.0 / Mo, s);
+    return check_launch("avgpool_ceil_stats");
+}
+
+extern "C" int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad, const float* sqmeangrad,
+                                                 const void* output, void* dx, int32_t N, int32_t H, int32_t W,
+                                                 int32_t D, int32_t C, int32_t blocks, void* stream)
+{
+    PoolDims p;
+    int64_t nchunks = 0, need = 0;
+    int rc = pool_plan("avgpool_ceil_stats_bwd", N, H, W, D, C, &blocks, &p, &nchunks, &need);
+    if (rc != KEROPS_OK) return rc;
+    if (!inpgrad || !meangrad || !sqmeangrad || !output || !dx || !aligned16(inpgrad) || !aligned16(output) ||
+        !aligned16(dx)) {
+        set_error("avgpool_ceil_stats_bwd: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    const float fMo = (float)((int64_t)N * p.Ho * p.Wo * p.Do);
+    KEROPS_DISPATCH_V(C, {
+        hipLaunchKernelGGL((avgpool_bwd_kernel<V>), dim3(blocks), dim3(kStreamThreads), 0, (hipStream_t)stream,
+                           (const half_t*)inpgrad, meangrad, sqmeangrad, (const half_t*)output, (half_t*)dx, p,
+                           nchunks, fMo);
+    });
+    return check_launch("avgpool_ceil_stats_bwd");
+}

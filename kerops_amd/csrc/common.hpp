@@ -1,0 +1,190 @@
+// Shared device/host helpers for the gfx950 kernels of kerops_amd.
+//
+// Data layout everywhere: a torch (N, C, H, W, D) channels_last_3d tensor is the
+// dense array [N][H][W][D][C] of fp16; D is the innermost spatial axis and the
+// C channels of one voxel are contiguous (2*C bytes).  All kernels move data as
+// 16-byte chunks of 8 consecutive channels ("c8 chunks"): consecutive lanes of a
+// 64-wide wavefront take consecutive chunks, so every global access of a
+// wavefront is one contiguous 1 KiB run.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/kerops_hip.h"
+
+namespace kerops {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// ---- error reporting (host) -------------------------------------------------
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+// ---- small host helpers -----------------------------------------------------
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The 8 XCDs of the chip receive workgroups round-robin (workgroup b runs on XCD
+// b % 8) and each XCD has a private L2.  remap_xcd turns the hardware workgroup
+// index into a logical tile index such that each XCD walks one contiguous range of
+// logical tiles: neighbouring tiles (which share halo voxels) then meet in the same
+// L2 instead of being fetched once per XCD.
+__device__ __forceinline__ uint32_t remap_xcd(uint32_t b, uint32_t nblocks)
+{
+    constexpr uint32_t kXcd = 8;
+    uint32_t per = (nblocks + kXcd - 1) / kXcd;  // logical tiles per XCD (last range may be short)
+    uint32_t xcd = b % kXcd;
+    uint32_t idx = b / kXcd;
+    // ranges [xcd*per, (xcd+1)*per); the tail ranges can exceed nblocks, so the
+    // grid is launched with per*kXcd workgroups and the caller drops ids >= nblocks.
+    return xcd * per + idx;
+}
+static inline uint32_t xcd_padded_grid(uint32_t nblocks) { return ((nblocks + 7u) / 8u) * 8u; }
+
+// ---- 16-byte chunk access ---------------------------------------------------
+__device__ __forceinline__ half8_t load_c8(const half_t* p) { return *reinterpret_cast<const half8_t*>(p); }
+__device__ __forceinline__ void store_c8(half_t* p, half8_t v) { *reinterpret_cast<half8_t*>(p) = v; }
+
+// Streaming (non-temporal) variants for data that is touched exactly once.
+__device__ __forceinline__ half8_t load_c8_nt(const half_t* p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(p));
+}
+__device__ __forceinline__ void store_c8_nt(half_t* p, half8_t v)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(p));
+}
+
+// ---- wavefront reductions -----------------------------------------------------
+// Sum over the lanes of a wavefront whose index differs only in bits >= log2(stride_lo):
+// i.e. lanes l and l' are combined when l % stride_lo == l' % stride_lo.
+template <int STRIDE_LO>
+__device__ __forceinline__ float wave_sum_stride(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= STRIDE_LO; off >>= 1) {
+        v += __shfl_xor(v, off, 64);
+    }
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        v = fmaxf(v, __shfl_xor(v, off, 64));
+    }
+    return v;
+}
+
+}  // namespace kerops
+
+// ---- per-channel streaming helpers (stream_ops.hip, avgpool.hip) --------------
+namespace kerops {
+
+// V consecutive fp16 channels moved as one access; V = min(8, C).
+template <int V>
+struct HVec {
+    typedef _Float16 type __attribute__((ext_vector_type(V)));
+};
+template <>
+struct HVec<1> {
+    struct type {
+        _Float16 s;
+        __device__ __forceinline__ _Float16& operator[](int) { return s; }
+        __device__ __forceinline__ const _Float16& operator[](int) const { return s; }
+    };
+};
+
+// Run the statement list with a constexpr `V` = min(8, C) in scope (C a power of two).
+#define KEROPS_DISPATCH_V(C, ...)  \
+    do {                           \
+        if ((C) >= 8) {            \
+            constexpr int V = 8;   \
+            __VA_ARGS__;           \
+        } else if ((C) == 4) {     \
+            constexpr int V = 4;   \
+            __VA_ARGS__;           \
+        } else if ((C) == 2) {     \
+            constexpr int V = 2;   \
+            __VA_ARGS__;           \
+        } else {                   \
+            constexpr int V = 1;   \
+            __VA_ARGS__;           \
+        }                          \
+    } while (0)
+
+template <int V>
+__device__ __forceinline__ typename HVec<V>::type ld(const _Float16* p, int64_t chunk)
+{
+    return *reinterpret_cast<const typename HVec<V>::type*>(p + chunk * V);
+}
+template <int V>
+__device__ __forceinline__ void st(_Float16* p, int64_t chunk, const typename HVec<V>::type& v)
+{
+    *reinterpret_cast<typename HVec<V>::type*>(p + chunk * V) = v;
+}
+
+constexpr int kStreamThreads = 256;
+constexpr int kStreamWaves = kStreamThreads / kWave;
+constexpr int kMaxReduceChannels = 512;  // per-channel reductions: C/V <= 64 lane groups
+
+// Default workgroup count of the persistent stream kernels: 8 workgroups of 4
+// wavefronts per CU fill every SIMD's 8 wavefront slots on a 256-CU part.
+static inline int stream_blocks_default(int64_t work_items)
+{
+    int64_t b = ceil_div64(work_items, kStreamThreads);
+    if (b > 2048) b = 2048;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+// Sum NACC*V per-thread accumulators over the threads of a workgroup that own the same
+// channel group (thread t owns group t % CG, CG <= 64 a power of two) and write the
+// workgroup's partial [NACC][CG*V] to `dst`.  `red` is LDS of kStreamWaves*NACC*CG*V floats.
+template <int NACC, int V>
+__device__ __forceinline__ void block_channel_partials(float (&acc)[NACC][V], int CG, float* red, float* dst)
+{
+    const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
+    const int cols = CG * V;
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            float v = acc[a][j];
+            for (int off = 32; off >= CG; off >>= 1) v += __shfl_xor(v, off, 64);
+            acc[a][j] = v;
+        }
+    if (lane < CG) {
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int j = 0; j < V; ++j) red[(wave * NACC + a) * cols + lane * V + j] = acc[a][j];
+    }
+    __syncthreads();
+    for (int o = t; o < NACC * cols; o += kStreamThreads) {
+        float s = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < kStreamWaves; ++wv) s += red[wv * NACC * cols + o];
+        dst[o] = s;
+    }
+}
+
+// out[j] = scale * sum_r ws[r*ncols + j] for j < ncols, summed in fp64 in a fixed order;
+// columns [0, split) go to out0, the rest to out1.  (Kernel lives in core.hip.)
+void launch_reduce_rows(const float* ws, int nrows, int ncols, float* out0, float* out1, int split, double scale,
+                        hipStream_t stream);
+
+}  // namespace kerops

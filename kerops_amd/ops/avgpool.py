@@ -1,0 +1,82 @@
+"""AvgPoolCeilStats / AvgPoolCeilStatsBackward: 2x2x2 ceil-mode average pooling fused with
+per-channel statistics of the pooled tensor.
+
+Host side of kerops_avgpool_ceil_stats_f16 / kerops_avgpool_ceil_stats_bwd_f16; names,
+positional arguments, asserts and results as kerops/ops/avgpool.py:11-122 of the reference.
+"""
+from math import ceil
+
+import torch
+
+from .. import _lib
+from ..settings import ConfigurableArg, configure, get_l1_cache
+from ._common import next_power_of_2, require_cuda
+
+
+@configure(l1_cache_bytes=get_l1_cache, num_warps=2, blocks=0)
+def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg):
+    """Returns (pooled fp16 (N,C,ceil(H/2),ceil(W/2),ceil(D/2)) channels_last_3d, mean, sqmean)."""
+    num_channels = x.shape[1]
+    input_d = x.shape[-1]
+    MAX_SIZE = l1_cache_bytes // x.element_size()
+
+    # the reference's kernel holds a whole D row per program; the limit is kept so the
+    # same inputs are rejected (kerops/ops/avgpool.py:20), the gfx950 kernel has none
+    assert input_d * num_channels <= MAX_SIZE
+    assert num_channels == next_power_of_2(num_channels)
+    assert x.ndim == 5
+    assert x.dtype == torch.float16
+    assert x.is_contiguous(memory_format=torch.channels_last_3d)
+    require_cuda(x)
+
+    n, _, h, w, d = x.shape
+    out_shape = [n] + [ceil(sh / 2) for sh in x.shape[2:]] + [num_channels]
+    output = torch.empty(out_shape, dtype=torch.float16, device=x.device).permute(0, 4, 1, 2, 3)
+    mean = torch.empty(num_channels, device=x.device, dtype=torch.float32)
+    sqmean = torch.empty(num_channels, device=x.device, dtype=torch.float32)
+    ws_bytes = _lib.query('kerops_avgpool_ceil_stats_workspace_bytes', n, h, w, d, num_channels, int(blocks))
+    ws = _lib.workspace(ws_bytes, x.device)
+    _lib.call('kerops_avgpool_ceil_stats_f16', x.data_ptr(), output.data_ptr(), mean.data_ptr(), sqmean.data_ptr(),
+              n, h, w, d, num_channels, ws.data_ptr(), ws_bytes, int(blocks), _lib.stream_of(x))
+    return output, mean, sqmean
+
+
+@configure(l1_cache_bytes=get_l1_cache, num_warps=4, blocks=0)
+def AvgPoolCeilStatsBackward(
+    inpgrad,
+    meangrad,
+    sqmeangrad,
+    output,
+    outgrad_shape,
+    *,
+    l1_cache_bytes: ConfigurableArg,
+    num_warps: ConfigurableArg,
+    blocks: ConfigurableArg,
+):
+    """Gradient w.r.t. the pooling input, fp16, shape `outgrad_shape`, channels_last_3d."""
+    MAX_SIZE = l1_cache_bytes // inpgrad.element_size()
+    bsize, num_channels, h_outgrad, w_outgrad, d_outgrad = outgrad_shape
+
+    assert d_outgrad * num_channels <= MAX_SIZE
+    assert inpgrad.shape[1] == num_channels
+    assert inpgrad.shape == output.shape
+    assert meangrad.numel() == sqmeangrad.numel() == num_channels
+    assert inpgrad.ndim == 5
+    assert inpgrad.is_contiguous(memory_format=torch.channels_last_3d)
+    assert output.is_contiguous(memory_format=torch.channels_last_3d)
+    assert num_channels == next_power_of_2(num_channels)
+    assert inpgrad.dtype == output.dtype == torch.float16
+    assert meangrad.dtype == sqmeangrad.dtype == torch.float32
+    assert list(inpgrad.shape[2:]) == [ceil(s / 2) for s in (h_outgrad, w_outgrad, d_outgrad)]
+    assert inpgrad.shape[0] == bsize
+    require_cuda(inpgrad, output, meangrad, sqmeangrad)
+
+    outgrad = torch.empty(
+        [bsize, h_outgrad, w_outgrad, d_outgrad, num_channels], dtype=torch.float16, device=inpgrad.device
+    ).permute(0, 4, 1, 2, 3)
+    meangrad = meangrad.contiguous()
+    sqmeangrad = sqmeangrad.contiguous()
+    _lib.call('kerops_avgpool_ceil_stats_bwd_f16', inpgrad.data_ptr(), meangrad.data_ptr(), sqmeangrad.data_ptr(),
+              output.data_ptr(), outgrad.data_ptr(), bsize, h_outgrad, w_outgrad, d_outgrad, num_channels,
+              int(blocks), _lib.stream_of(inpgrad))
+    return outgrad

@@ -1,0 +1,81 @@
+"""DWConv: depthwise 3x3x3 convolution on channels_last_3d fp16 tensors.
+
+Host side of kerops_dwconv_fwd_f16; same name, positional arguments, asserts and
+result as kerops/ops/conv/dwconv.py:20-63 of the reference.
+"""
+import torch
+
+from ... import _lib
+from ...settings import ConfigurableArg, confexc, configure
+from .._common import cl3d, next_power_of_2, require_cuda
+
+# gfx950 launch table, keyed by channel count like the reference's `warps` / `dblock`
+# (kerops/ops/conv/dwconv.py:10-17): (wavefronts per workgroup, tile extent along D,
+# tile extent along W).  A missing key means "no kernel for this channel count".
+_WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
+_TILE_D = {8: 32, 16: 16, 32: 16, 64: 16, 128: 16}
+_TILE_W = {8: 8, 16: 8, 32: 4, 64: 4, 128: 4}
+
+
+@confexc(KeyError)
+def warps(channels):
+    return _WAVES[channels]
+
+
+@confexc(KeyError)
+def dblock(channels):
+    return _TILE_D[channels]
+
+
+@confexc(KeyError)
+def wtile(channels):
+    return _TILE_W[channels]
+
+
+@configure(
+    ACCTYPE='float32',
+    num_warps=lambda x: warps(x.shape[1]),
+    D_block=lambda x: dblock(x.shape[1]),
+    W_block=lambda x: wtile(x.shape[1]),
+    H_chunk=0,
+)
+def DWConv(
+    x,
+    weight,
+    *,
+    ACCTYPE: ConfigurableArg,
+    num_warps: ConfigurableArg,
+    D_block: ConfigurableArg,
+    W_block: ConfigurableArg,
+    H_chunk: ConfigurableArg,
+):
+    """y = conv3d(x, weight, padding=1, stride=1, groups=C) with weight laid out [3,3,3,C].
+
+    ACCTYPE / num_warps / D_block keep the reference's names: accumulation is always
+    fp32 ('float16' is accepted and computed in fp32), num_warps is the number of
+    64-wide wavefronts per workgroup (the built kernels use 4) and D_block the tile
+    extent along D.  W_block (tile extent along W) and H_chunk (rows one workgroup
+    marches over, 0 = automatic) are additional gfx950 knobs.
+    """
+    channels = x.shape[1]
+
+    assert x.ndim == 5
+    assert x.is_contiguous(memory_format=torch.channels_last_3d)
+    assert x.dtype == weight.dtype == torch.float16
+    assert channels == next_power_of_2(channels)
+    assert list(weight.shape) == [3, 3, 3, channels]
+    assert D_block == next_power_of_2(D_block)
+    {'float32': None, 'float16': None}[ACCTYPE]
+    assert num_warps == 4, 'the gfx950 kernels are built for 4 wavefronts per workgroup'
+    require_cuda(x, weight)
+
+    bsize, _, H, W, D = x.shape
+    weight = weight.contiguous()
+    output = torch.empty_like(x)
+    assert cl3d(output)
+
+    _lib.call(
+        'kerops_dwconv_fwd_f16', x.data_ptr(), weight.data_ptr(), output.data_ptr(), bsize, H, W, D, channels,
+        int(W_block), int(D_block), int(H_chunk), _lib.stream_of(x),
+    )
+    return output

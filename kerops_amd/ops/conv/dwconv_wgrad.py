@@ -1,0 +1,86 @@
+"""DWConvWGRAD: weight gradient of the depthwise 3x3x3 convolution.
+
+Host side of kerops_dwconv_wgrad_f16; same name, positional arguments and asserts as
+kerops/ops/conv/dwconv_wgrad.py:25-79 of the reference.  The reference stores fp16
+partials and returns an fp16 [3,3,3,C] tensor; here the sum is fp32 end to end and is
+cast once to `out_dtype` (fp16 by default so the result type matches the reference).
+"""
+import torch
+
+from ... import _lib
+from ...settings import ConfigurableArg, confexc, configure
+from .._common import next_power_of_2, require_cuda
+
+_WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
+_TILE_D = {8: 32, 16: 32, 32: 16, 64: 16, 128: 16}
+_TILE_W = {8: 16, 16: 8, 32: 8, 64: 4, 128: 4}
+
+
+@confexc(KeyError)
+def warps(channels):
+    return _WAVES[channels]
+
+
+@confexc(KeyError)
+def dblock(channels):
+    return _TILE_D[channels]
+
+
+@confexc(KeyError)
+def wtile(channels):
+    return _TILE_W[channels]
+
+
+@confexc(KeyError)
+def ilp(channels):
+    # the reference's ILP (2*ILP rows of H per program, kerops/ops/conv/dwconv_wgrad.py:20-22)
+    # has no separate meaning here: a workgroup marches over H_chunk rows
+    return {8: 1, 16: 1, 32: 1, 64: 1, 128: 1}[channels]
+
+
+@configure(
+    ACCTYPE='float32',
+    num_warps=lambda x: warps(x.shape[1]),
+    D_block=lambda x: dblock(x.shape[1]),
+    ILP=lambda x: ilp(x.shape[1]),
+    W_block=lambda x: wtile(x.shape[1]),
+    H_chunk=0,
+    out_dtype=torch.float16,
+)
+def DWConvWGRAD(
+    x,
+    grad,
+    *,
+    ACCTYPE: ConfigurableArg,
+    num_warps: ConfigurableArg,
+    D_block: ConfigurableArg,
+    ILP: ConfigurableArg,
+    W_block: ConfigurableArg,
+    H_chunk: ConfigurableArg,
+    out_dtype: ConfigurableArg,
+):
+    """grad_w[kh,kw,kd,c] = sum_{n,h,w,d} grad[n,c,h,w,d] * x[n,c,h+kh-1,w+kw-1,d+kd-1]."""
+    channels = x.shape[1]
+
+    assert x.ndim == grad.ndim == 5
+    assert x.shape == grad.shape
+    assert x.is_contiguous(memory_format=torch.channels_last_3d)
+    assert grad.is_contiguous(memory_format=torch.channels_last_3d)
+    assert x.dtype == grad.dtype == torch.float16
+    assert channels == next_power_of_2(channels)
+    assert D_block == next_power_of_2(D_block)
+    {'float32': None, 'float16': None}[ACCTYPE]
+    assert num_warps == 4, 'the gfx950 kernels are built for 4 wavefronts per workgroup'
+    require_cuda(x, grad)
+
+    bsize, _, H, W, D = x.shape
+    cfg = (int(W_block), int(D_block), int(H_chunk))
+    ws_bytes = _lib.query('kerops_dwconv_wgrad_workspace_bytes', bsize, H, W, D, channels, *cfg)
+    ws = _lib.workspace(ws_bytes, x.device)
+    grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=torch.float32)
+
+    _lib.call(
+        'kerops_dwconv_wgrad_f16', x.data_ptr(), grad.data_ptr(), grad_w.data_ptr(), ws.data_ptr(), ws_bytes,
+        bsize, H, W, D, channels, *cfg, _lib.stream_of(x),
+    )
+    return grad_w if out_dtype == torch.float32 else grad_w.to(out_dtype)
