@@ -21,8 +21,10 @@
  *  - Return value: KEROPS_OK or a negative KEROPS_E_* code; the text of the last
  *    failure on the calling thread is available from kerops_last_error_string().
  *    Nothing throws.
- *  - Trailing `tile_*`, `h_chunk` and `blocks` arguments are launch-shape knobs;
- *    0 selects the built-in choice for gfx950.
+ *  - Trailing `tile_*`, `h_chunk`, `lane_channels` and `blocks` arguments are
+ *    launch-shape knobs (patch extents along W and D, rows of H one workgroup
+ *    marches over, channels one lane owns, workgroup count); 0 selects the built-in
+ *    choice for gfx950, an unbuilt combination returns KEROPS_E_BADARG.
  */
 #ifndef KEROPS_HIP_H
 #define KEROPS_HIP_H
@@ -52,7 +54,8 @@ const char* kerops_last_error_string(void);
  * Replaces the `_DWConv_cl3d_impl[grid](...)` launch and its per-sample Python
  * loop: kerops/ops/conv/dwconv.py:47-61 (kernel kerops/kernels/dw_conv.py:6-142). */
 int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W, int32_t D,
-                          int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk, void* stream);
+                          int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk, int32_t lane_channels,
+                          void* stream);
 
 /* Depthwise weight gradient, fp32 end to end:
  *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]
@@ -62,10 +65,10 @@ int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int
  * launches and the trailing `grad_w.sum(dim=(0, 1))`:
  * kerops/ops/conv/dwconv_wgrad.py:54-77 (kernel kerops/kernels/dw_conv.py:147-287). */
 int64_t kerops_dwconv_wgrad_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w,
-                                            int32_t tile_d, int32_t h_chunk);
+                                            int32_t tile_d, int32_t h_chunk, int32_t lane_channels);
 int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* workspace, int64_t workspace_bytes,
                             int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d,
-                            int32_t h_chunk, void* stream);
+                            int32_t h_chunk, int32_t lane_channels, void* stream);
 
 /* Per-channel mean and mean of squares over M = numel / C voxels, fp32.
  * Replaces the zero-fill of mean/sqmean and the `_Stats_cl3d_impl[(grid,)](...)`

@@ -12,24 +12,33 @@
 // Lane mapping.  One thread = one c8 chunk (8 channels, 16 bytes) of one voxel;
 // consecutive lanes take consecutive chunks in memory order (channel group fastest,
 // then D), so global loads/stores of a wavefront are contiguous 1 KiB runs and LDS
-// reads are consecutive 16-byte words (conflict free).  The 27 weight chunks of the
-// thread's channel group stay packed as fp16 in registers; products are formed by
-// mixed-precision FMA (fp16 x fp16 + fp32 -> fp32).
+// reads are consecutive words (conflict free).  The weights of the thread's channels stay
+// packed as fp16 pairs in registers; products are formed by the 2-way fp16 dot
+// instruction and mixed-precision FMA, both accumulating in fp32.
 #include "common.hpp"
 
 namespace kerops {
 
-template <int CG_, int TW_, int TD_, int NT_>
+template <int CG_, int TW_, int TD_, int CL_, int NT_, int WPE_>
 struct FwdCfg {
-    static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_;
+    static constexpr int CG = CG_, TW = TW_, TD = TD_, CL = CL_, NT = NT_;
+    static constexpr int WPE = WPE_;           // wavefronts per SIMD the register budget is held to
+    static constexpr int SC = CG * 8;          // channels in the slab
+    static constexpr int NCL = SC / CL;        // lane groups (CL channels each) per voxel
     static constexpr int PW = TW + 2, PD = TD + 2;
-    static constexpr int NPOS = TW * TD * CG;  // output chunks per plane
-    static constexpr int P = NPOS / NT;        // output chunks per thread per plane
-    static constexpr int NCH = PW * PD * CG;   // staged chunks per plane
+    static constexpr int NPOS = TW * TD * NCL;  // output pieces per plane
+    static constexpr int P = NPOS / NT;         // output pieces per thread per plane
+    static constexpr int NCH = PW * PD * CG;    // staged c8 chunks per plane
     static constexpr int NLD = (NCH + NT - 1) / NT;
     static_assert(NPOS % NT == 0, "patch must divide evenly over the threads");
-    static_assert(NT % CG == 0, "a thread keeps one channel group");
+    static_assert(NT % NCL == 0, "a thread keeps one lane group");
     static_assert((TD & (TD - 1)) == 0, "TD power of two");
+    static_assert(CL == 2 || CL == 4 || CL == 8, "2, 4 or 8 channels per lane");
+};
+
+template <int CL>
+struct HalfN {
+    typedef _Float16 type __attribute__((ext_vector_type(CL)));
 };
 
 struct FwdArgs {
@@ -41,37 +50,226 @@ struct FwdArgs {
     uint32_t nblocks;
 };
 
-template <class Cfg, bool DO_F, bool DO_M, bool DO_S>
-__device__ __forceinline__ void scatter_plane(const half8_t* __restrict__ plane, const int (&lbase)[Cfg::P],
-                                              const half8_t (&wr)[27], float (&aF)[Cfg::P][8],
-                                              float (&aM)[Cfg::P][8], float (&aS)[Cfg::P][8])
+// Packed weights of one thread: for every weight row kh and every channel j of the lane,
+// the nine in-plane taps t = kw*3 + kd are held as four fp16 pairs (t = 0/1, 2/3, 4/5, 6/7)
+// for the 2-way dot instruction plus the single tap t = 8.
+template <int CL>
+struct LaneWeights {
+    half2_t pair[3][4][CL];
+    half_t single[3][CL];
+};
+
+__device__ __forceinline__ half2_t pack_halves(uint32_t a, uint32_t b, int hi)
 {
+    // (half `hi` of a, half `hi` of b) as one dword: v_perm_b32 {b, a}
+    const uint32_t r = hi ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
+    return __builtin_bit_cast(half2_t, r);
+}
+
+// Scatter one staged input plane into the three accumulator sets.  Per output piece and
+// channel: 4 byte-permutes pair up the 9 in-plane neighbours once, then each of the three
+// weight rows costs 4 two-way dots (fp16 x fp16 -> fp32) and 1 mixed-precision FMA:
+// 19 instructions for 27 multiply-adds, all accumulation in fp32.
+template <class Cfg, bool DO_F, bool DO_M, bool DO_S>
+__device__ __forceinline__ void scatter_plane(const half_t* __restrict__ plane, const int (&lbase)[Cfg::P],
+                                              const LaneWeights<Cfg::CL>& lw, float (&aF)[Cfg::P][Cfg::CL],
+                                              float (&aM)[Cfg::P][Cfg::CL], float (&aS)[Cfg::P][Cfg::CL])
+{
+    constexpr int CL = Cfg::CL, ND = CL / 2;
+    typedef uint32_t dv_t __attribute__((ext_vector_type(ND)));
 #pragma unroll
     for (int k = 0; k < Cfg::P; ++k) {
+        uint32_t v[9][ND];
 #pragma unroll
         for (int kw = 0; kw < 3; ++kw) {
 #pragma unroll
             for (int kd = 0; kd < 3; ++kd) {
-                const half8_t v = plane[lbase[k] + (kw * Cfg::PD + kd) * Cfg::CG];
+                if constexpr (ND == 1) {
+                    v[kw * 3 + kd][0] =
+                        *reinterpret_cast<const uint32_t*>(plane + lbase[k] + (kw * Cfg::PD + kd) * Cfg::SC);
+                } else {
+                    const dv_t q = *reinterpret_cast<const dv_t*>(plane + lbase[k] + (kw * Cfg::PD + kd) * Cfg::SC);
 #pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                    const float xv = (float)v[c];
-                    if (DO_F) aF[k][c] = __builtin_fmaf(xv, (float)wr[(2 * 3 + kw) * 3 + kd][c], aF[k][c]);
-                    if (DO_M) aM[k][c] = __builtin_fmaf(xv, (float)wr[(1 * 3 + kw) * 3 + kd][c], aM[k][c]);
-                    if (DO_S) aS[k][c] = __builtin_fmaf(xv, (float)wr[(0 * 3 + kw) * 3 + kd][c], aS[k][c]);
+                    for (int e = 0; e < ND; ++e) v[kw * 3 + kd][e] = q[e];
                 }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CL; ++c) {
+            half2_t pr[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) pr[p] = pack_halves(v[2 * p][c / 2], v[2 * p + 1][c / 2], c & 1);
+            const half2_t last = __builtin_bit_cast(half2_t, v[8][c / 2]);
+            const float xs = (float)last[c & 1];
+            if (DO_F) {
+                float s = aF[k][c];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) s = __builtin_amdgcn_fdot2(pr[p], lw.pair[2][p][c], s, false);
+                aF[k][c] = __builtin_fmaf(xs, (float)lw.single[2][c], s);
+            }
+            if (DO_M) {
+                float s = aM[k][c];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) s = __builtin_amdgcn_fdot2(pr[p], lw.pair[1][p][c], s, false);
+                aM[k][c] = __builtin_fmaf(xs, (float)lw.single[1][c], s);
+            }
+            if (DO_S) {
+                float s = 0.0f;  // the row hp+1 starts here: no separate zeroing pass
+#pragma unroll
+                for (int p = 0; p < 4; ++p) s = __builtin_amdgcn_fdot2(pr[p], lw.pair[0][p][c], s, false);
+                aS[k][c] = __builtin_fmaf(xs, (float)lw.single[0][c], s);
             }
         }
     }
 }
 
-template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, 2) void dwconv_fwd_kernel(const FwdArgs a)
+// OUT_FULL: every output piece of the patch lies inside the volume (true for all patches
+// but the last ones along W / D), so stores need no per-lane predicate.
+template <class Cfg, bool OUT_FULL>
+__device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)[2][Cfg::NCH + 1], int slab, int dt,
+                                                int wt_i, int hc, int n)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, P = Cfg::P, NLD = Cfg::NLD, NCH = Cfg::NCH;
-    constexpr int PD = Cfg::PD;
-    __shared__ half8_t lds[2][NCH];
+    constexpr int PD = Cfg::PD, CL = Cfg::CL, NCL = Cfg::NCL, SC = Cfg::SC;
+    typedef typename HalfN<CL>::type hv_t;
+    const int t = threadIdx.x;
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
+    const int hs = hc * a.h_chunk;
+    const int he = min(hs + a.h_chunk, H);
+    const int cslab = slab * SC;
+    const int64_t plane_stride = (int64_t)W * D * C;
+    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
+    half_t* yn = a.y + (int64_t)n * H * plane_stride;
 
+    // weights of this thread's lane group (CL channels), kept packed as fp16
+    const int cl = t % NCL;
+    LaneWeights<CL> lw;
+    {
+        hv_t wr[27];
+#pragma unroll
+        for (int tap = 0; tap < 27; ++tap)
+            wr[tap] = *reinterpret_cast<const hv_t*>(a.wt + tap * C + cslab + cl * CL);
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int c = 0; c < CL; ++c) {
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    half2_t w2 = {wr[kh * 9 + 2 * p][c], wr[kh * 9 + 2 * p + 1][c]};
+                    lw.pair[kh][p][c] = w2;
+                }
+                lw.single[kh][c] = wr[kh * 9 + 8][c];
+            }
+    }
+
+    // staging assignment (fixed for the whole march)
+    // Every lane issues every load and every LDS write unconditionally (straight-line code,
+    // no per-lane branches around memory operations): a lane with nothing to stage loads the
+    // first chunk of the plane and writes it to the dump slot.
+    uint32_t goff[NLD];  // byte offset inside one (W, D, C) plane
+    int ldst[NLD];       // destination chunk in the LDS plane buffer
+    bool gval[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+        const int q = t + j * NT;
+        const int wq = q / (PD * CG);
+        const int r = q - wq * (PD * CG);
+        const int dq = r / CG;
+        const int cq = r - dq * CG;
+        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
+        gval[j] = (q < NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+        goff[j] = gval[j] ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        ldst[j] = gval[j] ? q : NCH;
+        // halo chunks outside the volume never change: zero them once in both buffers
+        if (q < NCH && !gval[j]) {
+            const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            lds[0][q] = z;
+            lds[1][q] = z;
+        }
+    }
+
+    // output assignment
+    int lbase[P];
+    uint32_t ooff[P];  // byte offset inside one plane
+    bool oval[P];
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+        const int i = t + k * NT;
+        const int dl = (i / NCL) % TD;
+        const int wl = i / (NCL * TD);
+        lbase[k] = (wl * PD + dl) * SC + cl * CL;  // in halves
+        const int w = w0 + wl, d = d0 + dl;
+        oval[k] = (w < W) && (d < D);
+        ooff[k] = oval[k] ? (uint32_t)(((w * D + d) * C + cslab + cl * CL) * 2) : 0u;
+    }
+
+    float a0[P][CL], a1[P][CL], a2[P][CL];
+#pragma unroll
+    for (int k = 0; k < P; ++k)
+#pragma unroll
+        for (int c = 0; c < CL; ++c) a0[k][c] = a1[k][c] = a2[k][c] = 0.0f;
+
+    half8_t pre[NLD];
+    auto prefetch = [&](int hp) {
+        if ((hp >= 0) && (hp < H)) {
+            const char* xplane = reinterpret_cast<const char*>(xn + hp * plane_stride);  // wavefront-uniform
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
+        }
+    };
+
+    int parity = 0;
+    auto step = [&](int hp, float(&aF)[P][CL], float(&aM)[P][CL], float(&aS)[P][CL]) {
+        const bool inb = (hp >= 0) && (hp < H);
+        half8_t* buf = lds[parity];
+        parity ^= 1;
+        if (inb) {
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) buf[ldst[j]] = pre[j];
+        }
+        __syncthreads();
+        if (hp + 1 <= he) prefetch(hp + 1);
+        if (inb) {
+            scatter_plane<Cfg, true, true, true>(reinterpret_cast<const half_t*>(buf), lbase, lw, aF, aM, aS);
+        } else {
+#pragma unroll
+            for (int k = 0; k < P; ++k)
+#pragma unroll
+                for (int c = 0; c < CL; ++c) aS[k][c] = 0.0f;
+        }
+        const int ho = hp - 1;
+        if (ho >= hs) {
+            char* yplane = reinterpret_cast<char*>(yn + ho * plane_stride);  // wavefront-uniform
+#pragma unroll
+            for (int k = 0; k < P; ++k) {
+                if (OUT_FULL || oval[k]) {
+                    hv_t o;
+#pragma unroll
+                    for (int c = 0; c < CL; ++c) o[c] = (half_t)aF[k][c];
+                    *reinterpret_cast<hv_t*>(yplane + ooff[k]) = o;
+                }
+            }
+        }
+    };
+
+    int hp = hs - 1;
+    prefetch(hp);
+    __syncthreads();  // the one-off zero fill of the halo chunks is visible before any plane is read
+    for (;;) {
+        step(hp, a0, a1, a2);
+        if (++hp > he) break;
+        step(hp, a1, a2, a0);
+        if (++hp > he) break;
+        step(hp, a2, a0, a1);
+        if (++hp > he) break;
+    }
+}
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const FwdArgs a)
+{
+    __shared__ half8_t lds[2][Cfg::NCH + 1];  // +1: write-only dump slot for lanes with nothing to stage
     uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
     if (L >= a.nblocks) return;
     // logical order, fastest first: slab, d-tile, w-tile, h-chunk, n
@@ -83,122 +281,18 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_fwd_kernel(const FwdArgs a)
     L /= a.n_wt;
     const int hc = L % a.n_hc;
     const int n = L / a.n_hc;
-
-    const int t = threadIdx.x;
-    const int H = a.H, W = a.W, D = a.D, C = a.C;
-    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
-    const int hs = hc * a.h_chunk;
-    const int he = min(hs + a.h_chunk, H);
-    const int cslab = slab * CG * 8;
-    const int64_t plane_stride = (int64_t)W * D * C;
-    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
-    half_t* yn = a.y + (int64_t)n * H * plane_stride;
-
-    // weights of this thread's channel group
-    const int cg = t % CG;
-    half8_t wr[27];
-#pragma unroll
-    for (int tap = 0; tap < 27; ++tap) wr[tap] = load_c8(a.wt + tap * C + cslab + cg * 8);
-
-    // staging assignment (fixed for the whole march)
-    int goff[NLD];
-    bool gval[NLD];
-#pragma unroll
-    for (int j = 0; j < NLD; ++j) {
-        const int q = t + j * NT;
-        const int wq = q / (PD * CG);
-        const int r = q - wq * (PD * CG);
-        const int dq = r / CG;
-        const int cq = r - dq * CG;
-        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
-        gval[j] = (q < NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
-        goff[j] = (w * D + d) * C + cslab + cq * 8;
-    }
-
-    // output assignment
-    int lbase[P], ooff[P];
-    bool oval[P];
-#pragma unroll
-    for (int k = 0; k < P; ++k) {
-        const int i = t + k * NT;
-        const int dl = (i / CG) % TD;
-        const int wl = i / (CG * TD);
-        lbase[k] = (wl * PD + dl) * CG + cg;
-        const int w = w0 + wl, d = d0 + dl;
-        oval[k] = (w < W) && (d < D);
-        ooff[k] = (w * D + d) * C + cslab + cg * 8;
-    }
-
-    float a0[P][8], a1[P][8], a2[P][8];
-#pragma unroll
-    for (int k = 0; k < P; ++k)
-#pragma unroll
-        for (int c = 0; c < 8; ++c) a0[k][c] = a1[k][c] = a2[k][c] = 0.0f;
-
-    half8_t pre[NLD];
-    auto prefetch = [&](int hp) {
-        const bool inb = (hp >= 0) && (hp < H);
-#pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (inb && gval[j]) v = load_c8(xn + hp * plane_stride + goff[j]);
-            pre[j] = v;
-        }
-    };
-
-    int parity = 0;
-    auto step = [&](int hp, float(&aF)[P][8], float(&aM)[P][8], float(&aS)[P][8]) {
-        const bool inb = (hp >= 0) && (hp < H);
-        half8_t* buf = lds[parity];
-        parity ^= 1;
-        if (inb) {
-#pragma unroll
-            for (int j = 0; j < NLD; ++j) {
-                const int q = t + j * NT;
-                if (q < NCH) buf[q] = pre[j];
-            }
-        }
-        __syncthreads();
-        if (hp + 1 <= he) prefetch(hp + 1);
-        // Keep the weights packed as fp16: without this the compiler hoists the 216
-        // fp16->fp32 conversions out of the march and holds them in 216 registers.
-#pragma unroll
-        for (int tap = 0; tap < 27; ++tap) asm("" : "+v"(wr[tap]));
-#pragma unroll
-        for (int k = 0; k < P; ++k)
-#pragma unroll
-            for (int c = 0; c < 8; ++c) aS[k][c] = 0.0f;
-        if (inb) scatter_plane<Cfg, true, true, true>(buf, lbase, wr, aF, aM, aS);
-        const int ho = hp - 1;
-        if (ho >= hs) {
-#pragma unroll
-            for (int k = 0; k < P; ++k) {
-                if (oval[k]) {
-                    half8_t o;
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) o[c] = (half_t)aF[k][c];
-                    store_c8(yn + ho * plane_stride + ooff[k], o);
-                }
-            }
-        }
-    };
-
-    int hp = hs - 1;
-    prefetch(hp);
-    for (;;) {
-        step(hp, a0, a1, a2);
-        if (++hp > he) break;
-        step(hp, a1, a2, a0);
-        if (++hp > he) break;
-        step(hp, a2, a0, a1);
-        if (++hp > he) break;
+    const bool out_full = ((wt_i + 1) * Cfg::TW <= a.W) && ((dt + 1) * Cfg::TD <= a.D);
+    if (out_full) {
+        dwconv_fwd_body<Cfg, true>(a, lds, slab, dt, wt_i, hc, n);
+    } else {
+        dwconv_fwd_body<Cfg, false>(a, lds, slab, dt, wt_i, hc, n);
     }
 }
 
-template <int CG, int TW, int TD>
+template <int CG, int TW, int TD, int CL, int WPE>
 static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t stream)
 {
-    using Cfg = FwdCfg<CG, TW, TD, 256>;
+    using Cfg = FwdCfg<CG, TW, TD, CL, 256, WPE>;
     FwdArgs a = base;
     a.n_slab = a.C / (CG * 8);
     a.n_wt = ceil_div(a.W, TW);
@@ -229,7 +323,7 @@ using namespace kerops;
 
 extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W,
                                      int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
-                                     void* stream)
+                                     int32_t lane_channels, void* stream)
 {
     if (!x || !wt || !y || !aligned16(x) || !aligned16(wt) || !aligned16(y)) {
         set_error("dwconv_fwd: null or misaligned pointer");
@@ -257,26 +351,30 @@ extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int
     a.C = C;
     hipStream_t s = (hipStream_t)stream;
     const int cg = C >= 64 ? 8 : C / 8;
-    if (tile_w == 0 && tile_d == 0) {
+    if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
+        // measured best on MI355X at (1, C, 350, 350, 128)
         switch (cg) {
-            case 1: tile_w = 8; tile_d = 32; break;
-            case 2: tile_w = 8; tile_d = 16; break;
-            case 4: tile_w = 4; tile_d = 16; break;
-            default: tile_w = 4; tile_d = 16; break;
+            case 1: tile_w = 16; tile_d = 32; lane_channels = 4; break;
+            case 2: tile_w = 8; tile_d = 32; lane_channels = 2; break;
+            case 4: tile_w = 8; tile_d = 16; lane_channels = 2; break;
+            default: tile_w = 8; tile_d = 8; lane_channels = 2; break;
         }
     }
-#define KEROPS_FWD_CASE(CGv, TWv, TDv) \
-    if (cg == CGv && tile_w == TWv && tile_d == TDv) return launch_fwd<CGv, TWv, TDv>(a, N, h_chunk, s);
-    KEROPS_FWD_CASE(1, 8, 32)
-    KEROPS_FWD_CASE(1, 16, 32)
-    KEROPS_FWD_CASE(2, 8, 16)
-    KEROPS_FWD_CASE(2, 8, 32)
-    KEROPS_FWD_CASE(4, 4, 16)
-    KEROPS_FWD_CASE(4, 8, 16)
-    KEROPS_FWD_CASE(8, 4, 8)
-    KEROPS_FWD_CASE(8, 4, 16)
-    KEROPS_FWD_CASE(8, 8, 8)
+#define KEROPS_FWD_CASE(CGv, TWv, TDv, CLv, WPEv)                                  \
+    if (cg == CGv && tile_w == TWv && tile_d == TDv && lane_channels == CLv) \
+        return launch_fwd<CGv, TWv, TDv, CLv, WPEv>(a, N, h_chunk, s);
+    KEROPS_FWD_CASE(1, 16, 32, 4, 3)
+    KEROPS_FWD_CASE(1, 16, 32, 2, 3)
+    KEROPS_FWD_CASE(2, 8, 32, 4, 3)
+    KEROPS_FWD_CASE(2, 8, 32, 2, 3)
+    KEROPS_FWD_CASE(4, 8, 16, 4, 3)
+    KEROPS_FWD_CASE(4, 8, 16, 2, 3)
+    KEROPS_FWD_CASE(8, 4, 8, 4, 3)
+    KEROPS_FWD_CASE(8, 4, 8, 2, 4)
+    KEROPS_FWD_CASE(8, 4, 16, 2, 3)
+    KEROPS_FWD_CASE(8, 8, 8, 2, 3)
 #undef KEROPS_FWD_CASE
-    set_error("dwconv_fwd: no kernel built for C=%d tile_w=%d tile_d=%d", C, tile_w, tile_d);
+    set_error("dwconv_fwd: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, tile_w, tile_d,
+              lane_channels);
     return KEROPS_E_BADARG;
 }

@@ -259,7 +259,8 @@ struct WgPlan {
     int64_t nblocks;
 };
 
-static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d, int h_chunk, WgPlan* p)
+static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d, int h_chunk, int lane_channels,
+                      WgPlan* p)
 {
     if (N <= 0 || H <= 0 || W <= 0 || D <= 0) {
         set_error("dwconv_wgrad: non-positive extent");
@@ -274,14 +275,17 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
         return KEROPS_E_BADARG;
     }
     p->cg = C >= 64 ? 8 : C / 8;
-    if (tile_w == 0 && tile_d == 0) {
+    if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
+        // measured best on MI355X at (1, C, 350, 350, 128)
         switch (p->cg) {
             case 1: tile_w = 16; tile_d = 32; break;
             case 2: tile_w = 8; tile_d = 32; break;
             case 4: tile_w = 8; tile_d = 16; break;
-            default: tile_w = 4; tile_d = 16; break;
+            default: tile_w = 8; tile_d = 8; break;
         }
+        lane_channels = 2;
     }
+    p->cl = lane_channels;
     p->tile_w = tile_w;
     p->tile_d = tile_d;
     p->n_slab = C / (p->cg * 8);
@@ -328,24 +332,26 @@ static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStrea
 using namespace kerops;
 
 extern "C" int64_t kerops_dwconv_wgrad_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
-                                                       int32_t tile_w, int32_t tile_d, int32_t h_chunk)
+                                                       int32_t tile_w, int32_t tile_d, int32_t h_chunk,
+                                                       int32_t lane_channels)
 {
     WgPlan p;
-    int rc = plan_wgrad(N, H, W, D, C, tile_w, tile_d, h_chunk, &p);
+    int rc = plan_wgrad(N, H, W, D, C, tile_w, tile_d, h_chunk, lane_channels, &p);
     if (rc != KEROPS_OK) return rc;
     return p.nblocks * 27 * (p.cg * 8) * (int64_t)sizeof(float);
 }
 
 extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* workspace,
                                        int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
-                                       int32_t tile_w, int32_t tile_d, int32_t h_chunk, void* stream)
+                                       int32_t tile_w, int32_t tile_d, int32_t h_chunk, int32_t lane_channels,
+                                       void* stream)
 {
     if (!x || !g || !gw || !aligned16(x) || !aligned16(g) || !aligned16(gw)) {
         set_error("dwconv_wgrad: null or misaligned pointer");
         return KEROPS_E_BADARG;
     }
     WgPlan p;
-    int rc = plan_wgrad(N, H, W, D, C, tile_w, tile_d, h_chunk, &p);
+    int rc = plan_wgrad(N, H, W, D, C, tile_w, tile_d, h_chunk, lane_channels, &p);
     if (rc != KEROPS_OK) return rc;
     const int64_t need = p.nblocks * 27 * (p.cg * 8) * (int64_t)sizeof(float);
     if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
@@ -363,17 +369,19 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     a.C = C;
     hipStream_t s = (hipStream_t)stream;
 #define KEROPS_WG_CASE(CGv, TWv, TDv, CLv) \
-    if (p.cg == CGv && p.tile_w == TWv && p.tile_d == TDv) return launch_wgrad<CGv, TWv, TDv, CLv>(a, p, gw, s);
+    if (p.cg == CGv && p.tile_w == TWv && p.tile_d == TDv && p.cl == CLv) \
+        return launch_wgrad<CGv, TWv, TDv, CLv>(a, p, gw, s);
+    KEROPS_WG_CASE(1, 16, 32, 2)
     KEROPS_WG_CASE(1, 16, 32, 4)
-    KEROPS_WG_CASE(1, 8, 32, 4)
+    KEROPS_WG_CASE(2, 8, 32, 2)
     KEROPS_WG_CASE(2, 8, 32, 4)
-    KEROPS_WG_CASE(2, 8, 16, 4)
+    KEROPS_WG_CASE(4, 8, 16, 2)
     KEROPS_WG_CASE(4, 8, 16, 4)
-    KEROPS_WG_CASE(4, 4, 16, 4)
+    KEROPS_WG_CASE(8, 8, 8, 2)
+    KEROPS_WG_CASE(8, 4, 16, 2)
     KEROPS_WG_CASE(8, 4, 16, 4)
-    KEROPS_WG_CASE(8, 4, 8, 4)
-    KEROPS_WG_CASE(8, 8, 16, 4)
 #undef KEROPS_WG_CASE
-    set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d", C, p.tile_w, p.tile_d);
+    set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, p.tile_w, p.tile_d,
+              p.cl);
     return KEROPS_E_BADARG;
 }

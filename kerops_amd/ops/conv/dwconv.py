@@ -13,8 +13,9 @@ from .._common import cl3d, next_power_of_2, require_cuda
 # (kerops/ops/conv/dwconv.py:10-17): (wavefronts per workgroup, tile extent along D,
 # tile extent along W).  A missing key means "no kernel for this channel count".
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
-_TILE_D = {8: 32, 16: 16, 32: 16, 64: 16, 128: 16}
-_TILE_W = {8: 8, 16: 8, 32: 4, 64: 4, 128: 4}
+_TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
+_TILE_W = {8: 16, 16: 8, 32: 8, 64: 8, 128: 8}
+_LANE_C = {8: 4, 16: 2, 32: 2, 64: 2, 128: 2}
 
 
 @confexc(KeyError)
@@ -32,12 +33,18 @@ def wtile(channels):
     return _TILE_W[channels]
 
 
+@confexc(KeyError)
+def lanec(channels):
+    return _LANE_C[channels]
+
+
 @configure(
     ACCTYPE='float32',
     num_warps=lambda x: warps(x.shape[1]),
     D_block=lambda x: dblock(x.shape[1]),
     W_block=lambda x: wtile(x.shape[1]),
     H_chunk=0,
+    lane_channels=lambda x: lanec(x.shape[1]),
 )
 def DWConv(
     x,
@@ -48,6 +55,7 @@ def DWConv(
     D_block: ConfigurableArg,
     W_block: ConfigurableArg,
     H_chunk: ConfigurableArg,
+    lane_channels: ConfigurableArg,
 ):
     """y = conv3d(x, weight, padding=1, stride=1, groups=C) with weight laid out [3,3,3,C].
 
@@ -55,7 +63,8 @@ def DWConv(
     fp32 ('float16' is accepted and computed in fp32), num_warps is the number of
     64-wide wavefronts per workgroup (the built kernels use 4) and D_block the tile
     extent along D.  W_block (tile extent along W) and H_chunk (rows one workgroup
-    marches over, 0 = automatic) are additional gfx950 knobs.
+    marches over, 0 = automatic) and lane_channels (channels one lane owns: 2, 4 or 8)
+    are additional gfx950 knobs.
     """
     channels = x.shape[1]
 
@@ -76,6 +85,6 @@ def DWConv(
 
     _lib.call(
         'kerops_dwconv_fwd_f16', x.data_ptr(), weight.data_ptr(), output.data_ptr(), bsize, H, W, D, channels,
-        int(W_block), int(D_block), int(H_chunk), _lib.stream_of(x),
+        int(W_block), int(D_block), int(H_chunk), int(lane_channels), _lib.stream_of(x),
     )
     return output

@@ -12,8 +12,8 @@ from ...settings import ConfigurableArg, confexc, configure
 from .._common import next_power_of_2, require_cuda
 
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
-_TILE_D = {8: 32, 16: 32, 32: 16, 64: 16, 128: 16}
-_TILE_W = {8: 16, 16: 8, 32: 8, 64: 4, 128: 4}
+_TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
+_TILE_W = {8: 16, 16: 8, 32: 8, 64: 8, 128: 8}
 
 
 @confexc(KeyError)
@@ -45,6 +45,7 @@ def ilp(channels):
     ILP=lambda x: ilp(x.shape[1]),
     W_block=lambda x: wtile(x.shape[1]),
     H_chunk=0,
+    lane_channels=2,
     out_dtype=torch.float16,
 )
 def DWConvWGRAD(
@@ -57,6 +58,7 @@ def DWConvWGRAD(
     ILP: ConfigurableArg,
     W_block: ConfigurableArg,
     H_chunk: ConfigurableArg,
+    lane_channels: ConfigurableArg,
     out_dtype: ConfigurableArg,
 ):
     """grad_w[kh,kw,kd,c] = sum_{n,h,w,d} grad[n,c,h,w,d] * x[n,c,h+kh-1,w+kw-1,d+kd-1]."""
@@ -74,7 +76,7 @@ def DWConvWGRAD(
     require_cuda(x, grad)
 
     bsize, _, H, W, D = x.shape
-    cfg = (int(W_block), int(D_block), int(H_chunk))
+    cfg = (int(W_block), int(D_block), int(H_chunk), int(lane_channels))
     ws_bytes = _lib.query('kerops_dwconv_wgrad_workspace_bytes', bsize, H, W, D, channels, *cfg)
     ws = _lib.workspace(ws_bytes, x.device)
     grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=torch.float32)
