@@ -1,0 +1,132 @@
+"""CPU tests of the C-ABI boundary: the built library loads, exports every symbol the header
+declares, validates arguments before touching a device, and the Python ops keep the
+reference's host-side contract checks (same exception types, raised before the ABI is
+crossed).  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from kerops_amd import _lib
+from kerops_amd.settings import CongiguratorError
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'kerops_hip.h')
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(kerops_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), f'{name} is declared in include/kerops_hip.h but not exported'
+    # and the ctypes table binds exactly the declared set
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.kerops_hip_version() >= 100
+
+
+def test_argument_validation_needs_no_device():
+    lib = _lib.load()
+    rc = lib.kerops_dwconv_fwd_f16(None, None, None, 1, 4, 4, 4, 8, 0, 0, 0, 0, None)
+    assert rc == _lib.KEROPS_E_BADARG and 'pointer' in _lib.last_error()
+    buf = (ctypes.c_char * 4096)()
+    addr = (ctypes.addressof(buf) + 15) & ~15
+    rc = lib.kerops_dwconv_fwd_f16(addr, addr, addr, 1, 4, 4, 4, 24, 0, 0, 0, 0, None)
+    assert rc == _lib.KEROPS_E_UNSUPPORTED_C
+    rc = lib.kerops_dwconv_fwd_f16(addr, addr, addr, 1, 4, 4, 4, 64, 5, 7, 0, 2, None)
+    assert rc == _lib.KEROPS_E_BADARG and 'no kernel built' in _lib.last_error()
+    rc = lib.kerops_dwconv_fwd_f16(addr + 2, addr, addr, 1, 4, 4, 4, 64, 0, 0, 0, 0, None)
+    assert rc == _lib.KEROPS_E_BADARG
+    rc = lib.kerops_dwconv_wgrad_f16(addr, addr, addr, addr, 16, 1, 4, 4, 4, 64, 0, 0, 0, 0, None)
+    assert rc == _lib.KEROPS_E_WORKSPACE
+    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 1024, addr, 1 << 30, 0, None)
+    assert rc == _lib.KEROPS_E_UNSUPPORTED_C
+    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 12, addr, 1 << 30, 0, None)
+    assert rc == _lib.KEROPS_E_BADARG
+    rc = lib.kerops_quant_u8_window(addr, 7, addr, 16, 1.0, 0, None)
+    assert rc == _lib.KEROPS_E_BADARG and 'dtype' in _lib.last_error()
+
+
+def test_workspace_queries():
+    lib = _lib.load()
+    assert lib.kerops_stats_workspace_bytes(1000, 64, 16) == 16 * 2 * 64 * 4
+    assert lib.kerops_stats_workspace_bytes(1000, 24, 16) == _lib.KEROPS_E_BADARG
+    n = lib.kerops_dwconv_wgrad_workspace_bytes(1, 350, 350, 128, 64, 0, 0, 0, 0)
+    assert n > 0 and n % (27 * 64 * 4) == 0
+    assert lib.kerops_dwconv_wgrad_workspace_bytes(1, 8, 8, 8, 24, 0, 0, 0, 0) == _lib.KEROPS_E_UNSUPPORTED_C
+    assert lib.kerops_avgpool_ceil_stats_workspace_bytes(1, 7, 7, 7, 8, 4) == 4 * 2 * 8 * 4
+    assert lib.kerops_absmax_workspace_bytes(10) == 40
+
+
+def cl3d(*shape, dtype=torch.float16):
+    return torch.zeros(*shape, dtype=dtype).to(memory_format=torch.channels_last_3d)
+
+
+def test_ops_keep_reference_contract_checks():
+    from kerops_amd.ops.avgpool import AvgPoolCeilStats
+    from kerops_amd.ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
+    from kerops_amd.ops.conv import DWConv, DWConvWGRAD
+    from kerops_amd.ops.stats import Stats
+
+    x = cl3d(1, 8, 4, 4, 4)
+    w = torch.zeros(3, 3, 3, 8, dtype=torch.float16)
+    with pytest.raises(AssertionError):  # not channels_last_3d
+        DWConv(torch.zeros(1, 8, 4, 4, 4, dtype=torch.float16), w)
+    with pytest.raises(AssertionError):  # dtype
+        DWConv(x.float(), w.float())
+    with pytest.raises(AssertionError):  # weight layout
+        DWConv(x, torch.zeros(8, 1, 3, 3, 3, dtype=torch.float16))
+    with pytest.raises(CongiguratorError):  # channel count with no launch table entry
+        DWConv(cl3d(1, 4, 4, 4, 4), torch.zeros(3, 3, 3, 4, dtype=torch.float16))
+    with pytest.raises(CongiguratorError):
+        DWConvWGRAD(cl3d(1, 256, 2, 2, 2), cl3d(1, 256, 2, 2, 2))
+    with pytest.raises(KeyError):
+        DWConv(x, w, ACCTYPE='bfloat16')
+    with pytest.raises(AssertionError):
+        DWConvWGRAD(x, cl3d(1, 8, 4, 4, 5))
+    with pytest.raises(AssertionError):  # non power of two
+        Stats(cl3d(1, 6, 4, 4, 4))
+    with pytest.raises(AssertionError):
+        ApplyBNReLU(x, torch.zeros(4), torch.zeros(8))
+    with pytest.raises(AssertionError):  # fp32 weight / bias required by the backward
+        ApplyBNReLUBackward(x, torch.zeros(8, dtype=torch.float64), torch.zeros(8, dtype=torch.float64), x)
+    with pytest.raises(AssertionError):  # D*C above the reference's row limit
+        AvgPoolCeilStats(cl3d(1, 128, 2, 2, 512))
+
+
+def test_no_cpu_fallback():
+    from kerops_amd.ops.conv import DWConv
+    from kerops_amd.ops.quantization import QuantUint8Window
+    from kerops_amd.ops.stats import Stats
+
+    x = cl3d(1, 8, 4, 4, 4)
+    with pytest.raises(RuntimeError, match='no CPU path'):
+        DWConv(x, torch.zeros(3, 3, 3, 8, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match='no CPU path'):
+        Stats(x)
+    with pytest.raises(RuntimeError, match='no CPU path'):
+        QuantUint8Window(x, 1.0)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, '_lib', None)
+    monkeypatch.setattr(_lib, 'LIB_PATH', os.path.join(ROOT, 'kerops_amd', '_C', 'does_not_exist.so'))
+    with pytest.raises(RuntimeError, match='no fallback'):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, 'kerops_amd')
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(('.py', '.hip', '.hpp', '.h', '.cpp')):
+                text = open(os.path.join(dirpath, f)).read()
+                assert 'import oracle' not in text and 'from oracle' not in text and 'oracle/' not in text, f

@@ -1,0 +1,200 @@
+"""GPU parity tests of DWConv / DWConvWGRAD: the HIP kernels, called through the C ABI by the
+drop-in ops, against the CPU oracle, the golden vectors, closed forms and, at the full README
+shape, size-independent properties.  Tolerances are the reference's own test criteria
+(tests/ops/test_conv.py:28-36,75-83) plus tighter ones that fp32 accumulation makes possible."""
+import itertools
+import math
+
+import pytest
+import torch
+
+import oracle
+from conftest import cpu_gen, from_bits, rand_cl3d, rand_dw_weight
+from kerops_amd.ops.conv import DWConv, DWConvWGRAD
+from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+# odd / prime extents exercise every edge mask (the reference sweeps {2,3,7,13,16,32,37,53,111,128})
+SHAPES = [
+    (1, 8, 5, 4, 3), (2, 8, 7, 13, 37), (1, 8, 64, 64, 32), (3, 8, 2, 2, 2), (1, 8, 3, 111, 16),
+    (1, 16, 13, 16, 32), (2, 16, 37, 3, 53), (1, 16, 2, 128, 7),
+    (1, 32, 16, 7, 53), (2, 32, 3, 37, 13), (1, 32, 53, 2, 33),
+    (1, 64, 9, 11, 35), (2, 64, 3, 2, 2), (1, 64, 33, 10, 40), (1, 64, 7, 53, 17),
+    (1, 128, 6, 9, 18), (2, 128, 13, 3, 37),
+]
+
+
+def check_fwd(x, wk, y):
+    ref16, ref32 = oracle.dwconv_fwd(x, wk, wide=True, return_fp32=True)
+    y = y.cpu()
+    assert y.shape == x.shape and y.dtype == torch.float16
+    assert y.stride() == x.stride()
+    # the reference's criterion (oracle plays the role of torch's conv3d there)
+    assert allclose_two_stage(ref16, y, rtol_strict=1e-4, atol_strict=1e-3, rtol_narrow=1e-3, atol_narrow=2e-3)
+    # fp32 accumulation: never more than one fp16 rounding away from the exact sum
+    err = (y.float() - ref32).abs()
+    assert (err <= 2.0 ** -11 * ref32.abs().clamp(min=2.0 ** -14) * 1.01 + 1e-6).all()
+    same = (y.contiguous().view(torch.int16) == ref16.contiguous().view(torch.int16)).float().mean().item()
+    assert same >= 0.998, same
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+def test_dwconv_matches_oracle(shape):
+    g = cpu_gen()
+    x = rand_cl3d(g, *shape)
+    _, wk = rand_dw_weight(g, shape[1])
+    check_fwd(x, wk, DWConv(x.to(DEV), wk.to(DEV)))
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+def test_dwconv_wgrad_matches_oracle(shape):
+    g = cpu_gen()
+    x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    ref = oracle.dwconv_wgrad(x, grad)
+    gw32 = DWConvWGRAD(x.to(DEV), grad.to(DEV), out_dtype=torch.float32).cpu()
+    assert list(gw32.shape) == [3, 3, 3, shape[1]] and gw32.dtype == torch.float32
+    rel = ((gw32.double() - ref).norm() / ref.norm()).item()
+    assert rel < 2e-6, rel
+    # drop-in result type (fp16) and the reference's own criterion
+    gw16 = DWConvWGRAD(x.to(DEV), grad.to(DEV)).cpu()
+    assert gw16.dtype == torch.float16
+    if ref.abs().max() < 6e4:
+        assert weight_grad_similarity(ref.float(), gw16.float(), rtol_cos=1e-4, atol_cos=1e-4,
+                                      rtol_len=1e-3 * shape[0], atol_len=1e-3)
+
+
+FWD_VARIANTS = {8: [(16, 32, 4), (16, 32, 2)], 16: [(8, 32, 4), (8, 32, 2)], 32: [(8, 16, 4), (8, 16, 2)],
+                64: [(4, 8, 4), (4, 8, 2), (4, 16, 2), (8, 8, 2)], 128: [(4, 8, 4), (4, 8, 2), (4, 16, 2), (8, 8, 2)]}
+WG_VARIANTS = {8: [(16, 32, 2), (16, 32, 4)], 16: [(8, 32, 2), (8, 32, 4)], 32: [(8, 16, 2), (8, 16, 4)],
+               64: [(8, 8, 2), (4, 16, 2), (4, 16, 4)], 128: [(8, 8, 2), (4, 16, 2), (4, 16, 4)]}
+
+
+@pytest.mark.parametrize('c', [8, 16, 32, 64, 128])
+def test_every_built_launch_shape(c):
+    """Every (W_block, D_block, lane_channels) the library is built with, with several H_chunk
+    values (chunk borders inside the volume, chunk of one row, chunk larger than H)."""
+    g = cpu_gen(7)
+    shape = (2, c, 11, 19, 37)
+    x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    _, wk = rand_dw_weight(g, c)
+    ref_gw = oracle.dwconv_wgrad(x, grad)
+    xd, gd, wd = x.to(DEV), grad.to(DEV), wk.to(DEV)
+    for (tw, td, cl), hc in itertools.product(FWD_VARIANTS[c], (0, 1, 4, 100)):
+        check_fwd(x, wk, DWConv(xd, wd, W_block=tw, D_block=td, lane_channels=cl, H_chunk=hc))
+    for (tw, td, cl), hc in itertools.product(WG_VARIANTS[c], (0, 1, 4, 100)):
+        gw = DWConvWGRAD(xd, gd, W_block=tw, D_block=td, lane_channels=cl, H_chunk=hc, out_dtype=torch.float32)
+        rel = ((gw.cpu().double() - ref_gw).norm() / ref_gw.norm()).item()
+        assert rel < 2e-6, (tw, td, cl, hc, rel)
+
+
+def test_golden_vectors(golden):
+    x = from_bits(golden['x']).to(memory_format=torch.channels_last_3d)
+    grad = from_bits(golden['grad']).to(memory_format=torch.channels_last_3d)
+    wk = from_bits(golden['weight_c13x3x3'])[:, 0].permute(1, 2, 3, 0).contiguous()
+    y = DWConv(x.to(DEV), wk.to(DEV)).cpu()
+    y32 = torch.from_numpy(golden['dwconv_y_f32'])
+    assert (y.float() - y32).abs().max() <= 2.0 ** -11 * max(1.0, y32.abs().max().item()) * 1.01
+    assert torch.allclose(y.float(), y32, rtol=1e-2, atol=1e-2)  # the tolerance of BASELINE config 2
+    gw = DWConvWGRAD(x.to(DEV), grad.to(DEV), out_dtype=torch.float32).cpu().double()
+    ref = torch.from_numpy(golden['dwconv_wgrad_f64'])
+    assert ((gw - ref).norm() / ref.norm()).item() < 1e-6
+
+
+def test_single_taps_copy_every_fp16_value():
+    """Weight = one 1.0 at a tap: the output is the input shifted, bit for bit, for every finite
+    fp16 pattern including subnormals (no flush to zero, no rounding in the fp32 path)."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    fin = bits[torch.isfinite(bits)]
+    H, W, D, c = 31, 16, 16, 8
+    flat = torch.zeros(H * W * D * c, dtype=torch.float16)
+    flat[:fin.numel()] = fin
+    x = flat.view(1, H, W, D, c).permute(0, 4, 1, 2, 3)
+    xd = x.to(DEV)
+    for kh, kw, kd in [(1, 1, 1), (0, 0, 0), (2, 2, 2), (0, 1, 2), (2, 1, 0), (1, 2, 1)]:
+        wk = torch.zeros(3, 3, 3, c, dtype=torch.float16)
+        wk[kh, kw, kd] = 1.0
+        y = DWConv(xd, wk.to(DEV)).cpu()
+        exp = torch.zeros_like(x)
+        sh, sw, sd = kh - 1, kw - 1, kd - 1
+        src = x[:, :, max(sh, 0):H + min(sh, 0), max(sw, 0):W + min(sw, 0), max(sd, 0):D + min(sd, 0)]
+        exp[:, :, max(-sh, 0):H + min(-sh, 0), max(-sw, 0):W + min(-sw, 0), max(-sd, 0):D + min(-sd, 0)] = src
+        same = (y.view(torch.int16) == exp.view(torch.int16)) | ((y == 0) & (exp == 0))
+        assert same.all(), (kh, kw, kd)
+
+
+def test_ones_count_neighbours_and_wgrad_closed_form():
+    c, H, W, D = 64, 5, 9, 21
+    ones = torch.ones(1, c, H, W, D, dtype=torch.float16).to(memory_format=torch.channels_last_3d).to(DEV)
+    y = DWConv(ones, torch.ones(3, 3, 3, c, dtype=torch.float16, device=DEV)).cpu()
+
+    def cnt(n):
+        v = torch.full((n,), 3.0)
+        v[0] = v[-1] = 2.0
+        return v
+
+    exp = cnt(H).view(H, 1, 1) * cnt(W).view(1, W, 1) * cnt(D).view(1, 1, D)
+    assert torch.equal(y[0, 0].float(), exp) and torch.equal(y[0, c - 1].float(), exp)
+    gw = DWConvWGRAD(ones, ones, out_dtype=torch.float32).cpu()
+    for kh, kw, kd in itertools.product(range(3), repeat=3):
+        assert gw[kh, kw, kd, 0].item() == (H - abs(kh - 1)) * (W - abs(kw - 1)) * (D - abs(kd - 1))
+
+
+def test_wgrad_is_deterministic():
+    g = cpu_gen(21)
+    x, grad = rand_cl3d(g, 2, 64, 23, 17, 40).to(DEV), rand_cl3d(g, 2, 64, 23, 17, 40).to(DEV)
+    a = DWConvWGRAD(x, grad, out_dtype=torch.float32)
+    b = DWConvWGRAD(x, grad, out_dtype=torch.float32)
+    assert torch.equal(a, b)
+
+
+def test_config3_wgrad_crop_fp64():
+    """BASELINE config 3: rel L2 error <= 1e-3 against an fp64 CPU reduction on (1,64,96,96,64)."""
+    g = cpu_gen()
+    shape = (1, 64, 96, 96, 64)
+    x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    ref = oracle.dwconv_wgrad(x, grad)
+    gw = DWConvWGRAD(x.to(DEV), grad.to(DEV), out_dtype=torch.float32).cpu().double()
+    rel = ((gw - ref).norm() / ref.norm()).item()
+    assert rel <= 1e-3 and rel < 1e-5, rel
+    gw16 = DWConvWGRAD(x.to(DEV), grad.to(DEV)).cpu().double()
+    assert ((gw16 - ref).norm() / ref.norm()).item() <= 1e-3
+
+
+@pytest.mark.parametrize('c', [8, 64, 128])
+def test_readme_shape_properties(c):
+    """Full (1, C, 350, 350, 128): (a) slabs of the output, including every border, equal the
+    oracle run on the matching input slab; (b) the adjoint identity
+    <DWConv(x, w), g> = <w, DWConvWGRAD(x, g)> ties forward and weight gradient together at a
+    size the CPU oracle cannot sweep."""
+    gen = torch.Generator(DEV).manual_seed(322)
+    H, W, D = 350, 350, 128
+    x = torch.randn(1, H, W, D, c, device=DEV, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+    grad = torch.randn(1, H, W, D, c, device=DEV, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+    _, wk = rand_dw_weight(cpu_gen(), c)
+    wd = wk.to(DEV)
+    y = DWConv(x, wd)
+    gw = DWConvWGRAD(x, grad, out_dtype=torch.float32)
+
+    lhs = torch.zeros((), dtype=torch.float64, device=DEV)
+    for h0 in range(0, H, 50):  # chunked fp64 reduction keeps temporaries small
+        lhs += (y[:, :, h0:h0 + 50].double() * grad[:, :, h0:h0 + 50].double()).sum()
+    rhs = (wd.double() * gw.double()).sum()
+    assert abs(lhs.item() - rhs.item()) <= 1e-3 * max(abs(rhs.item()), 1e3), (lhs.item(), rhs.item())
+
+    # slabs: (h range, w range, d range) of the output; the input slab carries a halo of one
+    for (h0, h1), (w0, w1), (d0, d1) in [((0, 6), (0, 9), (0, 20)), ((344, 350), (341, 350), (108, 128)),
+                                         ((170, 176), (0, 9), (50, 90)), ((57, 63), (170, 182), (0, 128))]:
+        ha, hb = max(h0 - 1, 0), min(h1 + 1, H)
+        wa, wb = max(w0 - 1, 0), min(w1 + 1, W)
+        da, db = max(d0 - 1, 0), min(d1 + 1, D)
+        xs = x[:, :, ha:hb, wa:wb, da:db].cpu().contiguous(memory_format=torch.channels_last_3d)
+        ref16, ref32 = oracle.dwconv_fwd(xs, wk, wide=True, return_fp32=True)
+        sl = (slice(None), slice(None), slice(h0 - ha, h0 - ha + h1 - h0), slice(w0 - wa, w0 - wa + w1 - w0),
+              slice(d0 - da, d0 - da + d1 - d0))
+        got = y[:, :, h0:h1, w0:w1, d0:d1].cpu()
+        # a slab border that is not a volume border sees zero padding in the oracle run: the
+        # halo removes exactly those rows from the comparison
+        assert torch.allclose(got.float(), ref32[sl], rtol=1e-2, atol=1e-2)  # BASELINE config 2 tolerance
+        assert (got.float() - ref32[sl]).abs().max() <= 2.0 ** -11 * max(1.0, ref32.abs().max().item()) * 1.01

@@ -1,0 +1,235 @@
+"""GPU parity tests of the per-voxel stream ops (Stats, AddStats, ApplyBNReLU, AvgPoolCeilStats,
+their backward ops and the quantisers), called through the C ABI by the drop-in ops.
+
+fp16 outputs are compared bit for bit with the CPU oracle (every step is a defined IEEE fp32
+operation); fp32 per-channel sums are compared with the oracle's fp64 sums at the reference's
+tolerances (tests/ops/test_stats.py:19-20, test_bn_relu.py:65-67, test_avgpool.py:20-21) and
+tighter; the quantisers are bit-exact, exhaustively over fp16."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from conftest import cpu_gen, from_bits, rand_cl3d
+from kerops_amd.ops.addition import AddStats, AddStatsBackward
+from kerops_amd.ops.avgpool import AvgPoolCeilStats, AvgPoolCeilStatsBackward
+from kerops_amd.ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
+from kerops_amd.ops.quantization import AbsMax, DequantUint8Window, QuantInt8Sym, QuantUint8Window
+from kerops_amd.ops.stats import Stats, StatsBackward
+from kerops_amd.utils import allclose_two_stage
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+SHAPES = [(1, 2, 3, 3, 3), (2, 4, 7, 5, 3), (3, 2, 2, 2, 2), (1, 8, 5, 4, 3), (2, 16, 7, 13, 37),
+          (1, 32, 16, 16, 16), (1, 64, 9, 11, 35), (2, 128, 3, 53, 7), (4, 8, 2, 111, 2), (1, 256, 5, 3, 2)]
+
+
+def bits_equal(a, b):
+    return torch.equal(a.cpu().contiguous().view(torch.int16), b.contiguous().view(torch.int16))
+
+
+def close64(a, b, tol=2e-6):
+    return torch.allclose(a.cpu().double(), b, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+def test_stats_and_backward(shape):
+    g = cpu_gen()
+    x = rand_cl3d(g, *shape)
+    mean, sq = Stats(x.to(DEV))
+    rm, rs = oracle.stats(x)
+    assert mean.dtype == sq.dtype == torch.float32 and mean.shape == (shape[1],)
+    assert torch.allclose(mean.cpu(), rm.float(), atol=1e-4, rtol=1e-4)   # reference criterion
+    assert close64(mean, rm) and close64(sq, rs)
+    c = shape[1]
+    mg, sg = torch.randn(c, generator=g) / 3, torch.randn(c, generator=g) / 3
+    dx = StatsBackward(x.to(DEV), mg.to(DEV), sg.to(DEV))
+    assert dx.stride() == x.stride()
+    assert bits_equal(dx, oracle.stats_bwd(x, mg, sg))
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+def test_add_stats_and_backward(shape):
+    g = cpu_gen(1)
+    x, y = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    z, mean, sq = AddStats(x.to(DEV), y.to(DEV))
+    rz, rm, rs = oracle.add_stats(x, y)
+    assert bits_equal(z, rz) and torch.equal(z.cpu(), x + y)
+    assert close64(mean, rm) and close64(sq, rs)
+    xin = x.to(DEV).clone()
+    z2, _, _ = AddStats(xin, y.to(DEV), True)
+    assert z2.data_ptr() == xin.data_ptr() and bits_equal(z2, rz)
+    c = shape[1]
+    ug = rand_cl3d(g, *shape)
+    mg, sg = torch.randn(c, generator=g) / 3, torch.randn(c, generator=g) / 3
+    out = AddStatsBackward(ug.to(DEV), mg.to(DEV), sg.to(DEV), z)
+    assert bits_equal(out, oracle.add_stats_bwd(ug, mg, sg, rz))
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+def test_bnrelu_and_backward(shape):
+    g = cpu_gen(2)
+    c = shape[1]
+    x = rand_cl3d(g, *shape)
+    W = torch.randn(c, generator=g) + 0.5
+    B = torch.randn(c, generator=g) * 2
+    y = ApplyBNReLU(x.to(DEV), W.to(DEV), B.to(DEV))
+    assert y.stride() == x.stride()
+    assert bits_equal(y, oracle.bnrelu_fwd(x, W, B))
+    grad = rand_cl3d(g, *shape, std=0.1)
+    Wd, Bd = W.view(1, c, 1, 1, 1).to(DEV), B.view(1, c, 1, 1, 1).to(DEV)
+    dx, dW, dB = ApplyBNReLUBackward(x.to(DEV), Wd, Bd, grad.to(DEV))
+    rdx, rdW, rdB = oracle.bnrelu_bwd(x, W, B, grad)
+    assert dW.shape == Wd.shape and dB.shape == Bd.shape
+    assert bits_equal(dx, rdx)
+    assert torch.allclose(dW.cpu().flatten(), rdW.float(), rtol=1e-4, atol=1e-3)  # reference criterion
+    assert close64(dW.flatten(), rdW, 1e-5) and close64(dB.flatten(), rdB, 1e-5)
+
+
+def test_bn_block_end_to_end_vs_train_mode_batchnorm(golden):
+    """Stats -> fold -> ApplyBNReLU as tests/ops/test_bn_relu.py:26-30 of the reference composes
+    them, against the golden relu(BatchNorm3d(train)(x)) computed by torch on the CPU."""
+    x = from_bits(golden['x']).to(memory_format=torch.channels_last_3d).to(DEV)
+    gamma, beta = torch.from_numpy(golden['gamma']).to(DEV), torch.from_numpy(golden['beta']).to(DEV)
+    mean, sq = Stats(x)
+    rvareps = torch.rsqrt(sq - mean ** 2 + 1e-5)
+    y = ApplyBNReLU(x, gamma * rvareps, beta - mean * rvareps * gamma)
+    ref = torch.from_numpy(golden['bnrelu_y_f32']).half()
+    assert allclose_two_stage(ref, y.cpu().contiguous(), rtol_strict=1e-5, atol_strict=1e-4, percentile_strict=0.995,
+                              rtol_narrow=1e-3, atol_narrow=1e-3)
+    assert torch.allclose(mean.cpu().double(), torch.from_numpy(golden['stats_mean_f64']), atol=1e-6)
+
+
+@pytest.mark.parametrize('shape', SHAPES + [(1, 8, 1, 1, 1), (2, 16, 2, 3, 2), (1, 64, 13, 7, 128)])
+def test_avgpool_and_backward(shape):
+    g = cpu_gen(3)
+    c = shape[1]
+    x = rand_cl3d(g, *shape)
+    yp, mean, sq = AvgPoolCeilStats(x.to(DEV))
+    ryp, rm, rs = oracle.avgpool_ceil_stats(x)
+    assert list(yp.shape) == [shape[0], c] + [math.ceil(s / 2) for s in shape[2:]]
+    assert yp.permute(0, 2, 3, 4, 1).is_contiguous()
+    assert bits_equal(yp, ryp)
+    assert torch.allclose(mean.cpu(), rm.float(), atol=1e-3, rtol=1e-5)  # reference criterion
+    assert close64(mean, rm) and close64(sq, rs)
+    ig = rand_cl3d(g, *ryp.shape)
+    mg, sg = torch.randn(c, generator=g), torch.randn(c, generator=g)
+    ypc = yp.contiguous(memory_format=torch.channels_last_3d)
+    dx = AvgPoolCeilStatsBackward(ig.to(DEV), mg.to(DEV), sg.to(DEV), ypc, x.shape)
+    assert list(dx.shape) == list(x.shape)
+    assert bits_equal(dx, oracle.avgpool_ceil_stats_bwd(ig, mg, sg, ryp, x.shape))
+
+
+def test_avgpool_golden(golden):
+    x = from_bits(golden['x']).to(memory_format=torch.channels_last_3d).to(DEV)
+    yp, mean, sq = AvgPoolCeilStats(x)
+    assert torch.equal(yp.cpu().contiguous(), torch.from_numpy(golden['avgpool_y_f32']).half())
+    assert torch.allclose(mean.cpu().double(), torch.from_numpy(golden['avgpool_mean_f64']), atol=1e-6)
+    assert torch.allclose(sq.cpu().double(), torch.from_numpy(golden['avgpool_sqmean_f64']), atol=1e-6)
+
+
+@pytest.mark.parametrize('blocks', [1, 3, 64])
+def test_explicit_block_counts_and_determinism(blocks):
+    g = cpu_gen(4)
+    x = rand_cl3d(g, 2, 32, 9, 13, 21)
+    a = Stats(x.to(DEV), blocks=blocks)
+    b = Stats(x.to(DEV), blocks=blocks)
+    rm, rs = oracle.stats(x)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert close64(a[0], rm) and close64(a[1], rs)
+    yp, m, s = AvgPoolCeilStats(x.to(DEV), blocks=blocks)
+    ryp, rm, rs = oracle.avgpool_ceil_stats(x)
+    assert bits_equal(yp, ryp) and close64(m, rm) and close64(s, rs)
+
+
+@pytest.mark.parametrize('window', [1.0, 3.0, 0.37, 6.5])
+def test_quant_u8_window_bit_exact_exhaustive(window):
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    x = bits[~torch.isnan(bits)]
+    q = QuantUint8Window(x.to(DEV), window)
+    rq = oracle.quant_u8_window(x, window)
+    assert q.dtype == torch.uint8 and torch.equal(q.cpu(), rq)
+    assert torch.equal(QuantUint8Window(x.float().to(DEV), window).cpu(), rq)
+    for dt in (torch.float16, torch.float32):
+        dq = DequantUint8Window(q, dt, window)
+        ref = oracle.dequant_u8_window(rq, dt, window)
+        assert dq.dtype == dt
+        assert torch.equal(dq.cpu().view(torch.int16 if dt == torch.float16 else torch.int32),
+                           ref.view(torch.int16 if dt == torch.float16 else torch.int32))
+
+
+def test_quant_u8_ragged_lengths_and_layouts():
+    g = cpu_gen(5)
+    for n in (1, 7, 8, 9, 1023, 100003):
+        x = torch.randn(n, generator=g) * 2
+        assert torch.equal(QuantUint8Window(x.to(DEV), 2.5).cpu(), oracle.quant_u8_window(x, 2.5))
+        xh = x.half()
+        q = QuantUint8Window(xh.to(DEV), 2.5)
+        assert torch.equal(q.cpu(), oracle.quant_u8_window(xh, 2.5))
+        assert torch.equal(DequantUint8Window(q, torch.float16, 2.5).cpu(),
+                           oracle.dequant_u8_window(q.cpu(), torch.float16, 2.5))
+    x = rand_cl3d(g, 2, 8, 5, 3, 7)
+    q = QuantUint8Window(x.to(DEV), 1.0)
+    assert q.stride() == x.stride()
+    assert torch.equal(q.cpu(), oracle.quant_u8_window(x.permute(0, 2, 3, 4, 1), 1.0).permute(0, 4, 1, 2, 3))
+
+
+def test_quant_i8_sym_bit_exact():
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    fin = bits[torch.isfinite(bits)]
+    am = AbsMax(fin.to(DEV))
+    assert am.item() == oracle.absmax_f16(fin) == 65504.0
+    g = cpu_gen(6)
+    for n, scale in ((200001, 3.0), (8, 1.0), (5, 100.0), (65536, 0.01)):
+        y = (torch.randn(n, generator=g) * scale).half()
+        q, s = QuantInt8Sym(y.to(DEV))
+        a = oracle.absmax_f16(y)
+        assert q.dtype == torch.int8 and torch.equal(q.cpu(), oracle.quant_i8_sym(y, a))
+        assert s.item() == torch.tensor(a, dtype=torch.float32).div(127.0).item()
+    # exhaustive over fp16 for a few explicit maxima, ties included
+    for amax in (127.0, 1.0, 3.3):
+        am = torch.tensor([amax], dtype=torch.float32, device=DEV)
+        q, _ = QuantInt8Sym(fin.to(DEV), am)
+        assert torch.equal(q.cpu(), oracle.quant_i8_sym(fin, amax))
+    z, _ = QuantInt8Sym(torch.zeros(100, dtype=torch.float16, device=DEV))
+    assert (z == 0).all()
+
+
+def test_config4_pipeline_full_shape():
+    """BASELINE config 4 at (1,64,350,350,128): Stats -> fold -> ApplyBNReLU -> AvgPoolCeilStats.
+    Checked through properties that do not need a full-size CPU run: the statistics against an
+    fp64 reduction on the GPU, BN-ReLU against the formula evaluated by torch on a slab, the
+    pooled tensor against torch's AvgPool3d on a slab, and the pooled statistics against the
+    pooled tensor itself."""
+    gen = torch.Generator(DEV).manual_seed(322)
+    c, H, W, D = 64, 350, 350, 128
+    x = (torch.randn(1, H, W, D, c, device=DEV, generator=gen) * math.sqrt(2.0) + 0.5).half().permute(0, 4, 1, 2, 3)
+    gamma = torch.rand(c, device=DEV, generator=gen) + 0.5
+    beta = torch.randn(c, device=DEV, generator=gen) * math.sqrt(0.1)
+    mean, sq = Stats(x)
+    m64 = torch.zeros(c, dtype=torch.float64, device=DEV)
+    s64 = torch.zeros(c, dtype=torch.float64, device=DEV)
+    for h0 in range(0, H, 50):
+        xs = x[:, :, h0:h0 + 50].double()
+        m64 += xs.sum(dim=(0, 2, 3, 4))
+        s64 += (xs * xs).sum(dim=(0, 2, 3, 4))
+    M = H * W * D
+    assert torch.allclose(mean.double(), m64 / M, rtol=1e-6, atol=1e-6)
+    assert torch.allclose(sq.double(), s64 / M, rtol=1e-6, atol=1e-6)
+    rvareps = torch.rsqrt(sq - mean ** 2 + 1e-5)
+    Wf, Bf = gamma * rvareps, beta - mean * rvareps * gamma
+    y = ApplyBNReLU(x, Wf, Bf)
+    sl = (slice(None), slice(None), slice(340, 350), slice(0, 350), slice(0, 128))
+    ref = torch.relu(x[sl].float() * Wf.view(1, c, 1, 1, 1) + Bf.view(1, c, 1, 1, 1))
+    assert torch.allclose(y[sl].float(), ref, rtol=1e-2, atol=1e-3)  # fp16 rtol of config 4
+    assert bits_equal(y[:, :, 100:102], oracle.bnrelu_fwd(x[:, :, 100:102].cpu().contiguous(
+        memory_format=torch.channels_last_3d), Wf.cpu(), Bf.cpu()))
+    yp, pm, ps = AvgPoolCeilStats(y)
+    assert list(yp.shape) == [1, c, 175, 175, 64]
+    refp = torch.nn.AvgPool3d(2, ceil_mode=True)(y[:, :, 0:20].float())
+    assert torch.equal(yp[:, :, 0:10].float(), refp.half().float())
+    pm64 = yp.double().mean(dim=(0, 2, 3, 4))
+    assert torch.allclose(pm.double(), pm64, rtol=1e-4, atol=1e-4)  # pooled stats use unrounded values
+    assert torch.allclose(ps.double(), (yp.double() ** 2).mean(dim=(0, 2, 3, 4)), rtol=1e-3, atol=1e-4)

@@ -1,0 +1,107 @@
+"""CPU tests of the configuration mechanism (same rules as kerops/settings of the reference)."""
+import pytest
+
+from kerops_amd.settings import ConfigurableArg, CongiguratorError, confexc, configure, get_l1_cache
+from kerops_amd.settings import hardware_conf
+from kerops_amd.settings.wrapper import ConfiguredFunction
+
+
+@confexc(KeyError)
+def table(channels):
+    return {8: 1, 16: 2}[channels]
+
+
+class FakeTensor:
+    def __init__(self, c):
+        self.shape = (1, c, 4, 4, 4)
+
+
+@configure(a=lambda x: table(x.shape[1]), b=7)
+def op(x, y=3, *, a: ConfigurableArg, b: ConfigurableArg):
+    return x.shape[1], y, a, b
+
+
+def test_configurators_fill_missing_kwargs():
+    assert isinstance(op, ConfiguredFunction)
+    assert op(FakeTensor(8)) == (8, 3, 1, 7)
+    assert op(FakeTensor(16), 5) == (16, 5, 2, 7)
+    assert op.__name__ == 'op'
+
+
+def test_explicit_kwargs_win():
+    assert op(FakeTensor(8), a=99) == (8, 3, 99, 7)
+    assert op(FakeTensor(8), b=0, a=None) == (8, 3, None, 0)
+    # an explicit value means the configurator is not even consulted
+    assert op(FakeTensor(5), a=1) == (5, 3, 1, 7)
+
+
+def test_unsupported_key_raises_configurator_error():
+    with pytest.raises(CongiguratorError):
+        op(FakeTensor(5))
+    assert op.can_be_configured(x=FakeTensor(8)) is True
+    assert op.can_be_configured(x=FakeTensor(5)) is False
+
+
+def test_configurator_receives_arguments_by_name():
+    @configure(k=lambda second, first: (first, second))
+    def f(first, second, *, k: ConfigurableArg):
+        return k
+
+    assert f(1, 2) == (1, 2)
+    assert f(second=2, first=1) == (1, 2)
+
+
+def test_signature_rules():
+    with pytest.raises(RuntimeError, match='ConfigurableArg must be keyword-only'):
+        @configure(a=1)
+        def bad1(x, a: ConfigurableArg):
+            return a
+
+    with pytest.raises(RuntimeError, match='non-ConfigurableArg must not be keyword-only'):
+        @configure(a=1)
+        def bad2(x, *, a: ConfigurableArg, stray=2):
+            return a
+
+    with pytest.raises(RuntimeError, match='Configuration mismatch'):
+        @configure(a=1, zzz=2)
+        def bad3(x, *, a: ConfigurableArg):
+            return a
+
+    with pytest.raises(RuntimeError, match='Configuration mismatch'):
+        @configure()
+        def bad4(x, *, a: ConfigurableArg):
+            return a
+
+
+def test_reconfigure_and_repr():
+    @configure(a=1, b=lambda x: x + 1)
+    def f(x, *, a: ConfigurableArg, b: ConfigurableArg):
+        return a, b
+
+    assert f(1) == (1, 2)
+    f.reconfigure(a=10, b=20)
+    assert f(1) == (10, 20)
+    with pytest.raises(RuntimeError, match='Configuration mismatch'):
+        f.reconfigure(a=1)
+    f.reconfigure(a=1, b=lambda x: x * 2)
+    text = repr(f)
+    assert text.splitlines()[0].startswith('f(x, *, a')
+    assert 'a: 1' in text and 'b: Configurator(x)' in text
+
+
+def test_l1_cache_knob():
+    assert get_l1_cache() == 65536
+    hardware_conf.set_l1_cache(1024)
+    try:
+        assert get_l1_cache() == 1024
+    finally:
+        hardware_conf.set_l1_cache(65536)
+
+
+def test_confexc_passes_other_exceptions():
+    @confexc(KeyError)
+    def c(v):
+        raise ValueError('x')
+
+    with pytest.raises(ValueError):
+        c(1)
