@@ -1,0 +1,273 @@
+#!/usr/bin/env python3
+"""Benchmark of the channels-last 3D depthwise-conv hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--channels 64] [--no-cpu-baseline]
+
+One "step" is one pass of the hot path over one synthetic batch that is already resident in
+HBM: DWConv forward followed by DWConvWGRAD at the README shape (1, C, 350, 350, 128), fp16,
+channels_last_3d (BASELINE.json configs 2 and 3).  The script prints ONE JSON line:
+
+  metric / value / unit   DWConv fwd + wgrad milliseconds per step (lower is better)
+  fwd / wgrad             per-op ms, algorithmic GB/s (4*V*C bytes), % of the 8 TB/s HBM peak and
+                          % of the bandwidth torch.clone reaches on the same tensor in this run
+  roofline                the dominant kernel of the step, timed live with HIP events on the
+                          stream the kernels run on
+  ops                     the same figures for the other ops of the path (Stats, ApplyBNReLU,
+                          AvgPoolCeilStats, QuantUint8Window) and for every C of the README table
+  cpu_baseline            the CPU oracle (oracle/kerops_oracle.c, OpenMP) on a bounded crop of the
+                          same workload, scaled by the voxel ratio; torch's CPU conv3d(groups=C),
+                          the reference tests' ground truth, is timed beside it
+
+Inputs are synthetic: x, grad ~ N(0, 1) (mean, variance), depthwise weight ~ N(0, 1/27), drawn
+with a fixed seed.  Every GPU on this pool is a single-GPU box, so --gpus above 1 is refused.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+H, W, D = 350, 350, 128
+V = H * W * D
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) at
+# (1,64,350,350,128), each counter scaled by what it reads for a 2 007 040 000-byte device copy
+# (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000): see profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    ('dwconv_fwd', 64): None,
+    ('dwconv_wgrad', 64): None,
+}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--channels', type=int, default=64, help='C of the timed step (README table: 8..128)')
+    ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the CPU legs (used under rocprofv3)')
+    ap.add_argument('--no-extra-ops', action='store_true', help='time only the DWConv step')
+    return ap.parse_args()
+
+
+def median(xs):
+    s = sorted(xs)
+    return s[len(s) // 2]
+
+
+def time_op(torch, fn, iters, warm):
+    """Median / min of per-launch HIP-event times on torch's current stream."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = [a.elapsed_time(b) for a, b in evs]
+    return median(ts), min(ts), sum(ts) / len(ts)
+
+
+def figures(ms, nbytes, clone_gbps):
+    gbps = nbytes / ms / 1e6
+    return {'ms': round(ms, 4), 'GBps': round(gbps, 1), 'frac_hbm_peak': round(gbps / HBM_PEAK_GBPS, 4),
+            'frac_of_clone': round(gbps / clone_gbps, 4) if clone_gbps else None, 'algorithmic_bytes': nbytes}
+
+
+def cpu_baseline(torch, C):
+    """Oracle (a scalar-per-voxel C port with OpenMP) and torch CPU conv3d on a crop."""
+    import oracle
+    from torch.nn import functional as F
+
+    crop = (1, C, 176, 176, 128)
+    vox = crop[2] * crop[3] * crop[4]
+    g = torch.Generator('cpu').manual_seed(322)
+    x = torch.randn(*crop, generator=g).half().to(memory_format=torch.channels_last_3d)
+    gr = torch.randn(*crop, generator=g).half().to(memory_format=torch.channels_last_3d)
+    wt = (torch.randn(C, 1, 3, 3, 3, generator=g) / math.sqrt(27)).half()
+    wk = wt[:, 0].permute(1, 2, 3, 0).contiguous()
+    oracle.dwconv_fwd(x[:, :, :8], wk, wide=False)  # load the library, warm the thread pool
+
+    reps_f, reps_w = 3, 1
+    t0 = time.perf_counter()
+    for _ in range(reps_f):
+        oracle.dwconv_fwd(x, wk, wide=False)
+    t_f = (time.perf_counter() - t0) / reps_f
+    t0 = time.perf_counter()
+    for _ in range(reps_w):
+        oracle.dwconv_wgrad(x, gr)
+    t_w = (time.perf_counter() - t0) / reps_w
+    scale = V / vox
+    port = {
+        'value': round((t_f + t_w) * 1e3 * scale, 1), 'unit': 'ms', 'cores': oracle.num_threads(), 'kind': 'port',
+        'sample': f'oracle DWConv fwd (fp32, {reps_f} runs) + wgrad (fp64, {reps_w} run) on the leading crop '
+                  f'(1,{C},176,176,128), time scaled by the voxel ratio {scale:.2f} to (1,{C},350,350,128)',
+        'fwd_ms_scaled': round(t_f * 1e3 * scale, 1), 'wgrad_ms_scaled': round(t_w * 1e3 * scale, 1),
+        'host_cpus': os.cpu_count(),
+    }
+    # the reference tests' ground truth on the same crop: conv3d(groups=C) in fp32 and its autograd
+    xf = x.float()
+    w32 = wt.float().requires_grad_(True)
+    ts_f, ts_w = [], []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        y = F.conv3d(xf, w32, None, 1, 1, 1, C)
+        ts_f.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        (gw,) = torch.autograd.grad(y, w32, gr.float())
+        ts_w.append(time.perf_counter() - t0)
+    torch_cpu = {
+        'fwd_ms_scaled': round(median(ts_f) * 1e3 * scale, 1), 'wgrad_ms_scaled': round(median(ts_w) * 1e3 * scale, 1),
+        'threads': torch.get_num_threads(), 'host_cpus': os.cpu_count(),
+        'sample': 'torch.nn.functional.conv3d(groups=C) fp32 and autograd wgrad on the same crop, median of 3, scaled',
+    }
+    return port, torch_cpu
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f'bench.py: every GPU box of this pool has one GPU and the hot path is a single-GPU kernel path; '
+              f'--gpus {args.gpus} is not supported (run with --gpus 1)', file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print('bench.py: no ROCm device visible; the benchmark measures HIP kernels only', file=sys.stderr)
+        sys.exit(3)
+    from kerops_amd.ops.avgpool import AvgPoolCeilStats
+    from kerops_amd.ops.bnrelu import ApplyBNReLU
+    from kerops_amd.ops.conv import DWConv, DWConvWGRAD
+    from kerops_amd.ops.quantization import QuantUint8Window
+    from kerops_amd.ops.stats import Stats
+
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+    C = args.channels
+    gen = torch.Generator(dev).manual_seed(322)
+
+    def make(c):
+        x = torch.randn(1, H, W, D, c, device=dev, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+        g = torch.randn(1, H, W, D, c, device=dev, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+        wk = (torch.randn(c, 1, 3, 3, 3, device=dev, generator=gen) / math.sqrt(27)).half()
+        return x, g, wk[:, 0].permute(1, 2, 3, 0).contiguous()
+
+    x, g, wk = make(C)
+    nbytes = 4 * V * C
+
+    # ---- copy floor on the same tensor
+    clone_ms, clone_min, _ = time_op(torch, lambda: x.clone(), 30, 5)
+    clone_gbps = nbytes / clone_ms / 1e6
+
+    # ---- the timed region: W warm-up steps, then exactly K steps
+    for _ in range(args.warmup):
+        DWConv(x, wk)
+        DWConvWGRAD(x, g)
+    torch.cuda.synchronize()
+    K = args.steps
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(K):
+        ev[k][0].record()
+        y = DWConv(x, wk)
+        ev[k][1].record()
+        gw = DWConvWGRAD(x, g)
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    fwd_ts = [e[0].elapsed_time(e[1]) for e in ev]
+    wg_ts = [e[1].elapsed_time(e[2]) for e in ev]
+    ms_per_step = wall_ms / K
+    fwd_avg, wg_avg = sum(fwd_ts) / K, sum(wg_ts) / K
+    del y, gw
+
+    fwd = figures(median(fwd_ts), nbytes, clone_gbps)
+    fwd['ms_avg'], fwd['ms_min'] = round(fwd_avg, 4), round(min(fwd_ts), 4)
+    wg = figures(median(wg_ts), nbytes, clone_gbps)
+    wg['ms_avg'], wg['ms_min'] = round(wg_avg, 4), round(min(wg_ts), 4)
+
+    dom_name, dom_avg = ('dwconv_wgrad', wg_avg) if wg_avg >= fwd_avg else ('dwconv_fwd', fwd_avg)
+    achieved = nbytes / dom_avg / 1e6
+    roofline = {
+        'kernel': 'kerops::dwconv_wgrad_kernel' if dom_name == 'dwconv_wgrad' else 'kerops::dwconv_fwd_kernel',
+        'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+        'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': MEASURED_TRAFFIC_BYTES.get((dom_name, C)),
+        'algorithmic_bytes': nbytes, 'avg_launch_ms': round(dom_avg, 4),
+        'note': 'avg over the timed steps of HIP events around the op on the launch stream; for wgrad the '
+                'launch includes its partial-sum reduce kernel (~1% of the time)',
+    }
+    other = 'dwconv_fwd' if dom_name == 'dwconv_wgrad' else 'dwconv_wgrad'
+    other_avg = fwd_avg if other == 'dwconv_fwd' else wg_avg
+    roofline_other = {
+        'kernel': 'kerops::' + other + '_kernel', 'bound': 'hbm', 'achieved': round(nbytes / other_avg / 1e6, 1),
+        'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(nbytes / other_avg / 1e6 / HBM_PEAK_GBPS, 4),
+        'traffic': MEASURED_TRAFFIC_BYTES.get((other, C)), 'algorithmic_bytes': nbytes,
+        'avg_launch_ms': round(other_avg, 4),
+    }
+
+    ops = {}
+    if not args.no_extra_ops:
+        Wv = torch.rand(C, device=dev, generator=gen) + 0.5
+        Bv = torch.randn(C, device=dev, generator=gen) * 0.3
+        it, wm = 20, 3
+        ops['Stats'] = figures(time_op(torch, lambda: Stats(x), it, wm)[0], 2 * V * C, clone_gbps)
+        ops['ApplyBNReLU'] = figures(time_op(torch, lambda: ApplyBNReLU(x, Wv, Bv), it, wm)[0], 4 * V * C, clone_gbps)
+        ops['AvgPoolCeilStats'] = figures(time_op(torch, lambda: AvgPoolCeilStats(x), it, wm)[0],
+                                          2 * V * C + 2 * (V // 8) * C, clone_gbps)
+        ops['QuantUint8Window'] = figures(time_op(torch, lambda: QuantUint8Window(x, 3.0), it, wm)[0], 3 * V * C,
+                                          clone_gbps)
+        table = {}
+        for c in (8, 16, 32, 64, 128):
+            if c == C:
+                table[str(c)] = {'clone_ms': round(clone_ms, 4), 'dwconv_ms': fwd['ms'], 'wgrad_ms': wg['ms'],
+                                 'dwconv_frac_of_clone': fwd['frac_of_clone'],
+                                 'wgrad_frac_of_clone': wg['frac_of_clone']}
+                continue
+            del x, g
+            torch.cuda.empty_cache()
+            x, g, wkc = make(c)
+            cm = time_op(torch, lambda: x.clone(), it, wm)[0]
+            fm = time_op(torch, lambda: DWConv(x, wkc), it, wm)[0]
+            wgm = time_op(torch, lambda: DWConvWGRAD(x, g), it, wm)[0]
+            table[str(c)] = {'clone_ms': round(cm, 4), 'dwconv_ms': round(fm, 4), 'wgrad_ms': round(wgm, 4),
+                             'dwconv_frac_of_clone': round(cm / fm, 4), 'wgrad_frac_of_clone': round(cm / wgm, 4),
+                             'dwconv_frac_hbm_peak': round(4 * V * c / fm / 1e6 / HBM_PEAK_GBPS, 4),
+                             'wgrad_frac_hbm_peak': round(4 * V * c / wgm / 1e6 / HBM_PEAK_GBPS, 4)}
+        ops['readme_table'] = table
+        ops['readme_table_note'] = 'C=8 (251 MB) fits the 256 MB Infinity Cache: its rows are not pure HBM numbers'
+
+    cpu, cpu_torch = (None, None)
+    if not args.no_cpu_baseline:
+        cpu, cpu_torch = cpu_baseline(torch, C)
+
+    out = {
+        'metric': 'DWConv fwd/wgrad ms + % HBM roofline, fp16 (1,64,350,350,128) NDHWC',
+        'value': round(ms_per_step, 4), 'unit': 'ms', 'n_gpus': 1, 'steps': K, 'warmup': args.warmup,
+        'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f16 in/out, f32 accumulate', 'data': 'synthetic',
+        'config': {'workload': f'DWConv fwd + DWConvWGRAD, x/grad fp16 channels_last_3d (1,{C},350,350,128), '
+                               'weight [3,3,3,C], pad 1, stride 1 (BASELINE configs[1] and configs[2])',
+                   'channels': C, 'voxels': V, 'inputs_resident_in_hbm': True},
+        'fwd': fwd, 'wgrad': wg,
+        'clone': {'ms': round(clone_ms, 4), 'ms_min': round(clone_min, 4), 'GBps': round(clone_gbps, 1),
+                  'frac_hbm_peak': round(clone_gbps / HBM_PEAK_GBPS, 4)},
+        'targets': {'fwd_frac_of_clone>=0.75': fwd['frac_of_clone'] >= 0.75,
+                    'wgrad_frac_of_clone>=0.50': wg['frac_of_clone'] >= 0.50},
+        'roofline': roofline, 'roofline_other': roofline_other,
+        'cpu_baseline': cpu, 'cpu_torch_conv3d': cpu_torch, 'ops': ops,
+        'device': torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()
