@@ -38,10 +38,11 @@ V = H * W * D
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) at
 # (1,64,350,350,128), each counter scaled by what it reads for a 2 007 040 000-byte device copy
-# (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000): see profiles/.
+# (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000):
+# profiles/dwconv_fwd_wgrad_c64_readme_shape.md.
 MEASURED_TRAFFIC_BYTES = {
-    ('dwconv_fwd', 64): None,
-    ('dwconv_wgrad', 64): None,
+    ('dwconv_fwd', 64): 4386780849,    # 2.380 GB read + 2.007 GB written (1.093 x algorithmic)
+    ('dwconv_wgrad', 64): 4331627724,  # 4.317 GB read + 0.015 GB written (1.079 x algorithmic)
 }
 
 
