@@ -4,12 +4,15 @@
 //
 // Same march as the forward kernel: a workgroup owns a (TW x TD) patch of the (W, D)
 // plane for a slab of CG*8 channels and walks a chunk of rows along H.  Each x plane
-// hp (with its halo) is staged through LDS once; a thread owns CL channels of a few
-// patch positions, reads the 9 in-plane neighbours of x from LDS and multiplies them
-// with the three rows of g that see this plane (g[hp+1] for kh=0, g[hp] for kh=1,
-// g[hp-1] for kh=2).  g needs no halo: it is read straight from global memory, one
-// row ahead, and kept in registers for three steps.  The 27*CL fp32 accumulators of a
-// thread live for the whole march; at the end lanes that own the same channels are
+// hp (with its halo) is staged through LDS once; a thread owns 2 channels of a few pairs
+// of D-adjacent patch positions (d, d+1), reads the in-plane neighbours of x from LDS and
+// multiplies them with the three rows of g that see this plane (g[hp+1] for kh=0, g[hp]
+// for kh=1, g[hp-1] for kh=2).  Both factors of a pair are packed per channel into one
+// dword with a byte permute, so one 2-way fp16 dot instruction adds the contributions of
+// both positions to a tap's fp32 accumulator: 54 dots + 20 permutes per pair and plane
+// instead of 108 multiply-adds.  g needs no halo: it is read straight from global memory,
+// one row ahead, and kept (packed) in registers for three steps.  The 27*2 fp32
+// accumulators of a thread live for the whole march; at the end lanes that own the same channels are
 // combined with wavefront shuffles, wavefronts through LDS, and the workgroup writes
 // one partial [27][slab] to the workspace.  A second kernel adds the partials in a
 // fixed order, so the result is deterministic (no atomics).
@@ -17,25 +20,24 @@
 
 namespace kerops {
 
-template <int CG_, int TW_, int TD_, int CL_, int NT_>
+template <int CG_, int TW_, int TD_, int NT_>
 struct WgCfg {
-    static constexpr int CG = CG_, TW = TW_, TD = TD_, CL = CL_, NT = NT_;
+    static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_;
+    static constexpr int CL = 2;               // channels per lane: one dword of fp16
     static constexpr int SC = CG * 8;          // channels in the slab
     static constexpr int NCL = SC / CL;        // lane groups per voxel
     static constexpr int PW = TW + 2, PD = TD + 2;
-    static constexpr int NPOS = TW * TD * NCL;
-    static constexpr int P = NPOS / NT;
+    static constexpr int NPAIR = TW * (TD / 2) * NCL;  // (d, d+1) position pairs per plane
+    static constexpr int PP = NPAIR / NT;              // pairs per thread per plane
     static constexpr int NCH = PW * PD * CG;   // staged c8 chunks per plane
     static constexpr int NLD = (NCH + NT - 1) / NT;
     static constexpr int NWAVE = NT / kWave;
-    static constexpr int STAGE_BYTES = 2 * NCH * 16;
+    static constexpr int STAGE_BYTES = 2 * (NCH + 1) * 16;  // +1: dump slot, see the forward kernel
     static constexpr int RED_BYTES = NWAVE * 27 * SC * 4;
     static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
-    static_assert(NPOS % NT == 0, "patch must divide evenly over the threads");
-    static_assert(NT % NCL == 0 && (kWave % NCL == 0 || NCL % kWave == 0), "lane groups tile a wavefront");
-    static_assert(NCL <= kWave, "a wavefront holds every lane group of a voxel");
-    static_assert((TD & (TD - 1)) == 0, "TD power of two");
-    static_assert(CL == 2 || CL == 4, "2 or 4 channels per lane");
+    static_assert(NPAIR % NT == 0, "patch must divide evenly over the threads");
+    static_assert(NT % NCL == 0 && kWave % NCL == 0, "lane groups tile a wavefront");
+    static_assert((TD & (TD - 1)) == 0 && TD >= 2, "TD power of two");
 };
 
 struct WgArgs {
@@ -47,23 +49,20 @@ struct WgArgs {
     uint32_t nblocks;
 };
 
-template <int CL>
-struct HalfVec;
-template <>
-struct HalfVec<2> {
-    typedef half2_t type;
-};
-template <>
-struct HalfVec<4> {
-    typedef half4_t type;
-};
+__device__ __forceinline__ half2_t pack_lo(uint32_t a, uint32_t b)
+{
+    return __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b, a, 0x05040100u));  // (a.lo, b.lo)
+}
+__device__ __forceinline__ half2_t pack_hi(uint32_t a, uint32_t b)
+{
+    return __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(b, a, 0x07060302u));  // (a.hi, b.hi)
+}
 
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, 2) void dwconv_wgrad_kernel(const WgArgs a)
+__global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a)
 {
-    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, P = Cfg::P, NLD = Cfg::NLD, NCH = Cfg::NCH;
+    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, PP = Cfg::PP, NLD = Cfg::NLD, NCH = Cfg::NCH;
     constexpr int PD = Cfg::PD, CL = Cfg::CL, NCL = Cfg::NCL, SC = Cfg::SC;
-    typedef typename HalfVec<CL>::type hv_t;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
     half8_t* stage = reinterpret_cast<half8_t*>(smem);
 
@@ -89,9 +88,10 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_wgrad_kernel(const WgArgs a
     const half_t* xn = a.x + (int64_t)n * H * plane_stride;
     const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
 
-    // staging assignment (c8 chunks of the halo patch)
-    int goff[NLD];
-    bool gval[NLD];
+    // staging assignment (c8 chunks of the halo patch); every lane loads and writes
+    // unconditionally, lanes with nothing to stage use the plane's first chunk and a dump slot
+    uint32_t goff[NLD];
+    int ldst[NLD];
 #pragma unroll
     for (int j = 0; j < NLD; ++j) {
         const int q = t + j * NT;
@@ -100,23 +100,32 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_wgrad_kernel(const WgArgs a
         const int dq = r / CG;
         const int cq = r - dq * CG;
         const int w = w0 - 1 + wq, d = d0 - 1 + dq;
-        gval[j] = (q < NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
-        goff[j] = (w * D + d) * C + cslab + cq * 8;
+        const bool ok = (q < NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+        goff[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        ldst[j] = ok ? q : NCH;
+        if (q < NCH && !ok) {
+            const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            stage[q] = z;
+            stage[(NCH + 1) + q] = z;
+        }
     }
 
-    // positions of this thread
+    // this thread's (d, d+1) position pairs
     const int cl = t % NCL;
-    int lbase[P], poff[P];
-    bool pval[P];
+    int lbase[PP];        // LDS offset (halves) of x[w-1][d-1] for the pair
+    uint32_t poff[PP];    // byte offset of g[w][d] inside a plane
+    bool pv0[PP], pv1[PP];
 #pragma unroll
-    for (int k = 0; k < P; ++k) {
+    for (int k = 0; k < PP; ++k) {
         const int i = t + k * NT;
-        const int dl = (i / NCL) % TD;
-        const int wl = i / (NCL * TD);
-        lbase[k] = ((wl * PD + dl) * CG) * 8 + cl * CL;  // in halves
+        const int dp = (i / NCL) % (TD / 2);
+        const int wl = i / (NCL * (TD / 2));
+        const int dl = 2 * dp;
+        lbase[k] = ((wl * PD + dl) * CG) * 8 + cl * CL;
         const int w = w0 + wl, d = d0 + dl;
-        pval[k] = (w < W) && (d < D);
-        poff[k] = (w * D + d) * C + cslab + cl * CL;
+        pv0[k] = (w < W) && (d < D);
+        pv1[k] = (w < W) && (d + 1 < D);
+        poff[k] = pv0[k] ? (uint32_t)(((w * D + d) * C + cslab + cl * CL) * 2) : 0u;
     }
 
     float acc[27][CL];
@@ -127,79 +136,91 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_wgrad_kernel(const WgArgs a
 
     half8_t pre[NLD];
     auto prefetch_x = [&](int hp) {
-        const bool inb = (hp >= 0) && (hp < H);
+        if ((hp >= 0) && (hp < H)) {
+            const char* xplane = reinterpret_cast<const char*>(xn + hp * plane_stride);
 #pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (inb && gval[j]) v = load_c8(xn + hp * plane_stride + goff[j]);
-            pre[j] = v;
+            for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
         }
     };
-    auto load_g = [&](int h, hv_t(&dst)[P]) {
+    // g of one row for every pair: raw dwords (c0,c1) at d and d+1; rows outside the chunk and
+    // positions outside the volume contribute zeros
+    uint32_t graw[PP][2];
+    auto load_g = [&](int h) {
         const bool inb = (h >= hs) && (h < he);
+        const char* gplane = reinterpret_cast<const char*>(gn_ptr + (inb ? h : hs) * plane_stride);
+        const uint32_t dstep = (uint32_t)C * 2u;
 #pragma unroll
-        for (int k = 0; k < P; ++k) {
-            hv_t v;
-#pragma unroll
-            for (int c = 0; c < CL; ++c) v[c] = (half_t)0;
-            if (inb && pval[k]) v = *reinterpret_cast<const hv_t*>(gn_ptr + h * plane_stride + poff[k]);
-            dst[k] = v;
+        for (int k = 0; k < PP; ++k) {
+            const uint32_t v0 = *reinterpret_cast<const uint32_t*>(gplane + poff[k]);
+            const uint32_t v1 = *reinterpret_cast<const uint32_t*>(gplane + poff[k] + (pv1[k] ? dstep : 0u));
+            graw[k][0] = (inb && pv0[k]) ? v0 : 0u;
+            graw[k][1] = (inb && pv1[k]) ? v1 : 0u;
         }
     };
-
-    hv_t gm[P], gc[P], gnx[P], gpre[P];
+    // packed (g[d][c], g[d+1][c]) per pair and channel for the rows hp-1, hp, hp+1
+    half2_t gm[PP][CL], gc[PP][CL], gnx[PP][CL];
+    auto pack_g = [&](half2_t(&dst)[PP][CL]) {
 #pragma unroll
-    for (int k = 0; k < P; ++k)
+        for (int k = 0; k < PP; ++k) {
+            dst[k][0] = pack_lo(graw[k][0], graw[k][1]);
+            dst[k][1] = pack_hi(graw[k][0], graw[k][1]);
+        }
+    };
+    const half2_t hz = {(half_t)0, (half_t)0};
 #pragma unroll
-        for (int c = 0; c < CL; ++c) gm[k][c] = gc[k][c] = (half_t)0;
-    load_g(hs, gnx);
+    for (int k = 0; k < PP; ++k)
+#pragma unroll
+        for (int c = 0; c < CL; ++c) gm[k][c] = gc[k][c] = hz;
+    load_g(hs);
+    pack_g(gnx);
 
     int parity = 0;
     prefetch_x(hs - 1);
+    __syncthreads();  // one-off zero fill of out-of-volume halo chunks
     for (int hp = hs - 1; hp <= he; ++hp) {
         const bool inb = (hp >= 0) && (hp < H);
-        half8_t* buf = stage + parity * NCH;
+        half8_t* buf = stage + parity * (NCH + 1);
         parity ^= 1;
         if (inb) {
 #pragma unroll
-            for (int j = 0; j < NLD; ++j) {
-                const int q = t + j * NT;
-                if (q < NCH) buf[q] = pre[j];
-            }
+            for (int j = 0; j < NLD; ++j) buf[ldst[j]] = pre[j];
         }
         __syncthreads();
         if (hp + 1 <= he) prefetch_x(hp + 1);
-        load_g(hp + 2, gpre);
+        load_g(hp + 2);
         if (inb) {
             const half_t* plane = reinterpret_cast<const half_t*>(buf);
 #pragma unroll
-            for (int k = 0; k < P; ++k) {
+            for (int k = 0; k < PP; ++k) {
 #pragma unroll
                 for (int kw = 0; kw < 3; ++kw) {
+                    uint32_t xv[4];  // x[w+kw-1][d-1 .. d+2], two channels each
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        xv[e] = *reinterpret_cast<const uint32_t*>(plane + lbase[k] + ((kw * PD + e) * CG) * 8);
 #pragma unroll
                     for (int kd = 0; kd < 3; ++kd) {
-                        const hv_t xv =
-                            *reinterpret_cast<const hv_t*>(plane + lbase[k] + ((kw * PD + kd) * CG) * 8);
-#pragma unroll
-                        for (int c = 0; c < CL; ++c) {
-                            const float xf = (float)xv[c];
-                            acc[(0 * 3 + kw) * 3 + kd][c] =
-                                __builtin_fmaf((float)gnx[k][c], xf, acc[(0 * 3 + kw) * 3 + kd][c]);
-                            acc[(1 * 3 + kw) * 3 + kd][c] =
-                                __builtin_fmaf((float)gc[k][c], xf, acc[(1 * 3 + kw) * 3 + kd][c]);
-                            acc[(2 * 3 + kw) * 3 + kd][c] =
-                                __builtin_fmaf((float)gm[k][c], xf, acc[(2 * 3 + kw) * 3 + kd][c]);
-                        }
+                        const half2_t x0 = pack_lo(xv[kd], xv[kd + 1]);  // channel 0 at (d+kd-1, d+kd)
+                        const half2_t x1 = pack_hi(xv[kd], xv[kd + 1]);  // channel 1
+                        const int t0 = (0 * 3 + kw) * 3 + kd, t1 = (1 * 3 + kw) * 3 + kd, t2 = (2 * 3 + kw) * 3 + kd;
+                        acc[t0][0] = __builtin_amdgcn_fdot2(gnx[k][0], x0, acc[t0][0], false);
+                        acc[t0][1] = __builtin_amdgcn_fdot2(gnx[k][1], x1, acc[t0][1], false);
+                        acc[t1][0] = __builtin_amdgcn_fdot2(gc[k][0], x0, acc[t1][0], false);
+                        acc[t1][1] = __builtin_amdgcn_fdot2(gc[k][1], x1, acc[t1][1], false);
+                        acc[t2][0] = __builtin_amdgcn_fdot2(gm[k][0], x0, acc[t2][0], false);
+                        acc[t2][1] = __builtin_amdgcn_fdot2(gm[k][1], x1, acc[t2][1], false);
                     }
                 }
             }
         }
 #pragma unroll
-        for (int k = 0; k < P; ++k) {
-            gm[k] = gc[k];
-            gc[k] = gnx[k];
-            gnx[k] = gpre[k];
-        }
+        for (int k = 0; k < PP; ++k)
+#pragma unroll
+            for (int c = 0; c < CL; ++c) {
+                gm[k][c] = gc[k][c];
+                gc[k][c] = gnx[k][c];
+            }
+        pack_g(gnx);
     }
 
     // ---- combine: lanes with equal cl inside a wavefront, then wavefronts via LDS ----
@@ -227,31 +248,47 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_wgrad_kernel(const WgArgs a
     }
 }
 
-// out[tap][slab*SC + cs] = sum over the partial slots that belong to `slab`, added in
-// slot order by 16 interleaved running sums that are then combined as a fixed tree.
-__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const float* __restrict__ ws, float* __restrict__ gw,
-                                                           int n_rest, int n_slab, int SC, int C)
+// Second pass, two small kernels, fixed summation order (deterministic).  The workspace holds one
+// row per (n, h-chunk, w-patch, d-patch) of width RW = slabs*27*SC floats.  Pass 1 sums the rows of
+// each of kRedSeg row segments (64 columns x 4 interleaved row slices per workgroup, coalesced
+// 256-byte reads); pass 2 sums the segments and scatters to the [27][C] layout.
+constexpr int kRedSeg = 32;
+
+__global__ __launch_bounds__(256) void wgrad_reduce1_kernel(const float* __restrict__ ws, float* __restrict__ ws2,
+                                                            int n_rows, int RW, int rows_per_seg)
 {
-    __shared__ float part[16][17];
-    const int lo = threadIdx.x % 16;   // output within the group of 16
-    const int sl = threadIdx.x / 16;   // slice of the slot range
-    const int o = blockIdx.x * 16 + lo;  // index into [27][C]
-    float s = 0.0f;
-    if (o < 27 * C) {
-        const int tap = o / C, c = o % C;
-        const int slab = c / SC, cs = c % SC;
-        for (int r = sl; r < n_rest; r += 16) {
-            s += ws[((int64_t)(r * n_slab + slab) * 27 + tap) * SC + cs];
+    __shared__ float part[4][64];
+    const int lane_col = threadIdx.x % 64, slice = threadIdx.x / 64;
+    const int col = blockIdx.x * 64 + lane_col;
+    const int seg = blockIdx.y;
+    const int r0 = seg * rows_per_seg, r1 = min(r0 + rows_per_seg, n_rows);
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    if (col < RW) {
+        int r = r0 + slice;
+        for (; r + 12 < r1; r += 16) {
+            s0 += ws[(int64_t)r * RW + col];
+            s1 += ws[(int64_t)(r + 4) * RW + col];
+            s2 += ws[(int64_t)(r + 8) * RW + col];
+            s3 += ws[(int64_t)(r + 12) * RW + col];
         }
+        for (; r < r1; r += 4) s0 += ws[(int64_t)r * RW + col];
     }
-    part[sl][lo] = s;
+    part[slice][lane_col] = (s0 + s1) + (s2 + s3);
     __syncthreads();
-    if (sl == 0 && o < 27 * C) {
-        float v = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) v += part[i][lo];
-        gw[o] = v;
-    }
+    if (slice == 0 && col < RW)
+        ws2[(int64_t)seg * RW + col] = (part[0][lane_col] + part[1][lane_col]) + (part[2][lane_col] + part[3][lane_col]);
+}
+
+__global__ __launch_bounds__(256) void wgrad_reduce2_kernel(const float* __restrict__ ws2, float* __restrict__ gw,
+                                                            int nseg, int RW, int SC, int C)
+{
+    const int col = blockIdx.x * 256 + threadIdx.x;
+    if (col >= RW) return;
+    float s = 0.0f;
+    for (int g = 0; g < nseg; ++g) s += ws2[(int64_t)g * RW + col];
+    const int slab = col / (27 * SC), rem = col % (27 * SC);
+    const int tap = rem / SC, cs = rem % SC;
+    gw[tap * C + slab * SC + cs] = s;
 }
 
 struct WgPlan {
@@ -278,10 +315,10 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
         // measured best on MI355X at (1, C, 350, 350, 128)
         switch (p->cg) {
-            case 1: tile_w = 16; tile_d = 32; break;
+            case 1: tile_w = 8; tile_d = 32; break;
             case 2: tile_w = 8; tile_d = 32; break;
-            case 4: tile_w = 8; tile_d = 16; break;
-            default: tile_w = 8; tile_d = 8; break;
+            case 4: tile_w = 4; tile_d = 16; break;
+            default: tile_w = 4; tile_d = 8; break;
         }
         lane_channels = 2;
     }
@@ -307,10 +344,17 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     return KEROPS_OK;
 }
 
-template <int CG, int TW, int TD, int CL>
+// per-workgroup partials followed by the kRedSeg x RW buffer of the second pass
+static int64_t wgrad_ws_bytes(const WgPlan& p)
+{
+    const int64_t sc = p.cg * 8;
+    return (p.nblocks * 27 * sc + (int64_t)kRedSeg * p.n_slab * 27 * sc) * (int64_t)sizeof(float);
+}
+
+template <int CG, int TW, int TD>
 static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
 {
-    using Cfg = WgCfg<CG, TW, TD, CL, 256>;
+    using Cfg = WgCfg<CG, TW, TD, 256>;
     WgArgs a = base;
     a.n_wt = p.n_wt;
     a.n_dt = p.n_dt;
@@ -321,10 +365,18 @@ static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStrea
     hipLaunchKernelGGL(dwconv_wgrad_kernel<Cfg>, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
     int rc = check_launch("dwconv_wgrad");
     if (rc != KEROPS_OK) return rc;
-    const int n_rest = (int)(p.nblocks / p.n_slab);
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(ceil_div(27 * a.C, 16)), dim3(256), 0, stream, a.ws, gw, n_rest,
-                       p.n_slab, Cfg::SC, a.C);
-    return check_launch("dwconv_wgrad_reduce");
+    const int n_rows = (int)(p.nblocks / p.n_slab);
+    const int RW = p.n_slab * 27 * Cfg::SC;
+    const int nseg = std::min(kRedSeg, n_rows);
+    const int rows_per_seg = ceil_div(n_rows, nseg);
+    float* ws2 = a.ws + p.nblocks * 27 * Cfg::SC;
+    hipLaunchKernelGGL(wgrad_reduce1_kernel, dim3(ceil_div(RW, 64), nseg), dim3(256), 0, stream, a.ws, ws2, n_rows, RW,
+                       rows_per_seg);
+    rc = check_launch("dwconv_wgrad_reduce1");
+    if (rc != KEROPS_OK) return rc;
+    hipLaunchKernelGGL(wgrad_reduce2_kernel, dim3(ceil_div(RW, 256)), dim3(256), 0, stream, ws2, gw, nseg, RW, Cfg::SC,
+                       a.C);
+    return check_launch("dwconv_wgrad_reduce2");
 }
 
 }  // namespace kerops
@@ -338,7 +390,7 @@ extern "C" int64_t kerops_dwconv_wgrad_workspace_bytes(int32_t N, int32_t H, int
     WgPlan p;
     int rc = plan_wgrad(N, H, W, D, C, tile_w, tile_d, h_chunk, lane_channels, &p);
     if (rc != KEROPS_OK) return rc;
-    return p.nblocks * 27 * (p.cg * 8) * (int64_t)sizeof(float);
+    return wgrad_ws_bytes(p);
 }
 
 extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* workspace,
@@ -353,7 +405,7 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     WgPlan p;
     int rc = plan_wgrad(N, H, W, D, C, tile_w, tile_d, h_chunk, lane_channels, &p);
     if (rc != KEROPS_OK) return rc;
-    const int64_t need = p.nblocks * 27 * (p.cg * 8) * (int64_t)sizeof(float);
+    const int64_t need = wgrad_ws_bytes(p);
     if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
         set_error("dwconv_wgrad: workspace of %lld bytes required, %lld given", (long long)need,
                   (long long)workspace_bytes);
@@ -368,18 +420,18 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     a.D = D;
     a.C = C;
     hipStream_t s = (hipStream_t)stream;
-#define KEROPS_WG_CASE(CGv, TWv, TDv, CLv) \
-    if (p.cg == CGv && p.tile_w == TWv && p.tile_d == TDv && p.cl == CLv) \
-        return launch_wgrad<CGv, TWv, TDv, CLv>(a, p, gw, s);
-    KEROPS_WG_CASE(1, 16, 32, 2)
-    KEROPS_WG_CASE(1, 16, 32, 4)
-    KEROPS_WG_CASE(2, 8, 32, 2)
-    KEROPS_WG_CASE(2, 8, 32, 4)
-    KEROPS_WG_CASE(4, 8, 16, 2)
-    KEROPS_WG_CASE(4, 8, 16, 4)
-    KEROPS_WG_CASE(8, 8, 8, 2)
-    KEROPS_WG_CASE(8, 4, 16, 2)
-    KEROPS_WG_CASE(8, 4, 16, 4)
+#define KEROPS_WG_CASE(CGv, TWv, TDv)                                      \
+    if (p.cg == CGv && p.tile_w == TWv && p.tile_d == TDv && p.cl == 2) \
+        return launch_wgrad<CGv, TWv, TDv>(a, p, gw, s);
+    KEROPS_WG_CASE(1, 16, 32)
+    KEROPS_WG_CASE(1, 8, 32)
+    KEROPS_WG_CASE(2, 8, 32)
+    KEROPS_WG_CASE(2, 8, 16)
+    KEROPS_WG_CASE(4, 8, 16)
+    KEROPS_WG_CASE(4, 4, 16)
+    KEROPS_WG_CASE(8, 8, 8)
+    KEROPS_WG_CASE(8, 4, 16)
+    KEROPS_WG_CASE(8, 4, 8)
 #undef KEROPS_WG_CASE
     set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, p.tile_w, p.tile_d,
               p.cl);
