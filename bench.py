@@ -233,7 +233,7 @@ def main():
                                  'dwconv_frac_of_clone': fwd['frac_of_clone'],
                                  'wgrad_frac_of_clone': wg['frac_of_clone']}
                 continue
-            del x, g
+            x = g = None
             torch.cuda.empty_cache()
             x, g, wkc = make(c)
             cm = time_op(torch, lambda: x.clone(), it, wm)[0]
@@ -244,6 +244,29 @@ def main():
                              'dwconv_frac_hbm_peak': round(4 * V * c / fm / 1e6 / HBM_PEAK_GBPS, 4),
                              'wgrad_frac_hbm_peak': round(4 * V * c / wgm / 1e6 / HBM_PEAK_GBPS, 4)}
         ops['readme_table'] = table
+        # BASELINE config 5: fused depthwise-separable block with int8 output at (1,64,128,128,128)
+        del x, g
+        torch.cuda.empty_cache()
+        from kerops_amd.ops.fused import DWSepBlock, PointwiseLinear
+        from kerops_amd.ops.quantization import QuantInt8Sym
+        V5 = 128 ** 3
+        x5 = torch.randn(1, 128, 128, 128, 64, device=dev, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+        wk5 = (torch.randn(3, 3, 3, 64, device=dev, generator=gen) / math.sqrt(27)).half()
+        sc5 = torch.rand(64, device=dev, generator=gen) + 0.5
+        sh5 = torch.randn(64, device=dev, generator=gen) * math.sqrt(0.1)
+        Wm5 = (torch.randn(64, 128, device=dev, generator=gen) / 8.0).half()
+        stage1_bytes = 2 * V5 * 64 + 2 * V5 * 128
+        c5 = time_op(torch, lambda: x5.clone(), it, wm)[0]
+        c5_gbps = 4 * V5 * 64 / c5 / 1e6
+        ops['config5_block_stage1'] = figures(time_op(torch, lambda: DWSepBlock(x5, wk5, sc5, sh5, Wm5), it, wm)[0],
+                                              stage1_bytes, c5_gbps)
+        ops['config5_pointwise_64_128'] = figures(time_op(torch, lambda: PointwiseLinear(x5, Wm5), it, wm)[0],
+                                                  stage1_bytes, c5_gbps)
+        y5, am5 = DWSepBlock(x5, wk5, sc5, sh5, Wm5)
+        ops['config5_int8_pass'] = figures(time_op(torch, lambda: QuantInt8Sym(y5, am5), it, wm)[0], 3 * V5 * 128,
+                                           c5_gbps)
+        ops['config5_note'] = ('stage 1 = DWConv with fused BN+ReLU epilogue, then the MFMA 1x1x1 GEMM with fused '
+                               'max|y|; the fp16 intermediate (268 MB) passes through a workspace')
         ops['readme_table_note'] = 'C=8 (251 MB) fits the 256 MB Infinity Cache: its rows are not pure HBM numbers'
 
     cpu, cpu_torch = (None, None)

@@ -30,6 +30,15 @@ constexpr int kWave = 64;
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 
+// ---- cross-file launchers (defined in dwconv_fwd.hip / pointwise.hip) ----------------
+int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, const float* shift, int32_t N,
+                   int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
+                   int32_t lane_channels, void* stream);
+int pointwise_dispatch(const _Float16* x, const _Float16* Wm, const _Float16* add, _Float16* out, float* amax_ws,
+                       int64_t V, int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s);
+int pointwise_blocks(int64_t V);
+void launch_pw_absmax_final(const float* ws, int n, float* out, hipStream_t s);
+
 // ---- small host helpers -----------------------------------------------------
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -45,6 +45,8 @@ struct FwdArgs {
     const half_t* x;
     const half_t* wt;
     half_t* y;
+    const float* scale;  // optional fused epilogue y = max(acc * scale[c] + shift[c], 0)
+    const float* shift;
     int H, W, D, C;
     int n_wt, n_dt, n_hc, n_slab, h_chunk;
     uint32_t nblocks;
@@ -125,7 +127,7 @@ __device__ __forceinline__ void scatter_plane(const half_t* __restrict__ plane, 
 
 // OUT_FULL: every output piece of the patch lies inside the volume (true for all patches
 // but the last ones along W / D), so stores need no per-lane predicate.
-template <class Cfg, bool OUT_FULL>
+template <class Cfg, bool OUT_FULL, bool EPI>
 __device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)[2][Cfg::NCH + 1], int slab, int dt,
                                                 int wt_i, int hc, int n)
 {
@@ -161,6 +163,13 @@ __device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)
                 }
                 lw.single[kh][c] = wr[kh * 9 + 8][c];
             }
+    }
+
+    float esc[CL], esh[CL];
+#pragma unroll
+    for (int c = 0; c < CL; ++c) {
+        esc[c] = EPI ? a.scale[cslab + cl * CL + c] : 1.0f;
+        esh[c] = EPI ? a.shift[cslab + cl * CL + c] : 0.0f;
     }
 
     // staging assignment (fixed for the whole march)
@@ -246,7 +255,11 @@ __device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)
                 if (OUT_FULL || oval[k]) {
                     hv_t o;
 #pragma unroll
-                    for (int c = 0; c < CL; ++c) o[c] = (half_t)aF[k][c];
+                    for (int c = 0; c < CL; ++c) {
+                        float v = aF[k][c];
+                        if (EPI) v = fmaxf(__builtin_fmaf(v, esc[c], esh[c]), 0.0f);
+                        o[c] = (half_t)v;
+                    }
                     *reinterpret_cast<hv_t*>(yplane + ooff[k]) = o;
                 }
             }
@@ -266,7 +279,7 @@ __device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)
     }
 }
 
-template <class Cfg>
+template <class Cfg, bool EPI>
 __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const FwdArgs a)
 {
     __shared__ half8_t lds[2][Cfg::NCH + 1];  // +1: write-only dump slot for lanes with nothing to stage
@@ -283,9 +296,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const Fwd
     const int n = L / a.n_hc;
     const bool out_full = ((wt_i + 1) * Cfg::TW <= a.W) && ((dt + 1) * Cfg::TD <= a.D);
     if (out_full) {
-        dwconv_fwd_body<Cfg, true>(a, lds, slab, dt, wt_i, hc, n);
+        dwconv_fwd_body<Cfg, true, EPI>(a, lds, slab, dt, wt_i, hc, n);
     } else {
-        dwconv_fwd_body<Cfg, false>(a, lds, slab, dt, wt_i, hc, n);
+        dwconv_fwd_body<Cfg, false, EPI>(a, lds, slab, dt, wt_i, hc, n);
     }
 }
 
@@ -313,7 +326,18 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
         return KEROPS_E_BADARG;
     }
     a.nblocks = (uint32_t)nb;
-    hipLaunchKernelGGL(dwconv_fwd_kernel<Cfg>, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
+    if (a.scale) {
+        if constexpr (CG == 8 && TW == 8 && TD == 8 && CL == 2) {
+            hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+                               stream, a);
+        } else {
+            set_error("dwconv_fwd: the fused affine+ReLU epilogue is built for the 64-channel 8x8 patch only");
+            return KEROPS_E_BADARG;
+        }
+    } else {
+        hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, false>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
+                           a);
+    }
     return check_launch("dwconv_fwd");
 }
 
@@ -321,9 +345,10 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
 
 using namespace kerops;
 
-extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W,
-                                     int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
-                                     int32_t lane_channels, void* stream)
+namespace kerops {
+int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, const float* shift, int32_t N,
+                   int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
+                   int32_t lane_channels, void* stream)
 {
     if (!x || !wt || !y || !aligned16(x) || !aligned16(wt) || !aligned16(y)) {
         set_error("dwconv_fwd: null or misaligned pointer");
@@ -345,6 +370,8 @@ extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int
     a.x = (const half_t*)x;
     a.wt = (const half_t*)wt;
     a.y = (half_t*)y;
+    a.scale = scale;
+    a.shift = shift;
     a.H = H;
     a.W = W;
     a.D = D;
@@ -377,4 +404,13 @@ extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int
     set_error("dwconv_fwd: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, tile_w, tile_d,
               lane_channels);
     return KEROPS_E_BADARG;
+}
+}  // namespace kerops
+
+extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W,
+                                     int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
+                                     int32_t lane_channels, void* stream)
+{
+    return kerops::dwconv_fwd_run(x, wt, y, nullptr, nullptr, N, H, W, D, C, tile_w, tile_d, h_chunk, lane_channels,
+                                  stream);
 }

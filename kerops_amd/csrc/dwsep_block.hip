@@ -1,0 +1,59 @@
+// Depthwise-separable block: DWConv 3x3x3 -> folded inference BN (scale, shift) -> ReLU ->
+// pointwise 1x1x1 GEMM on the matrix cores, plus max|y| for the symmetric int8 pass.
+//
+//   t = fp16(max(dwconv(x, wt) * scale[c] + shift[c], 0))   (fp32 accumulate, one rounding)
+//   y = fp16(t @ Wm)                                          (fp32 accumulate, one rounding)
+//
+// Built from the two kernels of this library: the forward depthwise kernel with the affine+ReLU
+// epilogue fused into its store, and the pointwise MFMA kernel with the running max fused into
+// its write-back.  The intermediate t goes through the caller's workspace.
+#include "common.hpp"
+
+using namespace kerops;
+
+static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+extern "C" int64_t kerops_dwsep_block_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t Cin,
+                                                      int32_t Cout)
+{
+    if (N <= 0 || H <= 0 || W <= 0 || D <= 0) {
+        set_error("dwsep_block: non-positive extent");
+        return KEROPS_E_BADARG;
+    }
+    if (Cin != 64 || !(Cout == 16 || Cout == 32 || Cout == 64 || Cout == 128)) {
+        set_error("dwsep_block: built for Cin = 64 and Cout in {16,32,64,128} (got %d -> %d)", Cin, Cout);
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    const int64_t V = (int64_t)N * H * W * D;
+    return align256(V * Cin * 2) + align256((int64_t)pointwise_blocks(V) * 4);
+}
+
+extern "C" int kerops_dwsep_block_f16(const void* x, const void* wt, const float* scale, const float* shift,
+                                      const void* Wm, void* y, float* absmax, int32_t N, int32_t H, int32_t W,
+                                      int32_t D, int32_t Cin, int32_t Cout, void* workspace, int64_t workspace_bytes,
+                                      void* stream)
+{
+    const int64_t need = kerops_dwsep_block_workspace_bytes(N, H, W, D, Cin, Cout);
+    if (need < 0) return (int)need;
+    if (!x || !wt || !scale || !shift || !Wm || !y || !absmax || !aligned16(x) || !aligned16(wt) || !aligned16(Wm) ||
+        !aligned16(y)) {
+        set_error("dwsep_block: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
+        set_error("dwsep_block: workspace of %lld bytes required, %lld given", (long long)need,
+                  (long long)workspace_bytes);
+        return KEROPS_E_WORKSPACE;
+    }
+    const int64_t V = (int64_t)N * H * W * D;
+    half_t* t = (half_t*)workspace;
+    float* amax_ws = (float*)((char*)workspace + align256(V * Cin * 2));
+    int rc = dwconv_fwd_run(x, wt, t, scale, shift, N, H, W, D, Cin, 8, 8, 0, 2, stream);
+    if (rc != KEROPS_OK) return rc;
+    const int blocks = pointwise_blocks(V);
+    rc = pointwise_dispatch(t, (const half_t*)Wm, nullptr, (half_t*)y, amax_ws, V, Cin, Cout, false, true, blocks,
+                            (hipStream_t)stream);
+    if (rc != KEROPS_OK) return rc;
+    launch_pw_absmax_final(amax_ws, blocks, absmax, (hipStream_t)stream);
+    return check_launch("dwsep_block");
+}

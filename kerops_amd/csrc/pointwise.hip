@@ -1,19 +1,248 @@
-// placeholder until the MFMA kernels land
+// Pointwise (1x1x1) channel mixing on the matrix cores (gfx950):
+//
+//   out[v, co] = fp16( sum_ci act(x[v, ci]) * Wm[ci, co] )  (+ add[v, co] in fp16)
+//
+// x is [V][CIN] fp16 (the memory of a channels_last_3d activation), Wm is [CIN][COUT] fp16.
+// The op moves 2*V*(CIN + COUT) bytes and does only 2*V*CIN*COUT flops: it is HBM-bound, the
+// matrix cores are used so that the arithmetic never shows up next to the memory stream.
+//
+// Each wavefront owns tiles of 32 voxels.  The product is computed transposed,
+// out^T[co, v] = Wm^T[co, :] . x^T[:, v], with v_mfma_f32_32x32x8_f16: the A operand is a
+// 32-row block of Wm^T (held in registers for the whole kernel), the B operand is x^T, whose
+// per-lane fragment "4 consecutive k of voxel lane%32" is simply 8 contiguous bytes of the
+// voxel's channel vector.  Any permutation of k is allowed as long as A and B agree, so a lane
+// loads whole 16-byte chunks: lane half h = lane/32 takes chunks 2q+h, MFMA step s uses half
+// s%2 of chunk 2*(s/2)+h.  The fp32 result fragment of a lane is 4 consecutive output channels
+// of one voxel (x 4 row groups x COUT/32 blocks); it is rounded to fp16, bounced through a
+// wavefront-private LDS tile [32][COUT] and written back as 16-byte chunks, coalesced, with
+// the optional fp16 residual add and the optional running max|out| fused into that pass.
 #include "common.hpp"
+
+namespace kerops {
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kPwThreads = 256;
+constexpr int kPwWaves = kPwThreads / kWave;
+
+template <int CIN, int COUT>
+struct PwCfg {
+    static constexpr int MT = (COUT + 31) / 32;      // 32-row blocks of output channels
+    static constexpr int KS = CIN / 8;               // MFMA steps (k = 8 each)
+    static constexpr int NQ = CIN / 16;              // 16-byte chunks a lane loads per voxel
+    static constexpr int ROW_HALVES = COUT + 4;      // LDS row pitch: +8 bytes staggers the banks
+    static constexpr int TILE_HALVES = 32 * ROW_HALVES;
+    static constexpr int OUT_CHUNKS = 32 * COUT / 8; // 16-byte chunks of one output tile
+    static_assert(CIN % 16 == 0 && CIN <= 128, "CIN in {16,32,64,128}");
+    static_assert(COUT % 8 == 0 && COUT <= 128, "COUT in {16,32,64,128}");
+};
+
+template <int CIN, int COUT, bool RELU_IN, bool HAS_ADD, bool ABSMAX>
+__global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __restrict__ x,
+                                                               const half_t* __restrict__ Wm,
+                                                               const half_t* __restrict__ add,
+                                                               half_t* __restrict__ out, float* __restrict__ amax_ws,
+                                                               int64_t V)
+{
+    using Cfg = PwCfg<CIN, COUT>;
+    constexpr int MT = Cfg::MT, KS = Cfg::KS, NQ = Cfg::NQ, RH = Cfg::ROW_HALVES;
+    __shared__ __attribute__((aligned(16))) half_t tile[kPwWaves][Cfg::TILE_HALVES];
+    __shared__ float red[kPwWaves];
+
+    const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
+    const int vl = lane % 32, hl = lane / 32;
+
+    // A fragments: Wm^T[32*mt + vl][k], k = channels of (chunk 2*(s/2)+hl, half s%2)
+    half4_t wa[MT][KS];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int co = 32 * mt + vl;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int k0 = 8 * (2 * (s / 2) + hl) + 4 * (s % 2);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wa[mt][s][j] = (co < COUT) ? Wm[(k0 + j) * COUT + co] : (half_t)0;
+        }
+    }
+
+    float amax = 0.0f;
+    const int64_t ntiles = (V + 31) / 32;
+    const int64_t tiles_per_round = (int64_t)gridDim.x * kPwWaves;
+    const int64_t nrounds = (ntiles + tiles_per_round - 1) / tiles_per_round;
+    half_t* my = tile[wave];
+
+    for (int64_t r = 0; r < nrounds; ++r) {
+        const int64_t tidx = (r * gridDim.x + blockIdx.x) * kPwWaves + wave;
+        const bool live = tidx < ntiles;
+        const int64_t v0 = tidx * 32;
+        if (live) {
+            // B fragments: this lane's voxel, chunks 2q+hl
+            int64_t v = v0 + vl;
+            if (v >= V) v = V - 1;  // ragged last tile: clamp the read, the write is masked
+            half8_t xb[NQ];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) xb[q] = load_c8(x + v * CIN + 8 * (2 * q + hl));
+            if (RELU_IN) {
+#pragma unroll
+                for (int q = 0; q < NQ; ++q)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) xb[q][j] = xb[q][j] > (half_t)0 ? xb[q][j] : (half_t)0;
+            }
+            float16_t acc[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[mt][i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                half4_t b;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b[j] = xb[s / 2][4 * (s % 2) + j];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_32x32x8f16(wa[mt][s], b, acc[mt], 0, 0, 0);
+            }
+            // acc[mt][i]: output channel 32*mt + 8*(i/4) + 4*hl + i%4 of voxel vl
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int co = 32 * mt + 8 * gq + 4 * hl;
+                    if (co < COUT) {
+                        half4_t o;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) o[j] = (half_t)acc[mt][4 * gq + j];
+                        *reinterpret_cast<half4_t*>(my + vl * RH + co) = o;
+                    }
+                }
+        }
+        __syncthreads();
+        if (live) {
+#pragma unroll
+            for (int c0 = 0; c0 < Cfg::OUT_CHUNKS; c0 += kWave) {
+                const int c = c0 + lane;
+                const int row = c / (COUT / 8), cc = c % (COUT / 8);
+                if (c < Cfg::OUT_CHUNKS && v0 + row < V) {
+                    const half4_t lo = *reinterpret_cast<const half4_t*>(my + row * RH + cc * 8);
+                    const half4_t hi = *reinterpret_cast<const half4_t*>(my + row * RH + cc * 8 + 4);
+                    half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    const int64_t off = (v0 + row) * COUT + cc * 8;
+                    if (HAS_ADD) {
+                        const half8_t a8 = load_c8(add + off);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) o[j] = (half_t)((float)o[j] + (float)a8[j]);  // fp16 add, RNE
+                    }
+                    if (ABSMAX) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf((float)o[j]));
+                    }
+                    store_c8(out + off, o);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (ABSMAX) {
+        amax = wave_max(amax);
+        if (lane == 0) red[wave] = amax;
+        __syncthreads();
+        if (t == 0) {
+            float m = red[0];
+#pragma unroll
+            for (int wv = 1; wv < kPwWaves; ++wv) m = fmaxf(m, red[wv]);
+            amax_ws[blockIdx.x] = m;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void pw_absmax_final_kernel(const float* __restrict__ ws, int n,
+                                                              float* __restrict__ out)
+{
+    __shared__ float red[4];
+    float m = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) m = fmaxf(m, ws[i]);
+    m = wave_max(m);
+    if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) out[0] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+static int pw_blocks(int64_t V)
+{
+    const int64_t ntiles = (V + 31) / 32;
+    int64_t b = (ntiles + kPwWaves - 1) / kPwWaves;
+    if (b > 1024) b = 1024;  // 4 workgroups of 4 wavefronts per CU, each looping over tiles
+    return (int)std::max<int64_t>(b, 1);
+}
+
+template <int CIN, int COUT>
+static int launch_pw(const half_t* x, const half_t* Wm, const half_t* add, half_t* out, float* amax_ws, int64_t V,
+                     bool relu_in, bool absmax, int blocks, hipStream_t s)
+{
+#define KEROPS_PW_GO(R, A, M)                                                                                    \
+    hipLaunchKernelGGL((pointwise_kernel<CIN, COUT, R, A, M>), dim3(blocks), dim3(kPwThreads), 0, s, x, Wm, add, \
+                       out, amax_ws, V)
+    if (absmax) {
+        if (relu_in) KEROPS_PW_GO(true, false, true);
+        else KEROPS_PW_GO(false, false, true);
+    } else if (add) {
+        if (relu_in) KEROPS_PW_GO(true, true, false);
+        else KEROPS_PW_GO(false, true, false);
+    } else {
+        if (relu_in) KEROPS_PW_GO(true, false, false);
+        else KEROPS_PW_GO(false, false, false);
+    }
+#undef KEROPS_PW_GO
+    return check_launch("pointwise");
+}
+
+int pointwise_dispatch(const half_t* x, const half_t* Wm, const half_t* add, half_t* out, float* amax_ws, int64_t V,
+                       int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s)
+{
+#define KEROPS_PW_CASE(CI, CO) \
+    if (Cin == CI && Cout == CO) return launch_pw<CI, CO>(x, Wm, add, out, amax_ws, V, relu_in, absmax, blocks, s);
+    KEROPS_PW_CASE(16, 16)
+    KEROPS_PW_CASE(16, 32)
+    KEROPS_PW_CASE(32, 16)
+    KEROPS_PW_CASE(32, 32)
+    KEROPS_PW_CASE(64, 16)
+    KEROPS_PW_CASE(64, 32)
+    KEROPS_PW_CASE(64, 64)
+    KEROPS_PW_CASE(64, 128)
+    KEROPS_PW_CASE(128, 16)
+    KEROPS_PW_CASE(128, 32)
+    KEROPS_PW_CASE(128, 64)
+    KEROPS_PW_CASE(128, 128)
+    KEROPS_PW_CASE(16, 64)
+    KEROPS_PW_CASE(32, 64)
+    KEROPS_PW_CASE(16, 128)
+    KEROPS_PW_CASE(32, 128)
+#undef KEROPS_PW_CASE
+    set_error("pointwise: no kernel built for Cin=%d Cout=%d (both in {16,32,64,128})", Cin, Cout);
+    return KEROPS_E_UNSUPPORTED_C;
+}
+
+int pointwise_blocks(int64_t V) { return pw_blocks(V); }
+
+void launch_pw_absmax_final(const float* ws, int n, float* out, hipStream_t s)
+{
+    hipLaunchKernelGGL(pw_absmax_final_kernel, dim3(1), dim3(256), 0, s, ws, n, out);
+}
+
+}  // namespace kerops
+
 using namespace kerops;
-extern "C" int kerops_pointwise_f16(const void*, const void*, const void*, void*, int64_t, int32_t, int32_t, int32_t,
-                                    void*)
+
+extern "C" int kerops_pointwise_f16(const void* x, const void* Wm, const void* add, void* out, int64_t V, int32_t Cin,
+                                    int32_t Cout, int32_t relu_in, void* stream)
 {
-    set_error("pointwise: not built");
-    return KEROPS_E_UNSUPPORTED_C;
-}
-extern "C" int64_t kerops_dwsep_block_workspace_bytes(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t)
-{
-    return KEROPS_E_UNSUPPORTED_C;
-}
-extern "C" int kerops_dwsep_block_f16(const void*, const void*, const float*, const float*, const void*, void*, float*,
-                                      int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, void*, int64_t, void*)
-{
-    set_error("dwsep_block: not built");
-    return KEROPS_E_UNSUPPORTED_C;
+    if (!x || !Wm || !out || !aligned16(x) || !aligned16(Wm) || !aligned16(out) || (add && !aligned16(add))) {
+        set_error("pointwise: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    if (V <= 0) {
+        set_error("pointwise: V must be positive");
+        return KEROPS_E_BADARG;
+    }
+    return pointwise_dispatch((const half_t*)x, (const half_t*)Wm, (const half_t*)add, (half_t*)out, nullptr, V, Cin,
+                              Cout, relu_in != 0, false, pw_blocks(V), (hipStream_t)stream);
 }

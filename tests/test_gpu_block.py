@@ -1,0 +1,104 @@
+"""GPU parity tests of the pointwise MFMA kernel, the ReLULinearAdd drop-in and the fused
+depthwise-separable block with its int8 output (BASELINE config 5)."""
+import math
+
+import pytest
+import torch
+from torch.nn import functional as F
+
+import oracle
+from conftest import cpu_gen, rand_cl3d, rand_dw_weight
+from kerops_amd.ops.fused import DWSepBlock, DWSepBlockInt8, PointwiseLinear
+from kerops_amd.ops.linear import ReLULinearAdd
+from kerops_amd.utils import allclose_two_stage
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def rand_pw(g, cin, cout):
+    return (torch.randn(cin, cout, generator=g) / math.sqrt(cin)).half()
+
+
+@pytest.mark.parametrize('cin,cout', [(16, 16), (16, 32), (32, 16), (32, 32), (64, 64), (64, 128), (128, 128),
+                                      (128, 32), (16, 128)])
+@pytest.mark.parametrize('spatial', [(1, 3, 5, 7), (2, 4, 4, 4), (1, 1, 1, 1), (3, 2, 13, 37)])
+def test_relu_linear_add_matches_oracle(cin, cout, spatial):
+    g = cpu_gen(cin * 1000 + cout)
+    n, h, w, d = spatial
+    x = rand_cl3d(g, n, cin, h, w, d)
+    add = rand_cl3d(g, n, cout, h, w, d)
+    Wm = rand_pw(g, cin, cout)
+    out = ReLULinearAdd(x.to(DEV), Wm.to(DEV), add.to(DEV)).cpu()
+    ref = oracle.pointwise(x, Wm, add=add, relu_in=True)
+    assert out.shape == add.shape and out.stride() == add.stride()
+    # fp32 MFMA accumulation vs the oracle's fp64: at most one fp16 rounding apart before the add
+    assert allclose_two_stage(ref.contiguous(), out.contiguous(), rtol_strict=1e-4, atol_strict=1e-3,
+                              rtol_narrow=1e-3, atol_narrow=2e-3)
+    assert (out.float() - ref.float()).abs().max() <= 2.0 ** -9 * max(1.0, ref.abs().max().item())
+    same = (out.contiguous().view(torch.int16) == ref.contiguous().view(torch.int16)).float().mean().item()
+    assert same > 0.99, same
+    # the reference's own ground truth: 1x1x1 conv3d of relu(x) plus the residual
+    conv = F.conv3d(F.relu(x.float()), Wm.float().t().reshape(cout, cin, 1, 1, 1)).half() + add
+    assert torch.allclose(out.float(), conv.float(), rtol=1e-3, atol=2e-3)
+
+
+def test_pointwise_identity_and_no_relu():
+    g = cpu_gen(5)
+    x = rand_cl3d(g, 1, 64, 5, 6, 7)
+    eye = torch.eye(64, dtype=torch.float16)
+    y = PointwiseLinear(x.to(DEV), eye.to(DEV)).cpu()
+    assert torch.equal(y, x)  # exact: one nonzero product per output
+    y = PointwiseLinear(x.to(DEV), eye.to(DEV), relu_in=True).cpu()
+    assert torch.equal(y, F.relu(x))
+    perm = torch.randperm(64, generator=g)
+    P = torch.zeros(64, 64, dtype=torch.float16)
+    P[torch.arange(64), perm] = 1.0  # out[:, perm[i]] = x[:, i]
+    y = PointwiseLinear(x.to(DEV), P.to(DEV)).cpu()
+    assert torch.equal(y[:, perm], x)
+
+
+@pytest.mark.parametrize('shape', [(1, 64, 9, 11, 13), (2, 64, 3, 17, 8), (1, 64, 16, 16, 16)])
+@pytest.mark.parametrize('cout', [128, 32])
+def test_dwsep_block_matches_oracle(shape, cout):
+    g = cpu_gen(31)
+    x = rand_cl3d(g, *shape)
+    _, wk = rand_dw_weight(g, 64)
+    scale = torch.rand(64, generator=g) + 0.5
+    shift = torch.randn(64, generator=g) * math.sqrt(0.1)
+    Wm = rand_pw(g, 64, cout)
+    y, amax = DWSepBlock(x.to(DEV), wk.to(DEV), scale.to(DEV), shift.to(DEV), Wm.to(DEV))
+    ref = oracle.dwsep_block(x, wk, scale, shift, Wm)
+    assert torch.allclose(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)  # config 5 tolerance
+    assert (y.cpu().float() - ref.float()).abs().max() <= 2.0 ** -8 * max(1.0, ref.abs().max().item())
+    assert amax.item() == y.abs().max().item()
+    q, qscale, y2 = DWSepBlockInt8(x.to(DEV), wk.to(DEV), scale.to(DEV), shift.to(DEV), Wm.to(DEV))
+    assert torch.equal(y2, y)
+    # int8 bit-exact given the identical pre-quant tensor
+    assert torch.equal(q.cpu(), oracle.quant_i8_sym(y.cpu(), amax.item()))
+    assert qscale.item() == torch.tensor(amax.item(), dtype=torch.float32).div(127.0).item()
+
+
+def test_config5_full_shape():
+    """(1,64,128,128,128) -> y (1,128,128,128,128) -> int8: slab comparison with the oracle,
+    absmax against torch, int8 against the closed form on the build's own y."""
+    gen = torch.Generator(DEV).manual_seed(322)
+    x = torch.randn(1, 128, 128, 128, 64, device=DEV, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+    g = cpu_gen()
+    _, wk = rand_dw_weight(g, 64)
+    scale = torch.rand(64, generator=g) + 0.5
+    shift = torch.randn(64, generator=g) * math.sqrt(0.1)
+    Wm = (torch.randn(64, 128, generator=g) / 8.0).half()
+    q, qscale, y = DWSepBlockInt8(x, wk.to(DEV), scale.to(DEV), shift.to(DEV), Wm.to(DEV))
+    assert list(y.shape) == [1, 128, 128, 128, 128] and q.dtype == torch.int8
+    amax = y.abs().max().float()
+    assert qscale.item() == (amax / 127.0).item()
+    for (h0, h1) in [(0, 5), (61, 66), (123, 128)]:
+        ha, hb = max(h0 - 1, 0), min(h1 + 1, 128)
+        xs = x[:, :, ha:hb].cpu().contiguous(memory_format=torch.channels_last_3d)
+        ref = oracle.dwsep_block(xs, wk, scale, shift, Wm)[:, :, h0 - ha:h0 - ha + h1 - h0]
+        assert torch.allclose(y[:, :, h0:h1].cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    ys = y[:, :, 40:44].cpu()
+    assert torch.equal(q[:, :, 40:44].cpu(), oracle.quant_i8_sym(ys, amax.item()))
+    ref_q = torch.round(y.float() / qscale).clamp(-127, 127).to(torch.int8)
+    assert (ref_q != q).float().mean().item() < 1e-6  # torch divides by the same fp32 scale
