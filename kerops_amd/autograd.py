@@ -1,0 +1,103 @@
+"""torch.autograd.Function wrappers around the forward / backward op pairs.
+
+The reference exposes forward and backward as separate plain functions (`Stats` /
+`StatsBackward`, ...) and leaves wiring them into autograd to the user; these classes do that
+wiring once.  Each `apply` takes and returns exactly what the forward op does.  `DWConvFn` also
+provides the input gradient, which the reference lacks (a TODO at kerops/kernels/dw_conv.py:145):
+it is the same depthwise kernel run on the upstream gradient with the weight flipped along the
+three spatial axes.
+"""
+import torch
+
+from .ops.addition import AddStats, AddStatsBackward
+from .ops.avgpool import AvgPoolCeilStats, AvgPoolCeilStatsBackward
+from .ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
+from .ops.conv import DWConv, DWConvWGRAD
+from .ops.stats import Stats, StatsBackward
+
+
+def _cl3d(t):
+    return t.contiguous(memory_format=torch.channels_last_3d)
+
+
+class DWConvFn(torch.autograd.Function):
+    """y = DWConv(x, weight); weight is [3, 3, 3, C] fp16."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        ctx.save_for_backward(x, weight)
+        return DWConv(x, weight)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weight = ctx.saved_tensors
+        grad_out = _cl3d(grad_out)
+        grad_x = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_x = DWConv(grad_out, torch.flip(weight, dims=(0, 1, 2)).contiguous())
+        if ctx.needs_input_grad[1]:
+            grad_w = DWConvWGRAD(x, grad_out, out_dtype=weight.dtype)
+        return grad_x, grad_w
+
+
+class StatsFn(torch.autograd.Function):
+    """(mean, sqmean) = Stats(x)."""
+
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        mean, sqmean = Stats(x)
+        return mean, sqmean
+
+    @staticmethod
+    def backward(ctx, grad_mean, grad_sqmean):
+        (x,) = ctx.saved_tensors
+        return StatsBackward(x, grad_mean.contiguous(), grad_sqmean.contiguous())
+
+
+class AddStatsFn(torch.autograd.Function):
+    """(z, mean, sqmean) = AddStats(x, y)."""
+
+    @staticmethod
+    def forward(ctx, x, y):
+        z, mean, sqmean = AddStats(x, y)
+        ctx.save_for_backward(z)
+        return z, mean, sqmean
+
+    @staticmethod
+    def backward(ctx, grad_z, grad_mean, grad_sqmean):
+        (z,) = ctx.saved_tensors
+        g = AddStatsBackward(_cl3d(grad_z), grad_mean.contiguous(), grad_sqmean.contiguous(), z)
+        return g, g
+
+
+class ApplyBNReLUFn(torch.autograd.Function):
+    """y = relu(x * weight[c] + bias[c]); weight, bias fp32 with C elements."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight, bias)
+        return ApplyBNReLU(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weight, bias = ctx.saved_tensors
+        dx, dw, db = ApplyBNReLUBackward(x, weight.float(), bias.float(), _cl3d(grad_out))
+        return dx, dw.reshape(weight.shape).to(weight.dtype), db.reshape(bias.shape).to(bias.dtype)
+
+
+class AvgPoolCeilStatsFn(torch.autograd.Function):
+    """(pooled, mean, sqmean) = AvgPoolCeilStats(x)."""
+
+    @staticmethod
+    def forward(ctx, x):
+        pooled, mean, sqmean = AvgPoolCeilStats(x)
+        ctx.save_for_backward(pooled)
+        ctx.in_shape = tuple(x.shape)
+        return pooled, mean, sqmean
+
+    @staticmethod
+    def backward(ctx, grad_pooled, grad_mean, grad_sqmean):
+        (pooled,) = ctx.saved_tensors
+        return AvgPoolCeilStatsBackward(_cl3d(grad_pooled), grad_mean.float().contiguous(),
+                                        grad_sqmean.float().contiguous(), _cl3d(pooled), ctx.in_shape)

@@ -116,10 +116,12 @@ __device__ __forceinline__ void scatter_plane(const half_t* __restrict__ plane, 
                 aM[k][c] = __builtin_fmaf(xs, (float)lw.single[1][c], s);
             }
             if (DO_S) {
-                float s = 0.0f;  // the row hp+1 starts here: no separate zeroing pass
+                // the row hp+1 starts here: the mixed-precision FMA takes the literal 0 as addend,
+                // so no separate zeroing pass (and no register move) is needed
+                float s = __builtin_fmaf(xs, (float)lw.single[0][c], 0.0f);
 #pragma unroll
                 for (int p = 0; p < 4; ++p) s = __builtin_amdgcn_fdot2(pr[p], lw.pair[0][p][c], s, false);
-                aS[k][c] = __builtin_fmaf(xs, (float)lw.single[0][c], s);
+                aS[k][c] = s;
             }
         }
     }
@@ -302,10 +304,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const Fwd
     }
 }
 
-template <int CG, int TW, int TD, int CL, int WPE>
+template <int CG, int TW, int TD, int CL, int WPE, int NT = 256>
 static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t stream)
 {
-    using Cfg = FwdCfg<CG, TW, TD, CL, 256, WPE>;
+    using Cfg = FwdCfg<CG, TW, TD, CL, NT, WPE>;
     FwdArgs a = base;
     a.n_slab = a.C / (CG * 8);
     a.n_wt = ceil_div(a.W, TW);
@@ -327,11 +329,11 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
     }
     a.nblocks = (uint32_t)nb;
     if (a.scale) {
-        if constexpr (CG == 8 && TW == 8 && TD == 8 && CL == 2) {
+        if constexpr (CG == 8 && TW == 4 && TD == 8 && CL == 2 && NT == 256) {
             hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
                                stream, a);
         } else {
-            set_error("dwconv_fwd: the fused affine+ReLU epilogue is built for the 64-channel 8x8 patch only");
+            set_error("dwconv_fwd: the fused affine+ReLU epilogue is built for the 64-channel 4x8 patch only");
             return KEROPS_E_BADARG;
         }
     } else {
@@ -384,7 +386,7 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
             case 1: tile_w = 16; tile_d = 32; lane_channels = 4; break;
             case 2: tile_w = 8; tile_d = 32; lane_channels = 2; break;
             case 4: tile_w = 8; tile_d = 16; lane_channels = 2; break;
-            default: tile_w = 8; tile_d = 8; lane_channels = 2; break;
+            default: tile_w = 4; tile_d = 8; lane_channels = 2; break;
         }
     }
 #define KEROPS_FWD_CASE(CGv, TWv, TDv, CLv, WPEv)                                  \

@@ -144,8 +144,7 @@ __global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a
     };
     // g of one row for every pair: raw dwords (c0,c1) at d and d+1; rows outside the chunk and
     // positions outside the volume contribute zeros
-    uint32_t graw[PP][2];
-    auto load_g = [&](int h) {
+    auto load_g = [&](int h, uint32_t(&graw)[PP][2]) {
         const bool inb = (h >= hs) && (h < he);
         const char* gplane = reinterpret_cast<const char*>(gn_ptr + (inb ? h : hs) * plane_stride);
         const uint32_t dstep = (uint32_t)C * 2u;
@@ -159,7 +158,7 @@ __global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a
     };
     // packed (g[d][c], g[d+1][c]) per pair and channel for the rows hp-1, hp, hp+1
     half2_t gm[PP][CL], gc[PP][CL], gnx[PP][CL];
-    auto pack_g = [&](half2_t(&dst)[PP][CL]) {
+    auto pack_g = [&](half2_t(&dst)[PP][CL], const uint32_t(&graw)[PP][2]) {
 #pragma unroll
         for (int k = 0; k < PP; ++k) {
             dst[k][0] = pack_lo(graw[k][0], graw[k][1]);
@@ -171,8 +170,12 @@ __global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a
     for (int k = 0; k < PP; ++k)
 #pragma unroll
         for (int c = 0; c < CL; ++c) gm[k][c] = gc[k][c] = hz;
-    load_g(hs);
-    pack_g(gnx);
+    // g rows are fetched two steps before they are packed, so their latency is hidden behind
+    // a whole plane of arithmetic: ga holds row hp+2 (in flight or landed), gb receives row hp+3
+    uint32_t ga[PP][2], gb[PP][2];
+    load_g(hs, ga);
+    pack_g(gnx, ga);
+    load_g(hs + 1, ga);
 
     int parity = 0;
     prefetch_x(hs - 1);
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a
         }
         __syncthreads();
         if (hp + 1 <= he) prefetch_x(hp + 1);
-        load_g(hp + 2);
+        load_g(hp + 3, gb);
         if (inb) {
             const half_t* plane = reinterpret_cast<const half_t*>(buf);
 #pragma unroll
@@ -220,7 +223,12 @@ __global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a
                 gm[k][c] = gc[k][c];
                 gc[k][c] = gnx[k][c];
             }
-        pack_g(gnx);
+        pack_g(gnx, ga);
+#pragma unroll
+        for (int k = 0; k < PP; ++k) {
+            ga[k][0] = gb[k][0];
+            ga[k][1] = gb[k][1];
+        }
     }
 
     // ---- combine: lanes with equal cl inside a wavefront, then wavefronts via LDS ----

@@ -14,7 +14,7 @@ from .._common import cl3d, next_power_of_2, require_cuda
 # tile extent along W).  A missing key means "no kernel for this channel count".
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
 _TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
-_TILE_W = {8: 16, 16: 8, 32: 8, 64: 8, 128: 8}
+_TILE_W = {8: 16, 16: 8, 32: 8, 64: 4, 128: 4}
 _LANE_C = {8: 4, 16: 2, 32: 2, 64: 2, 128: 2}
 
 
