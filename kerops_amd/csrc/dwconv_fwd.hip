@@ -329,11 +329,11 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
     }
     a.nblocks = (uint32_t)nb;
     if (a.scale) {
-        if constexpr (CG == 8 && TW == 4 && TD == 8 && CL == 2 && NT == 256) {
+        if constexpr (CG == 8 && TW == 8 && TD == 8 && CL == 2 && NT == 512) {
             hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
                                stream, a);
         } else {
-            set_error("dwconv_fwd: the fused affine+ReLU epilogue is built for the 64-channel 4x8 patch only");
+            set_error("dwconv_fwd: the fused affine+ReLU epilogue is built for the 64-channel 8x8 patch only");
             return KEROPS_E_BADARG;
         }
     } else {
@@ -386,22 +386,23 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
             case 1: tile_w = 16; tile_d = 32; lane_channels = 4; break;
             case 2: tile_w = 8; tile_d = 32; lane_channels = 2; break;
             case 4: tile_w = 8; tile_d = 16; lane_channels = 2; break;
-            default: tile_w = 4; tile_d = 8; lane_channels = 2; break;
+            default: tile_w = 8; tile_d = 8; lane_channels = 2; break;
         }
     }
-#define KEROPS_FWD_CASE(CGv, TWv, TDv, CLv, WPEv)                                  \
+    // (channel groups of 8, patch W, patch D, channels per lane, wavefronts per SIMD, threads)
+#define KEROPS_FWD_CASE(CGv, TWv, TDv, CLv, WPEv, NTv)                             \
     if (cg == CGv && tile_w == TWv && tile_d == TDv && lane_channels == CLv) \
-        return launch_fwd<CGv, TWv, TDv, CLv, WPEv>(a, N, h_chunk, s);
-    KEROPS_FWD_CASE(1, 16, 32, 4, 3)
-    KEROPS_FWD_CASE(1, 16, 32, 2, 3)
-    KEROPS_FWD_CASE(2, 8, 32, 4, 3)
-    KEROPS_FWD_CASE(2, 8, 32, 2, 3)
-    KEROPS_FWD_CASE(4, 8, 16, 4, 3)
-    KEROPS_FWD_CASE(4, 8, 16, 2, 3)
-    KEROPS_FWD_CASE(8, 4, 8, 4, 3)
-    KEROPS_FWD_CASE(8, 4, 8, 2, 4)
-    KEROPS_FWD_CASE(8, 4, 16, 2, 3)
-    KEROPS_FWD_CASE(8, 8, 8, 2, 3)
+        return launch_fwd<CGv, TWv, TDv, CLv, WPEv, NTv>(a, N, h_chunk, s);
+    KEROPS_FWD_CASE(1, 16, 32, 4, 3, 256)
+    KEROPS_FWD_CASE(1, 16, 32, 2, 3, 256)
+    KEROPS_FWD_CASE(2, 8, 32, 4, 3, 256)
+    KEROPS_FWD_CASE(2, 8, 32, 2, 3, 256)
+    KEROPS_FWD_CASE(4, 8, 16, 4, 3, 256)
+    KEROPS_FWD_CASE(4, 8, 16, 2, 3, 256)
+    KEROPS_FWD_CASE(8, 4, 8, 4, 3, 256)
+    KEROPS_FWD_CASE(8, 4, 8, 2, 4, 256)
+    KEROPS_FWD_CASE(8, 4, 16, 2, 3, 256)
+    KEROPS_FWD_CASE(8, 8, 8, 2, 4, 512)
 #undef KEROPS_FWD_CASE
     set_error("dwconv_fwd: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, tile_w, tile_d,
               lane_channels);

@@ -12,9 +12,9 @@ from .._common import cl3d, next_power_of_2, require_cuda
 # gfx950 launch table, keyed by channel count like the reference's `warps` / `dblock`
 # (kerops/ops/conv/dwconv.py:10-17): (wavefronts per workgroup, tile extent along D,
 # tile extent along W).  A missing key means "no kernel for this channel count".
-_WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
+_WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
 _TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
-_TILE_W = {8: 16, 16: 8, 32: 8, 64: 4, 128: 4}
+_TILE_W = {8: 16, 16: 8, 32: 8, 64: 8, 128: 8}
 _LANE_C = {8: 4, 16: 2, 32: 2, 64: 2, 128: 2}
 
 
@@ -61,7 +61,8 @@ def DWConv(
 
     ACCTYPE / num_warps / D_block keep the reference's names: accumulation is always
     fp32 ('float16' is accepted and computed in fp32), num_warps is the number of
-    64-wide wavefronts per workgroup (the built kernels use 4) and D_block the tile
+    64-wide wavefronts per workgroup (fixed per patch shape in the library: 4, or 8 for the
+    8x8 patch) and D_block the tile
     extent along D.  W_block (tile extent along W) and H_chunk (rows one workgroup
     marches over, 0 = automatic) and lane_channels (channels one lane owns: 2, 4 or 8)
     are additional gfx950 knobs.
@@ -75,7 +76,7 @@ def DWConv(
     assert list(weight.shape) == [3, 3, 3, channels]
     assert D_block == next_power_of_2(D_block)
     {'float32': None, 'float16': None}[ACCTYPE]
-    assert num_warps == 4, 'the gfx950 kernels are built for 4 wavefronts per workgroup'
+    assert num_warps in (4, 8), 'the gfx950 kernels are built with 4 or 8 wavefronts per workgroup'
     require_cuda(x, weight)
 
     bsize, _, H, W, D = x.shape
