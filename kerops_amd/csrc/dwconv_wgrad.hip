@@ -59,7 +59,7 @@ __device__ __forceinline__ half2_t pack_hi(uint32_t a, uint32_t b)
 }
 
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, 3) void dwconv_wgrad_kernel(const WgArgs a)
+__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, PP = Cfg::PP, NLD = Cfg::NLD, NCH = Cfg::NCH;
     constexpr int PD = Cfg::PD, CL = Cfg::CL, NCL = Cfg::NCL, SC = Cfg::SC;
@@ -359,10 +359,10 @@ static int64_t wgrad_ws_bytes(const WgPlan& p)
     return (p.nblocks * 27 * sc + (int64_t)kRedSeg * p.n_slab * 27 * sc) * (int64_t)sizeof(float);
 }
 
-template <int CG, int TW, int TD>
+template <int CG, int TW, int TD, int NT>
 static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
 {
-    using Cfg = WgCfg<CG, TW, TD, 256>;
+    using Cfg = WgCfg<CG, TW, TD, NT>;
     WgArgs a = base;
     a.n_wt = p.n_wt;
     a.n_dt = p.n_dt;
@@ -428,18 +428,19 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     a.D = D;
     a.C = C;
     hipStream_t s = (hipStream_t)stream;
-#define KEROPS_WG_CASE(CGv, TWv, TDv)                                      \
+    // (channel groups of 8, patch W, patch D, threads)
+#define KEROPS_WG_CASE(CGv, TWv, TDv, NTv)                                 \
     if (p.cg == CGv && p.tile_w == TWv && p.tile_d == TDv && p.cl == 2) \
-        return launch_wgrad<CGv, TWv, TDv>(a, p, gw, s);
-    KEROPS_WG_CASE(1, 16, 32)
-    KEROPS_WG_CASE(1, 8, 32)
-    KEROPS_WG_CASE(2, 8, 32)
-    KEROPS_WG_CASE(2, 8, 16)
-    KEROPS_WG_CASE(4, 8, 16)
-    KEROPS_WG_CASE(4, 4, 16)
-    KEROPS_WG_CASE(8, 8, 8)
-    KEROPS_WG_CASE(8, 4, 16)
-    KEROPS_WG_CASE(8, 4, 8)
+        return launch_wgrad<CGv, TWv, TDv, NTv>(a, p, gw, s);
+    KEROPS_WG_CASE(1, 16, 32, 256)
+    KEROPS_WG_CASE(1, 8, 32, 256)
+    KEROPS_WG_CASE(2, 8, 32, 256)
+    KEROPS_WG_CASE(2, 8, 16, 256)
+    KEROPS_WG_CASE(4, 8, 16, 256)
+    KEROPS_WG_CASE(4, 4, 16, 256)
+    KEROPS_WG_CASE(8, 8, 8, 512)
+    KEROPS_WG_CASE(8, 4, 16, 256)
+    KEROPS_WG_CASE(8, 4, 8, 256)
 #undef KEROPS_WG_CASE
     set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, p.tile_w, p.tile_d,
               p.cl);
