@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
                     hv t;
 #pragma unroll
                     for (int j = 0; j < V; ++j) t[j] = (half_t)0;
-                    if (ok) t = ld<V>(x, base + a * sH + b * sW + e * sD);
+                    if (ok) t = ld_stream<V>(x, base + a * sH + b * sW + e * sD);
                     v[a][b][e] = t;
                 }
         const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
             acc[0][j] += m;
             acc[1][j] = __builtin_fmaf(m, m, acc[1][j]);
         }
-        st<V>(y, i, o);
+        st_stream<V>(y, i, o);
     }
     block_channel_partials<2, V>(acc, p.CG, red, ws + (int64_t)blockIdx.x * 2 * p.CG * V);
 }
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_bwd_kernel(const half_
         const int n = (int)(r / p.Ho);
         const bool h1 = 2 * hO + 1 < p.H, w1 = 2 * wO + 1 < p.W, d1 = 2 * dO + 1 < p.D;
         const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
-        const hv g = ld<V>(inpgrad, i), o = ld<V>(output, i);
+        const hv g = ld_stream<V>(inpgrad, i), o = ld_stream<V>(output, i);
         hv res;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_bwd_kernel(const half_
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
                     const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
-                    if (ok) st<V>(dx, base + a * sH + b * sW + e * sD, res);
+                    if (ok) st_stream<V>(dx, base + a * sH + b * sW + e * sD, res);
                 }
     }
 }
@@ -146,7 +146,7 @@ static int pool_plan(const char* op, int N, int H, int W, int D, int C, int* blo
     p->C = C;
     p->CG = C / V;
     *nchunks = (int64_t)N * p->Ho * p->Wo * p->Do * p->CG;
-    if (*blocks <= 0) *blocks = stream_blocks_default(*nchunks);
+    if (*blocks <= 0) *blocks = stream_blocks_default(*nchunks, 512);
     if (*blocks > 65536) {
         set_error("%s: blocks must be <= 65536", op);
         return KEROPS_E_BADARG;

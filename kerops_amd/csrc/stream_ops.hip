@@ -27,12 +27,12 @@ __global__ __launch_bounds__(kStreamThreads) void stats_kernel(const half_t* x, 
     for (int j = 0; j < V; ++j) acc[0][j] = acc[1][j] = 0.0f;
 
     auto body = [&](int64_t i) {
-        hv v = ld<V>(x, i);
+        hv v = ld_stream<V>(x, i);
         if (ADD) {
-            const hv u = ld<V>(y, i);
+            const hv u = ld_stream<V>(y, i);
 #pragma unroll
             for (int j = 0; j < V; ++j) v[j] = (half_t)((float)v[j] + (float)u[j]);  // fp16 sum, RNE
-            st<V>(z, i, v);
+            st_stream<V>(z, i, v);
         }
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -44,7 +44,8 @@ __global__ __launch_bounds__(kStreamThreads) void stats_kernel(const half_t* x, 
     int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
     for (; i + 3 * T < nchunks; i += 4 * T) {
         if (!ADD) {
-            const hv v0 = ld<V>(x, i), v1 = ld<V>(x, i + T), v2 = ld<V>(x, i + 2 * T), v3 = ld<V>(x, i + 3 * T);
+            const hv v0 = ld_stream<V>(x, i), v1 = ld_stream<V>(x, i + T), v2 = ld_stream<V>(x, i + 2 * T),
+                     v3 = ld_stream<V>(x, i + 3 * T);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 const float f0 = (float)v0[j], f1 = (float)v1[j], f2 = (float)v2[j], f3 = (float)v3[j];
@@ -111,10 +112,10 @@ __global__ __launch_bounds__(kStreamThreads) void stats_bwd_kernel(const half_t*
         mg[j] = __fdiv_rn(mean_grad[cg * V + j], fm);
     }
     for (; i < nchunks; i += T) {
-        const hv v = ld<V>(x, i);
+        const hv v = ld_stream<V>(x, i);
         hv o;
         if (ADD) {
-            const hv g = ld<V>(add_grad, i);
+            const hv g = ld_stream<V>(add_grad, i);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 const float a = __fdiv_rn(__fmul_rn(__fmul_rn(2.0f, (float)v[j]), sg[j]), fm);
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(kStreamThreads) void stats_bwd_kernel(const half_t*
                 o[j] = (half_t)__fadd_rn(a, mg[j]);
             }
         }
-        st<V>(dx, i, o);
+        st_stream<V>(dx, i, o);
     }
 }
 
@@ -155,13 +156,13 @@ __global__ __launch_bounds__(kStreamThreads) void bnrelu_fwd_kernel(const half_t
         return o;
     };
     for (; i + 3 * T < nchunks; i += 4 * T) {
-        const hv v0 = ld<V>(x, i), v1 = ld<V>(x, i + T), v2 = ld<V>(x, i + 2 * T), v3 = ld<V>(x, i + 3 * T);
-        st<V>(y, i, act(v0));
-        st<V>(y, i + T, act(v1));
-        st<V>(y, i + 2 * T, act(v2));
-        st<V>(y, i + 3 * T, act(v3));
+        const hv v0 = ld_stream<V>(x, i), v1 = ld_stream<V>(x, i + T), v2 = ld_stream<V>(x, i + 2 * T), v3 = ld_stream<V>(x, i + 3 * T);
+        st_stream<V>(y, i, act(v0));
+        st_stream<V>(y, i + T, act(v1));
+        st_stream<V>(y, i + 2 * T, act(v2));
+        st_stream<V>(y, i + 3 * T, act(v3));
     }
-    for (; i < nchunks; i += T) st<V>(y, i, act(ld<V>(x, i)));
+    for (; i < nchunks; i += T) st_stream<V>(y, i, act(ld_stream<V>(x, i)));
 }
 
 template <int V>
@@ -196,15 +197,15 @@ __global__ __launch_bounds__(kStreamThreads) void bnrelu_bwd_kernel(const half_t
             acc[0][j] = __builtin_fmaf(xf, gm, acc[0][j]);
             acc[1][j] += gm;
         }
-        st<V>(dx, k, o);
+        st_stream<V>(dx, k, o);
     };
     for (; i + T < nchunks; i += 2 * T) {
-        const hv x0 = ld<V>(x, i), x1 = ld<V>(x, i + T);
-        const hv g0 = ld<V>(g, i), g1 = ld<V>(g, i + T);
+        const hv x0 = ld_stream<V>(x, i), x1 = ld_stream<V>(x, i + T);
+        const hv g0 = ld_stream<V>(g, i), g1 = ld_stream<V>(g, i + T);
         body(i, x0, g0);
         body(i + T, x1, g1);
     }
-    for (; i < nchunks; i += T) body(i, ld<V>(x, i), ld<V>(g, i));
+    for (; i < nchunks; i += T) body(i, ld_stream<V>(x, i), ld_stream<V>(g, i));
     block_channel_partials<2, V>(acc, CG, red, ws + (int64_t)blockIdx.x * 2 * CG * V);
 }
 
@@ -224,28 +225,59 @@ __device__ __forceinline__ uint32_t quant_u8_one(float t, float window, float tw
     return (uint32_t)t;  // truncation toward zero
 }
 
+// The byte-wide side of the quantisers is moved 16 bytes per lane like everything else: a thread
+// handles 16 consecutive elements (two 16-byte fp16 loads or four fp32 loads per 16-byte store).
+template <typename T>
+__device__ __forceinline__ void load16(const T* p, float (&f)[16])
+{
+    typedef T tv8 __attribute__((ext_vector_type(8)));
+    const tv8 a = __builtin_nontemporal_load(reinterpret_cast<const tv8*>(p));
+    const tv8 b = __builtin_nontemporal_load(reinterpret_cast<const tv8*>(p + 8));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        f[j] = (float)a[j];
+        f[8 + j] = (float)b[j];
+    }
+}
+template <typename T>
+__device__ __forceinline__ void store16(T* p, const float (&f)[16])
+{
+    typedef T tv8 __attribute__((ext_vector_type(8)));
+    tv8 a, b;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        a[j] = (T)f[j];
+        b[j] = (T)f[8 + j];
+    }
+    __builtin_nontemporal_store(a, reinterpret_cast<tv8*>(p));
+    __builtin_nontemporal_store(b, reinterpret_cast<tv8*>(p + 8));
+}
+__device__ __forceinline__ u32x4_t pack16(const uint32_t (&b)[16])
+{
+    u32x4_t o;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) o[w] = b[4 * w] | (b[4 * w + 1] << 8) | (b[4 * w + 2] << 16) | (b[4 * w + 3] << 24);
+    return o;
+}
+
 template <typename T>
 __global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
                                                                   int64_t numel, float window)
 {
     const float two_w = __fmul_rn(2.0f, window);
-    const int64_t nchunks = numel / 8;
+    const int64_t ngroups = numel / 16;
     const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
     const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    typedef T tv8 __attribute__((ext_vector_type(8)));
-    for (int64_t i = gid; i < nchunks; i += Tn) {
-        const tv8 v = *reinterpret_cast<const tv8*>(x + i * 8);
-        uint32_t lo = 0, hi = 0;
+    for (int64_t i = gid; i < ngroups; i += Tn) {
+        float f[16];
+        load16<T>(x + i * 16, f);
+        uint32_t b[16];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            lo |= quant_u8_one(to_f32(v[j]), window, two_w) << (8 * j);
-            hi |= quant_u8_one(to_f32(v[4 + j]), window, two_w) << (8 * j);
-        }
-        u32x2_t o = {lo, hi};
-        *reinterpret_cast<u32x2_t*>(q + i * 8) = o;
+        for (int j = 0; j < 16; ++j) b[j] = quant_u8_one(f[j], window, two_w);
+        __builtin_nontemporal_store(pack16(b), reinterpret_cast<u32x4_t*>(q + i * 16));
     }
     if (gid == 0) {
-        for (int64_t k = nchunks * 8; k < numel; ++k) q[k] = (uint8_t)quant_u8_one(to_f32(x[k]), window, two_w);
+        for (int64_t k = ngroups * 16; k < numel; ++k) q[k] = (uint8_t)quant_u8_one(to_f32(x[k]), window, two_w);
     }
 }
 
@@ -254,22 +286,19 @@ __global__ __launch_bounds__(kStreamThreads) void dequant_u8_kernel(const uint8_
                                                                     T* __restrict__ out, int64_t numel, float window)
 {
     const float scale = __fdiv_rn(__fmul_rn(2.0f, window), 255.0f);
-    const int64_t nchunks = numel / 8;
+    const int64_t ngroups = numel / 16;
     const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
     const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    typedef T tv8 __attribute__((ext_vector_type(8)));
-    for (int64_t i = gid; i < nchunks; i += Tn) {
-        const u32x2_t v = *reinterpret_cast<const u32x2_t*>(q + i * 8);
-        tv8 o;
+    for (int64_t i = gid; i < ngroups; i += Tn) {
+        const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(q + i * 16));
+        float f[16];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            o[j] = (T)__fsub_rn(__fmul_rn((float)((v[0] >> (8 * j)) & 0xffu), scale), window);
-            o[4 + j] = (T)__fsub_rn(__fmul_rn((float)((v[1] >> (8 * j)) & 0xffu), scale), window);
-        }
-        *reinterpret_cast<tv8*>(out + i * 8) = o;
+        for (int j = 0; j < 16; ++j)
+            f[j] = __fsub_rn(__fmul_rn((float)((v[j / 4] >> (8 * (j % 4))) & 0xffu), scale), window);
+        store16<T>(out + i * 16, f);
     }
     if (gid == 0) {
-        for (int64_t k = nchunks * 8; k < numel; ++k)
+        for (int64_t k = ngroups * 16; k < numel; ++k)
             out[k] = (T)__fsub_rn(__fmul_rn((float)q[k], scale), window);
     }
 }
@@ -284,8 +313,8 @@ __global__ __launch_bounds__(kStreamThreads) void absmax_kernel(const half_t* __
     float m = 0.0f;
     int64_t i = gid;
     for (; i + 3 * Tn < nchunks; i += 4 * Tn) {
-        const half8_t v0 = load_c8(y + i * 8), v1 = load_c8(y + (i + Tn) * 8), v2 = load_c8(y + (i + 2 * Tn) * 8),
-                      v3 = load_c8(y + (i + 3 * Tn) * 8);
+        const half8_t v0 = load_c8_nt(y + i * 8), v1 = load_c8_nt(y + (i + Tn) * 8), v2 = load_c8_nt(y + (i + 2 * Tn) * 8),
+                      v3 = load_c8_nt(y + (i + 3 * Tn) * 8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             m = fmaxf(m, fmaxf(fmaxf(fabsf((float)v0[j]), fabsf((float)v1[j])),
@@ -293,7 +322,7 @@ __global__ __launch_bounds__(kStreamThreads) void absmax_kernel(const half_t* __
         }
     }
     for (; i < nchunks; i += Tn) {
-        const half8_t v = load_c8(y + i * 8);
+        const half8_t v = load_c8_nt(y + i * 8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf((float)v[j]));
     }
@@ -341,24 +370,19 @@ __global__ __launch_bounds__(kStreamThreads) void quant_i8_kernel(const half_t* 
 {
     const float scale = __fdiv_rn(absmax[0], 127.0f);
     const bool zero = (scale == 0.0f);
-    const int64_t nchunks = numel / 8;
+    const int64_t ngroups = numel / 16;
     const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
     const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    for (int64_t i = gid; i < nchunks; i += Tn) {
-        const half8_t v = load_c8(y + i * 8);
-        uint32_t lo = 0, hi = 0;
-        if (!zero) {
+    for (int64_t i = gid; i < ngroups; i += Tn) {
+        float f[16];
+        load16<half_t>(y + i * 16, f);
+        uint32_t b[16];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                lo |= quant_i8_one((float)v[j], scale) << (8 * j);
-                hi |= quant_i8_one((float)v[4 + j], scale) << (8 * j);
-            }
-        }
-        u32x2_t o = {lo, hi};
-        *reinterpret_cast<u32x2_t*>(q + i * 8) = o;
+        for (int j = 0; j < 16; ++j) b[j] = zero ? 0u : quant_i8_one(f[j], scale);
+        __builtin_nontemporal_store(pack16(b), reinterpret_cast<u32x4_t*>(q + i * 16));
     }
     if (gid == 0) {
-        for (int64_t k = nchunks * 8; k < numel; ++k)
+        for (int64_t k = ngroups * 16; k < numel; ++k)
             q[k] = zero ? (int8_t)0 : (int8_t)quant_i8_one((float)y[k], scale);
     }
 }
@@ -539,7 +563,7 @@ static int check_flat(const char* op, const void* a, const void* b, int64_t nume
         set_error("%s: null or misaligned pointer, or non-positive numel", op);
         return KEROPS_E_BADARG;
     }
-    if (*blocks <= 0) *blocks = stream_blocks_default(ceil_div64(numel, 8));
+    if (*blocks <= 0) *blocks = stream_blocks_default(ceil_div64(numel, 16), 1280);
     return KEROPS_OK;
 }
 
@@ -583,14 +607,14 @@ extern "C" int kerops_dequant_u8_window(const void* q, void* out, int32_t dtype,
 
 extern "C" int64_t kerops_absmax_workspace_bytes(int32_t blocks)
 {
-    if (blocks <= 0) blocks = 2048;
+    if (blocks <= 0) blocks = 768;
     return (int64_t)blocks * (int64_t)sizeof(float);
 }
 
 extern "C" int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, void* workspace,
                                  int64_t workspace_bytes, int32_t blocks, void* stream)
 {
-    if (blocks <= 0) blocks = 2048;
+    if (blocks <= 0) blocks = 768;
     int b = blocks;
     int rc = check_flat("absmax", y, absmax, numel, &b);
     if (rc != KEROPS_OK) return rc;
