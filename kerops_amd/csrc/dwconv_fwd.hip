@@ -262,7 +262,7 @@ __device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)
                         if (EPI) v = fmaxf(__builtin_fmaf(v, esc[c], esh[c]), 0.0f);
                         o[c] = (half_t)v;
                     }
-                    *reinterpret_cast<hv_t*>(yplane + ooff[k]) = o;
+                    __builtin_nontemporal_store(o, reinterpret_cast<hv_t*>(yplane + ooff[k]));  // written once, never re-read
                 }
             }
         }
@@ -316,7 +316,7 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
         // enough workgroups to fill 256 CUs several times over, but rows per chunk
         // large enough that the two halo planes of a chunk stay a small overhead
         const int64_t per_plane = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
-        const int want_chunks = (int)std::max<int64_t>(1, ceil_div64(4096, per_plane));
+        const int want_chunks = (int)std::max<int64_t>(1, ceil_div64(3072, per_plane));
         h_chunk = std::max(ceil_div(a.H, want_chunks), std::min(a.H, 24));
     }
     h_chunk = std::min(h_chunk, a.H);
@@ -383,9 +383,9 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
         // measured best on MI355X at (1, C, 350, 350, 128)
         switch (cg) {
-            case 1: tile_w = 16; tile_d = 32; lane_channels = 4; break;
-            case 2: tile_w = 8; tile_d = 32; lane_channels = 2; break;
-            case 4: tile_w = 8; tile_d = 16; lane_channels = 2; break;
+            case 1: tile_w = 16; tile_d = 32; lane_channels = 2; break;
+            case 2: tile_w = 8; tile_d = 32; lane_channels = 4; break;
+            case 4: tile_w = 8; tile_d = 16; lane_channels = 4; break;
             default: tile_w = 8; tile_d = 8; lane_channels = 2; break;
         }
     }

@@ -150,8 +150,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
         const uint32_t dstep = (uint32_t)C * 2u;
 #pragma unroll
         for (int k = 0; k < PP; ++k) {
-            const uint32_t v0 = *reinterpret_cast<const uint32_t*>(gplane + poff[k]);
-            const uint32_t v1 = *reinterpret_cast<const uint32_t*>(gplane + poff[k] + (pv1[k] ? dstep : 0u));
+            // g is read exactly once: streaming hint, it should not displace the x halo rows in L2
+            const uint32_t v0 = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(gplane + poff[k]));
+            const uint32_t v1 =
+                __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(gplane + poff[k] + (pv1[k] ? dstep : 0u)));
             graw[k][0] = (inb && pv0[k]) ? v0 : 0u;
             graw[k][1] = (inb && pv1[k]) ? v1 : 0u;
         }

@@ -15,7 +15,7 @@ from .._common import cl3d, next_power_of_2, require_cuda
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
 _TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
 _TILE_W = {8: 16, 16: 8, 32: 8, 64: 8, 128: 8}
-_LANE_C = {8: 4, 16: 2, 32: 2, 64: 2, 128: 2}
+_LANE_C = {8: 2, 16: 4, 32: 4, 64: 2, 128: 2}
 
 
 @confexc(KeyError)
