@@ -216,11 +216,24 @@ __device__ __forceinline__ float to_f32(T v)
     return (float)v;
 }
 
-__device__ __forceinline__ uint32_t quant_u8_one(float t, float window, float two_w)
+// Correctly rounded a / b for a divisor that is constant over the launch, in 3 VALU instructions
+// instead of the ~11 of the generic IEEE sequence: with rb = RN(1/b) correctly rounded,
+// q0 = RN(a*rb), e = a - q0*b (exact in one FMA), q = RN(q0 + e*rb) is the correctly rounded
+// quotient (Markstein).  Valid when nothing over/underflows on the way; the callers guarantee the
+// operand ranges (see the launchers) and fall back to the IEEE division otherwise.
+__device__ __forceinline__ float div_by_const(float a, float b, float rb)
+{
+    const float q0 = __fmul_rn(a, rb);
+    const float e = __builtin_fmaf(-q0, b, a);
+    return __builtin_fmaf(e, rb, q0);
+}
+
+template <bool FAST>
+__device__ __forceinline__ uint32_t quant_u8_one(float t, float window, float two_w, float r_two_w)
 {
     t = fminf(fmaxf(t, -window), window);
     t = __fadd_rn(t, window);
-    t = __fdiv_rn(t, two_w);
+    t = FAST ? div_by_const(t, two_w, r_two_w) : __fdiv_rn(t, two_w);
     t = __fmul_rn(t, 255.0f);
     return (uint32_t)t;  // truncation toward zero
 }
@@ -260,9 +273,9 @@ __device__ __forceinline__ u32x4_t pack16(const uint32_t (&b)[16])
     return o;
 }
 
-template <typename T>
+template <typename T, bool FAST>
 __global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
-                                                                  int64_t numel, float window)
+                                                                  int64_t numel, float window, float r_two_w)
 {
     const float two_w = __fmul_rn(2.0f, window);
     const int64_t ngroups = numel / 16;
@@ -273,11 +286,12 @@ __global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __res
         load16<T>(x + i * 16, f);
         uint32_t b[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) b[j] = quant_u8_one(f[j], window, two_w);
+        for (int j = 0; j < 16; ++j) b[j] = quant_u8_one<FAST>(f[j], window, two_w, r_two_w);
         __builtin_nontemporal_store(pack16(b), reinterpret_cast<u32x4_t*>(q + i * 16));
     }
     if (gid == 0) {
-        for (int64_t k = ngroups * 16; k < numel; ++k) q[k] = (uint8_t)quant_u8_one(to_f32(x[k]), window, two_w);
+        for (int64_t k = ngroups * 16; k < numel; ++k)
+            q[k] = (uint8_t)quant_u8_one<FAST>(to_f32(x[k]), window, two_w, r_two_w);
     }
 }
 
@@ -357,9 +371,10 @@ __global__ __launch_bounds__(kStreamThreads) void absmax_final_kernel(const floa
     }
 }
 
-__device__ __forceinline__ uint32_t quant_i8_one(float v, float scale)
+__device__ __forceinline__ uint32_t quant_i8_one(float v, float scale, float rscale)
 {
-    float t = rintf(__fdiv_rn(v, scale));  // round half to even
+    // |v| <= 65504 and scale = absmax/127 >= 2^-31: no overflow; a quotient that underflows rounds to 0
+    float t = rintf(div_by_const(v, scale, rscale));  // round half to even
     t = fminf(fmaxf(t, -127.0f), 127.0f);
     return (uint32_t)((int)t) & 0xffu;
 }
@@ -370,6 +385,7 @@ __global__ __launch_bounds__(kStreamThreads) void quant_i8_kernel(const half_t* 
 {
     const float scale = __fdiv_rn(absmax[0], 127.0f);
     const bool zero = (scale == 0.0f);
+    const float rscale = __fdiv_rn(1.0f, zero ? 1.0f : scale);  // correctly rounded reciprocal, once per thread
     const int64_t ngroups = numel / 16;
     const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
     const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
@@ -378,12 +394,12 @@ __global__ __launch_bounds__(kStreamThreads) void quant_i8_kernel(const half_t* 
         load16<half_t>(y + i * 16, f);
         uint32_t b[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) b[j] = zero ? 0u : quant_i8_one(f[j], scale);
+        for (int j = 0; j < 16; ++j) b[j] = zero ? 0u : quant_i8_one(f[j], scale, rscale);
         __builtin_nontemporal_store(pack16(b), reinterpret_cast<u32x4_t*>(q + i * 16));
     }
     if (gid == 0) {
         for (int64_t k = ngroups * 16; k < numel; ++k)
-            q[k] = zero ? (int8_t)0 : (int8_t)quant_i8_one((float)y[k], scale);
+            q[k] = zero ? (int8_t)0 : (int8_t)quant_i8_one((float)y[k], scale, rscale);
     }
 }
 
@@ -573,16 +589,25 @@ extern "C" int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int
     int rc = check_flat("quant_u8_window", x, q, numel, &blocks);
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
+    // 1/(2w) correctly rounded to fp32: the double quotient rounded once more is exact for division
+    // (53 >= 2*24 + 2 bits).  The 3-instruction division needs 2w and its quotients to stay normal.
+    const float two_w = 2.0f * window;
+    const bool fast = window >= 0x1p-60f && window <= 0x1p60f;
+    const float r_two_w = fast ? (float)(1.0 / (double)two_w) : 0.0f;
+#define KEROPS_QU8_GO(T, F)                                                                                     \
+    hipLaunchKernelGGL((quant_u8_kernel<T, F>), dim3(blocks), dim3(kStreamThreads), 0, s, (const T*)x, (uint8_t*)q, \
+                       numel, window, r_two_w)
     if (dtype == KEROPS_DTYPE_F16) {
-        hipLaunchKernelGGL((quant_u8_kernel<half_t>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x,
-                           (uint8_t*)q, numel, window);
+        if (fast) KEROPS_QU8_GO(half_t, true);
+        else KEROPS_QU8_GO(half_t, false);
     } else if (dtype == KEROPS_DTYPE_F32) {
-        hipLaunchKernelGGL((quant_u8_kernel<float>), dim3(blocks), dim3(kStreamThreads), 0, s, (const float*)x,
-                           (uint8_t*)q, numel, window);
+        if (fast) KEROPS_QU8_GO(float, true);
+        else KEROPS_QU8_GO(float, false);
     } else {
         set_error("quant_u8_window: unknown dtype tag %d", dtype);
         return KEROPS_E_BADARG;
     }
+#undef KEROPS_QU8_GO
     return check_launch("quant_u8_window");
 }
 

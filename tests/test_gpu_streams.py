@@ -160,6 +160,23 @@ def test_quant_u8_window_bit_exact_exhaustive(window):
                            ref.view(torch.int16 if dt == torch.float16 else torch.int32))
 
 
+@pytest.mark.parametrize('window', [0.1, 1.0 / 3.0, 5e-5, 12345.678, 2.0, 0.7071, 1e-30, 1e20, 255.0, 1e-6])
+def test_quant_u8_division_is_ieee_exact(window):
+    """The kernel divides by the launch-constant 2*window with a 3-instruction correctly rounded
+    sequence (IEEE division outside the guarded range): bit-equality with the oracle's fp32
+    division on every finite fp16 value and on 2M random fp32 values spread around the bin edges."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    x16 = bits[torch.isfinite(bits)]
+    assert torch.equal(QuantUint8Window(x16.to(DEV), window).cpu(), oracle.quant_u8_window(x16, window))
+    g = cpu_gen(int(window * 1000) % 1000 + 7)
+    w32 = torch.tensor(window, dtype=torch.float32)
+    u = torch.rand(1000000, generator=g) * 2 - 1
+    edges = (torch.randint(0, 256, (1000000,), generator=g).float() / 255.0 * 2 - 1)
+    jitter = (torch.rand(1000000, generator=g) - 0.5) * 1e-6
+    x32 = torch.cat([u * w32 * 1.1, (edges + jitter) * w32])
+    assert torch.equal(QuantUint8Window(x32.to(DEV), window).cpu(), oracle.quant_u8_window(x32, window))
+
+
 def test_quant_u8_ragged_lengths_and_layouts():
     g = cpu_gen(5)
     for n in (1, 7, 8, 9, 1023, 100003):
@@ -189,7 +206,7 @@ def test_quant_i8_sym_bit_exact():
         assert q.dtype == torch.int8 and torch.equal(q.cpu(), oracle.quant_i8_sym(y, a))
         assert s.item() == torch.tensor(a, dtype=torch.float32).div(127.0).item()
     # exhaustive over fp16 for a few explicit maxima, ties included
-    for amax in (127.0, 1.0, 3.3):
+    for amax in (127.0, 1.0, 3.3, 65504.0, 6e-8, 0.001, 77.77, 1234.5, 2.0 ** -14):
         am = torch.tensor([amax], dtype=torch.float32, device=DEV)
         q, _ = QuantInt8Sym(fin.to(DEV), am)
         assert torch.equal(q.cpu(), oracle.quant_i8_sym(fin, amax))
