@@ -173,7 +173,7 @@ constexpr int kMaxReduceChannels = 512;  // per-channel reductions: C/V <= 64 la
 
 // Default workgroup count of the persistent stream kernels.  Measured on MI355X with 256-thread
 // workgroups at (1,64,350,350,128): 768 (three per CU, 3 wavefronts per SIMD) is fastest for the
-// read-dominated and read+write fp16 streams, 512 for the pooling gather, 1280 for the quantisers.
+// read-dominated and read+write fp16 streams, 512 for the pooling gather (whole multiples of the 256 CUs; 640 or 896 are measurably worse).
 static inline int stream_blocks_default(int64_t work_items, int preferred = 768)
 {
     int64_t b = ceil_div64(work_items, kStreamThreads);

@@ -579,7 +579,7 @@ static int check_flat(const char* op, const void* a, const void* b, int64_t nume
         set_error("%s: null or misaligned pointer, or non-positive numel", op);
         return KEROPS_E_BADARG;
     }
-    if (*blocks <= 0) *blocks = stream_blocks_default(ceil_div64(numel, 16), 1280);
+    if (*blocks <= 0) *blocks = stream_blocks_default(ceil_div64(numel, 16), 768);
     return KEROPS_OK;
 }
 
