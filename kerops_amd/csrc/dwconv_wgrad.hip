@@ -142,29 +142,38 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
             for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
         }
     };
-    // g of one row for every pair: raw dwords (c0,c1) at d and d+1; rows outside the chunk and
-    // positions outside the volume contribute zeros
+    // g of one row for every pair: raw dwords (c0,c1) at d and d+1.  The loads are unconditional and
+    // nothing looks at the values until they are packed one step later (a select right behind the
+    // load would force a wait on every load in flight): rows outside the chunk are replaced by zeros
+    // at packing time, positions outside the volume are masked with a precomputed per-lane AND mask.
+    uint32_t gmask[PP][2];
+#pragma unroll
+    for (int k = 0; k < PP; ++k) {
+        gmask[k][0] = pv0[k] ? 0xffffffffu : 0u;
+        gmask[k][1] = pv1[k] ? 0xffffffffu : 0u;
+    }
     auto load_g = [&](int h, uint32_t(&graw)[PP][2]) {
-        const bool inb = (h >= hs) && (h < he);
-        const char* gplane = reinterpret_cast<const char*>(gn_ptr + (inb ? h : hs) * plane_stride);
+        const int hc_row = min(max(h, hs), he - 1);  // any valid row: the values of other rows are dropped
+        const char* gplane = reinterpret_cast<const char*>(gn_ptr + hc_row * plane_stride);
         const uint32_t dstep = (uint32_t)C * 2u;
 #pragma unroll
         for (int k = 0; k < PP; ++k) {
             // g is read exactly once: streaming hint, it should not displace the x halo rows in L2
-            const uint32_t v0 = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(gplane + poff[k]));
-            const uint32_t v1 =
-                __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(gplane + poff[k] + (pv1[k] ? dstep : 0u)));
-            graw[k][0] = (inb && pv0[k]) ? v0 : 0u;
-            graw[k][1] = (inb && pv1[k]) ? v1 : 0u;
+            graw[k][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(gplane + poff[k]));
+            graw[k][1] = __builtin_nontemporal_load(
+                reinterpret_cast<const uint32_t*>(gplane + poff[k] + (pv1[k] ? dstep : 0u)));
         }
     };
     // packed (g[d][c], g[d+1][c]) per pair and channel for the rows hp-1, hp, hp+1
     half2_t gm[PP][CL], gc[PP][CL], gnx[PP][CL];
-    auto pack_g = [&](half2_t(&dst)[PP][CL], const uint32_t(&graw)[PP][2]) {
+    auto pack_g = [&](half2_t(&dst)[PP][CL], const uint32_t(&graw)[PP][2], int h) {
+        const bool inb = (h >= hs) && (h < he);  // wavefront-uniform
 #pragma unroll
         for (int k = 0; k < PP; ++k) {
-            dst[k][0] = pack_lo(graw[k][0], graw[k][1]);
-            dst[k][1] = pack_hi(graw[k][0], graw[k][1]);
+            const uint32_t a0 = inb ? (graw[k][0] & gmask[k][0]) : 0u;
+            const uint32_t a1 = inb ? (graw[k][1] & gmask[k][1]) : 0u;
+            dst[k][0] = pack_lo(a0, a1);
+            dst[k][1] = pack_hi(a0, a1);
         }
     };
     const half2_t hz = {(half_t)0, (half_t)0};
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
     // a whole plane of arithmetic: ga holds row hp+2 (in flight or landed), gb receives row hp+3
     uint32_t ga[PP][2], gb[PP][2];
     load_g(hs, ga);
-    pack_g(gnx, ga);
+    pack_g(gnx, ga, hs);
     load_g(hs + 1, ga);
 
     int parity = 0;
@@ -225,7 +234,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
                 gm[k][c] = gc[k][c];
                 gc[k][c] = gnx[k][c];
             }
-        pack_g(gnx, ga);
+        pack_g(gnx, ga, hp + 2);
 #pragma unroll
         for (int k = 0; k < PP; ++k) {
             ga[k][0] = gb[k][0];
