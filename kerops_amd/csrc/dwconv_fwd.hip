@@ -23,6 +23,9 @@ template <int CG_, int TW_, int TD_, int CL_, int NT_, int WPE_>
 struct FwdCfg {
     static constexpr int CG = CG_, TW = TW_, TD = TD_, CL = CL_, NT = NT_;
     static constexpr int WPE = WPE_;           // wavefronts per SIMD the register budget is held to
+    // Branch-free march with deferred stores (see dwconv_fwd_body). It needs a few more live registers, so
+    // only the configurations with room under their register budget use it.
+    static constexpr bool STRAIGHT = (WPE_ == 4);
     static constexpr int SC = CG * 8;          // channels in the slab
     static constexpr int NCL = SC / CL;        // lane groups (CL channels each) per voxel
     static constexpr int PW = TW + 2, PD = TD + 2;
@@ -221,63 +224,157 @@ __device__ __forceinline__ void dwconv_fwd_body(const FwdArgs& a, half8_t (&lds)
 #pragma unroll
         for (int c = 0; c < CL; ++c) a0[k][c] = a1[k][c] = a2[k][c] = 0.0f;
 
-    half8_t pre[NLD];
-    auto prefetch = [&](int hp) {
-        if ((hp >= 0) && (hp < H)) {
-            const char* xplane = reinterpret_cast<const char*>(xn + hp * plane_stride);  // wavefront-uniform
-#pragma unroll
-            for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
-        }
-    };
+    if constexpr (Cfg::STRAIGHT) {
+        // The march runs over the planes that exist, hp_lo..hp_hi; planes -1 and H are all zero and are
+        // skipped (a volume border only changes which accumulator holds the last row, see the end).
+        // Inside the loop every step does the same straight-line sequence, with no branch around a memory
+        // operation: the compiler's wait-count bookkeeping is exact only on branch-free paths, and a
+        // conservative wait would stall each step on the stores it has just issued.
+        const int hp_lo = max(hs - 1, 0), hp_hi = min(he, H - 1);
 
-    int parity = 0;
-    auto step = [&](int hp, float(&aF)[P][CL], float(&aM)[P][CL], float(&aS)[P][CL]) {
-        const bool inb = (hp >= 0) && (hp < H);
-        half8_t* buf = lds[parity];
-        parity ^= 1;
-        if (inb) {
-#pragma unroll
-            for (int j = 0; j < NLD; ++j) buf[ldst[j]] = pre[j];
-        }
-        __syncthreads();
-        if (hp + 1 <= he) prefetch(hp + 1);
-        if (inb) {
-            scatter_plane<Cfg, true, true, true>(reinterpret_cast<const half_t*>(buf), lbase, lw, aF, aM, aS);
-        } else {
-#pragma unroll
-            for (int k = 0; k < P; ++k)
-#pragma unroll
-                for (int c = 0; c < CL; ++c) aS[k][c] = 0.0f;
-        }
-        const int ho = hp - 1;
-        if (ho >= hs) {
-            char* yplane = reinterpret_cast<char*>(yn + ho * plane_stride);  // wavefront-uniform
-#pragma unroll
+        half8_t pre[NLD];
+        auto prefetch = [&](int hp) {
+            const char* xplane = reinterpret_cast<const char*>(xn + hp * plane_stride);  // wavefront-uniform
+    #pragma unroll
+            for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
+        };
+
+        // A finished row is rounded to fp16 at the end of its step but stored at the *start* of the next
+        // step's arithmetic, ahead of the next prefetch: the vector-memory counter retires in issue order
+        // and counts stores too, so a store issued right before the wait for the prefetched plane would
+        // expose its full latency on every step.
+        hv_t ostage[P];
+        int pending_row = -1;
+        auto round_row = [&](const float(&acc)[P][CL]) {
+    #pragma unroll
             for (int k = 0; k < P; ++k) {
-                if (OUT_FULL || oval[k]) {
-                    hv_t o;
-#pragma unroll
-                    for (int c = 0; c < CL; ++c) {
-                        float v = aF[k][c];
-                        if (EPI) v = fmaxf(__builtin_fmaf(v, esc[c], esh[c]), 0.0f);
-                        o[c] = (half_t)v;
-                    }
-                    __builtin_nontemporal_store(o, reinterpret_cast<hv_t*>(yplane + ooff[k]));  // written once, never re-read
+    #pragma unroll
+                for (int c = 0; c < CL; ++c) {
+                    float v = acc[k][c];
+                    if (EPI) v = fmaxf(__builtin_fmaf(v, esc[c], esh[c]), 0.0f);
+                    ostage[k][c] = (half_t)v;
                 }
             }
-        }
-    };
+        };
+        auto flush_row = [&]() {
+            if (pending_row >= 0) {
+                char* yplane = reinterpret_cast<char*>(yn + pending_row * plane_stride);  // wavefront-uniform
+    #pragma unroll
+                for (int k = 0; k < P; ++k) {
+                    if (OUT_FULL || oval[k]) {
+                        // written once, never re-read: streaming hint keeps L2 for the halo rows
+                        __builtin_nontemporal_store(ostage[k], reinterpret_cast<hv_t*>(yplane + ooff[k]));
+                    }
+                }
+            }
+        };
 
-    int hp = hs - 1;
-    prefetch(hp);
-    __syncthreads();  // the one-off zero fill of the halo chunks is visible before any plane is read
-    for (;;) {
-        step(hp, a0, a1, a2);
-        if (++hp > he) break;
-        step(hp, a1, a2, a0);
-        if (++hp > he) break;
-        step(hp, a2, a0, a1);
-        if (++hp > he) break;
+        int parity = 0;
+        // aF: row hp-1 (finishing), aM: row hp, aS: row hp+1 (starting from zero)
+        auto step = [&](int hp, float(&aF)[P][CL], float(&aM)[P][CL], float(&aS)[P][CL]) {
+            half8_t* buf = lds[parity];
+            parity ^= 1;
+    #pragma unroll
+            for (int j = 0; j < NLD; ++j) buf[ldst[j]] = pre[j];
+            __syncthreads();
+            flush_row();
+            prefetch(min(hp + 1, hp_hi));  // the last one re-reads the current plane (cache hit) and is dropped
+            // Scheduling fences: the loads stay ahead of the arithmetic that hides their latency, and the
+            // arithmetic of one plane is scheduled on its own (one big region inflates register pressure).
+            __builtin_amdgcn_sched_barrier(0);
+            scatter_plane<Cfg, true, true, true>(reinterpret_cast<const half_t*>(buf), lbase, lw, aF, aM, aS);
+            __builtin_amdgcn_sched_barrier(0);
+            const int ho = hp - 1;
+            pending_row = (ho >= hs) ? ho : -1;
+            round_row(aF);
+        };
+
+        int hp = hp_lo, phase = 0;
+        prefetch(hp);
+        __syncthreads();  // the one-off zero fill of the halo chunks is visible before any plane is read
+        for (;;) {
+            step(hp, a0, a1, a2);
+            phase = 1;
+            if (++hp > hp_hi) break;
+            step(hp, a1, a2, a0);
+            phase = 2;
+            if (++hp > hp_hi) break;
+            step(hp, a2, a0, a1);
+            phase = 0;
+            if (++hp > hp_hi) break;
+        }
+        flush_row();
+        if (he == H) {
+            // bottom border of the volume: plane H does not exist, so row H-1 is complete after plane H-1,
+            // where it was the middle row of the last step
+            pending_row = H - 1;
+            if (phase == 1) round_row(a1);
+            else if (phase == 2) round_row(a2);
+            else round_row(a0);
+            flush_row();
+        }
+    } else {
+        // Branching march: every step tests whether its plane exists. The branches keep the scheduling
+        // regions (and with them the register pressure) small, at the price of conservative memory waits.
+        half8_t pre[NLD];
+        auto prefetch = [&](int hp) {
+            if ((hp >= 0) && (hp < H)) {
+                const char* xplane = reinterpret_cast<const char*>(xn + hp * plane_stride);  // wavefront-uniform
+#pragma unroll
+                for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
+            }
+        };
+
+        int parity = 0;
+        auto step = [&](int hp, float(&aF)[P][CL], float(&aM)[P][CL], float(&aS)[P][CL]) {
+            const bool inb = (hp >= 0) && (hp < H);
+            half8_t* buf = lds[parity];
+            parity ^= 1;
+            if (inb) {
+#pragma unroll
+                for (int j = 0; j < NLD; ++j) buf[ldst[j]] = pre[j];
+            }
+            __syncthreads();
+            if (hp + 1 <= he) prefetch(hp + 1);
+            if (inb) {
+                scatter_plane<Cfg, true, true, true>(reinterpret_cast<const half_t*>(buf), lbase, lw, aF, aM, aS);
+            } else {
+#pragma unroll
+                for (int k = 0; k < P; ++k)
+#pragma unroll
+                    for (int c = 0; c < CL; ++c) aS[k][c] = 0.0f;
+            }
+            const int ho = hp - 1;
+            if (ho >= hs) {
+                char* yplane = reinterpret_cast<char*>(yn + ho * plane_stride);  // wavefront-uniform
+#pragma unroll
+                for (int k = 0; k < P; ++k) {
+                    if (OUT_FULL || oval[k]) {
+                        hv_t o;
+#pragma unroll
+                        for (int c = 0; c < CL; ++c) {
+                            float v = aF[k][c];
+                            if (EPI) v = fmaxf(__builtin_fmaf(v, esc[c], esh[c]), 0.0f);
+                            o[c] = (half_t)v;
+                        }
+                        // written once, never re-read: streaming hint keeps L2 for the halo rows
+                        __builtin_nontemporal_store(o, reinterpret_cast<hv_t*>(yplane + ooff[k]));
+                    }
+                }
+            }
+        };
+
+        int hp = hs - 1;
+        prefetch(hp);
+        __syncthreads();  // the one-off zero fill of the halo chunks is visible before any plane is read
+        for (;;) {
+            step(hp, a0, a1, a2);
+            if (++hp > he) break;
+            step(hp, a1, a2, a0);
+            if (++hp > he) break;
+            step(hp, a2, a0, a1);
+            if (++hp > he) break;
+        }
     }
 }
 
@@ -316,7 +413,7 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
         // enough workgroups to fill 256 CUs several times over, but rows per chunk
         // large enough that the two halo planes of a chunk stay a small overhead
         const int64_t per_plane = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
-        const int want_chunks = (int)std::max<int64_t>(1, ceil_div64(3072, per_plane));
+        const int want_chunks = (int)std::max<int64_t>(1, ceil_div64(2816, per_plane));
         h_chunk = std::max(ceil_div(a.H, want_chunks), std::min(a.H, 24));
     }
     h_chunk = std::min(h_chunk, a.H);

@@ -29,6 +29,7 @@ struct WgCfg {
     static constexpr int PW = TW + 2, PD = TD + 2;
     static constexpr int NPAIR = TW * (TD / 2) * NCL;  // (d, d+1) position pairs per plane
     static constexpr int PP = NPAIR / NT;              // pairs per thread per plane
+    static constexpr bool STRAIGHT = (PP <= 2);        // branch-free march (see the kernel); needs spare registers
     static constexpr int NCH = PW * PD * CG;   // staged c8 chunks per plane
     static constexpr int NLD = (NCH + NT - 1) / NT;
     static constexpr int NWAVE = NT / kWave;
@@ -59,7 +60,7 @@ __device__ __forceinline__ half2_t pack_hi(uint32_t a, uint32_t b)
 }
 
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_kernel(const WgArgs a)
+__global__ __launch_bounds__(Cfg::NT, (Cfg::NT >= 512 || Cfg::STRAIGHT) ? 4 : 3) void dwconv_wgrad_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, PP = Cfg::PP, NLD = Cfg::NLD, NCH = Cfg::NCH;
     constexpr int PD = Cfg::PD, CL = Cfg::CL, NCL = Cfg::NCL, SC = Cfg::SC;
@@ -134,9 +135,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
 #pragma unroll
         for (int c = 0; c < CL; ++c) acc[tap][c] = 0.0f;
 
+    // Straight march: only the x planes that exist are visited (planes -1 and H are all zero and contribute
+    // nothing), so a step has no branch around its memory operations; the compiler's wait-count bookkeeping
+    // is only exact on branch-free paths. It costs about 18 more live registers, so the configurations with
+    // four position pairs per lane keep the branching march, which tests every plane instead.
+    constexpr bool ST = Cfg::STRAIGHT;
+    const int hp_lo = ST ? max(hs - 1, 0) : hs - 1, hp_hi = ST ? min(he, H - 1) : he;
     half8_t pre[NLD];
     auto prefetch_x = [&](int hp) {
-        if ((hp >= 0) && (hp < H)) {
+        if (ST || ((hp >= 0) && (hp < H))) {
             const char* xplane = reinterpret_cast<const char*>(xn + hp * plane_stride);
 #pragma unroll
             for (int j = 0; j < NLD; ++j) pre[j] = *reinterpret_cast<const half8_t*>(xplane + goff[j]);
@@ -176,23 +183,22 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
             dst[k][1] = pack_hi(a0, a1);
         }
     };
-    const half2_t hz = {(half_t)0, (half_t)0};
-#pragma unroll
-    for (int k = 0; k < PP; ++k)
-#pragma unroll
-        for (int c = 0; c < CL; ++c) gm[k][c] = gc[k][c] = hz;
     // g rows are fetched two steps before they are packed, so their latency is hidden behind
     // a whole plane of arithmetic: ga holds row hp+2 (in flight or landed), gb receives row hp+3
     uint32_t ga[PP][2], gb[PP][2];
-    load_g(hs, ga);
-    pack_g(gnx, ga, hs);
-    load_g(hs + 1, ga);
+    load_g(hp_lo - 1, ga);
+    pack_g(gm, ga, hp_lo - 1);
+    load_g(hp_lo, ga);
+    pack_g(gc, ga, hp_lo);
+    load_g(hp_lo + 1, ga);
+    pack_g(gnx, ga, hp_lo + 1);
+    load_g(hp_lo + 2, ga);
 
     int parity = 0;
-    prefetch_x(hs - 1);
+    prefetch_x(hp_lo);
     __syncthreads();  // one-off zero fill of out-of-volume halo chunks
-    for (int hp = hs - 1; hp <= he; ++hp) {
-        const bool inb = (hp >= 0) && (hp < H);
+    for (int hp = hp_lo; hp <= hp_hi; ++hp) {
+        const bool inb = ST || ((hp >= 0) && (hp < H));
         half8_t* buf = stage + parity * (NCH + 1);
         parity ^= 1;
         if (inb) {
@@ -200,8 +206,14 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
             for (int j = 0; j < NLD; ++j) buf[ldst[j]] = pre[j];
         }
         __syncthreads();
-        if (hp + 1 <= he) prefetch_x(hp + 1);
+        if (ST) {
+            prefetch_x(min(hp + 1, hp_hi));  // the last one re-reads the current plane (cache hit) and is dropped
+        } else if (hp + 1 <= he) {
+            prefetch_x(hp + 1);
+        }
         load_g(hp + 3, gb);
+        // scheduling fences: the loads stay ahead of the arithmetic that hides their latency
+        if (ST) __builtin_amdgcn_sched_barrier(0);
         if (inb) {
             const half_t* plane = reinterpret_cast<const half_t*>(buf);
 #pragma unroll
@@ -227,6 +239,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
                 }
             }
         }
+        if (ST) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int k = 0; k < PP; ++k)
 #pragma unroll
@@ -335,7 +348,7 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
         // measured best on MI355X at (1, C, 350, 350, 128)
         switch (p->cg) {
             case 1: tile_w = 8; tile_d = 32; break;
-            case 2: tile_w = 8; tile_d = 32; break;
+            case 2: tile_w = 8; tile_d = 16; break;
             case 4: tile_w = 4; tile_d = 16; break;
             default: tile_w = 4; tile_d = 8; break;
         }

@@ -12,7 +12,7 @@ from ...settings import ConfigurableArg, confexc, configure
 from .._common import next_power_of_2, require_cuda
 
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
-_TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
+_TILE_D = {8: 32, 16: 16, 32: 16, 64: 8, 128: 8}
 _TILE_W = {8: 8, 16: 8, 32: 4, 64: 4, 128: 4}
 
 
