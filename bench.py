@@ -41,8 +41,8 @@ V = H * W * D
 # (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000):
 # profiles/dwconv_fwd_wgrad_c64_readme_shape.md.
 MEASURED_TRAFFIC_BYTES = {
-    ('dwconv_fwd', 64): 4323427939,    # 2.316 GB read + 2.007 GB written (1.077 x algorithmic)
-    ('dwconv_wgrad', 64): 4479787905,  # 4.460 GB read + 0.019 GB written (1.116 x algorithmic)
+    ('dwconv_fwd', 64): 4293346969,    # 2.286 GB read + 2.007 GB written (1.070 x algorithmic)
+    ('dwconv_wgrad', 64): 4567850092,  # 4.548 GB read + 0.019 GB written (1.138 x algorithmic)
 }
 
 
