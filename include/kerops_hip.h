@@ -61,6 +61,9 @@ int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int
  *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]
  * gw is [3][3][3][C] fp32.  Deterministic: per-workgroup partials go to the
  * workspace and a second kernel adds them in a fixed order.
+ * lane_channels selects the kernel family: 16 = matrix-core kernels (one 4x4x4
+ * MFMA block per channel, 16 channels per instruction; the built-in choice),
+ * 2 = vector kernels (two channels per lane, 2-way fp16 dot products).
  * Replaces the zero-filled partial buffer, the `_DWConv_wgrad_cl3d_impl[grid](...)`
  * launches and the trailing `grad_w.sum(dim=(0, 1))`:
  * kerops/ops/conv/dwconv_wgrad.py:54-77 (kernel kerops/kernels/dw_conv.py:147-287). */

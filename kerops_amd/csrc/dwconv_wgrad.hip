@@ -280,6 +280,279 @@ __global__ __launch_bounds__(Cfg::NT, (Cfg::NT >= 512 || Cfg::STRAIGHT) ? 4 : 3)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Matrix-core variant (lane_channels = 16).
+//
+// v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4 blocks, D_b[i][j] += sum_k A_b[i][k] * B_b[k][j];
+// lane 4b+i holds row i of A_b as four fp16 (k = 0..3), lane 4b+j holds column j of B_b, and lane 4b+j
+// receives column j of D_b in four fp32 registers (i = 0..3).  A depthwise weight gradient has no
+// reduction over channels, so a block is one channel and the reduction index k runs over four
+// D-adjacent positions d0..d0+3 of one (h, w) row:
+//
+//   A_b[i][k] = x[hp][w][d0 + k + i - 1][c_b]          (the window of lane i starts i-1 positions in: kd = i)
+//   B_b[k][j] = g[hp + 1 - j][w - kw + 1][d0 + k][c_b]  (lane j takes the g plane that sees x plane hp at kh = j)
+//   D_b[i][j] accumulates gw[kh = j][kw][kd = i][c_b]   (one accumulator tile per kw)
+//
+// Row i = 3 and column j = 3 compute nothing useful and are ignored (9 of 16 outputs, 576 of 1024
+// multiply-adds per instruction are useful); the meaning of a lane's accumulators never changes, so
+// three accumulator tiles are chained through the whole march.  Per g row, four positions and
+// 16 channels the cost is 3 matrix instructions instead of 54 dot + 20 permute vector instructions
+// per 2 positions x 2 channels: the arithmetic drops to a fraction of the memory time.
+//
+// Operands come from LDS as dwords (two channels per lane and position) and are split into the even
+// and the odd channel's operand by two byte permutes each.  The last four g planes stay in LDS (a
+// ring): lane j simply reads its plane's slot, so no operand is kept in registers across steps, and
+// the g operand of a row is gathered once per step and used by the three x rows around it.
+//
+// LDS layout: a position occupies PB = 2*SC bytes; inside it the channel offset is rotated by 32 bytes
+// per position (rot) so that the three distinct positions read by half a wavefront fall into disjoint
+// banks; g slots are 32 bytes apart modulo 128 for the same reason (lanes j read different slots).
+template <int CG_, int TW_, int TD_, int NT_>
+struct WmCfg {
+    static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, NWAVE = NT_ / 64;
+    static constexpr int SC = CG * 8;                      // channels in the slab
+    static constexpr int PB = SC * 2;                      // bytes of one position
+    static constexpr int NQ = SC >= 32 ? 16 : SC / 2;      // channel pairs per matrix instruction
+    static constexpr int NSUB = 16 / NQ;                   // groups of 4 positions per instruction
+    static constexpr int NHALF = SC / (2 * NQ);            // 32-channel halves of the slab
+    static constexpr int NPART = NWAVE / NHALF;            // wavefronts that share a half split the patch
+    static constexpr int GD = TD / (4 * NSUB);             // position groups along D, one per wavefront
+    static constexpr int RSPLIT = NPART / GD;              // ... and row ranges along W
+    static constexpr int RG = TW / RSPLIT;                 // g rows per wavefront (it reads RG + 2 x rows)
+    static constexpr int R = TW + 2;                       // x rows incl. halo
+    static constexpr int PDP = (TD + 2 + 3) / 4 * 4;       // x positions per row incl. halo, padded to 4
+    static constexpr int XSLOT = R * PDP * PB;
+    static constexpr int GSLOT = TW * TD * PB + 32;
+    static constexpr int XOFF = 4 * GSLOT;                 // [4 g slots][2 x slots][dump]
+    static constexpr int DUMP = XOFF + 2 * XSLOT;
+    static constexpr int STAGE_BYTES = DUMP + 16;
+    static constexpr int NXCH = R * (TD + 2) * CG, NGCH = TW * TD * CG;
+    static constexpr int NLDX = (NXCH + NT - 1) / NT, NLDG = (NGCH + NT - 1) / NT;
+    static constexpr int RED_BYTES = NPART * 27 * SC * 4;
+    static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
+    static_assert(TD % (4 * NSUB) == 0, "a row splits into whole position groups");
+    static_assert(NPART % GD == 0 && NPART >= GD, "one position group per wavefront");
+    static_assert(TW % RSPLIT == 0, "rows split evenly");
+    static_assert(STAGE_BYTES % 16 == 0, "16-byte chunks");
+    // byte offset of channel byte cb at position index p (p relative to any multiple of 4)
+    __device__ static constexpr int swz(int p, int cb)
+    {
+        return p * PB + ((cb + (PB >= 64 ? 32 * (p / (128 / PB)) : 0)) & (PB - 1));
+    }
+};
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+// four dwords (two channels at four positions) -> the even and the odd channel's operand
+__device__ __forceinline__ void split_operands(const uint32_t (&r)[4], half4_t& even, half4_t& odd)
+{
+    const uint2_t e = {__builtin_amdgcn_perm(r[1], r[0], 0x05040100u), __builtin_amdgcn_perm(r[3], r[2], 0x05040100u)};
+    const uint2_t o = {__builtin_amdgcn_perm(r[1], r[0], 0x07060302u), __builtin_amdgcn_perm(r[3], r[2], 0x07060302u)};
+    even = __builtin_bit_cast(half4_t, e);
+    odd = __builtin_bit_cast(half4_t, o);
+}
+
+template <class Cfg>
+__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_mfma_kernel(const WgArgs a)
+{
+    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
+    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RG = Cfg::RG, XSLOT = Cfg::XSLOT, GSLOT = Cfg::GSLOT;
+    constexpr int NLDX = Cfg::NLDX, NLDG = Cfg::NLDG;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+
+    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
+    if (L >= a.nblocks) return;
+    const uint32_t ws_slot = L;
+    const int slab = L % a.n_slab;
+    L /= a.n_slab;
+    const int dt = L % a.n_dt;
+    L /= a.n_dt;
+    const int wt_i = L % a.n_wt;
+    L /= a.n_wt;
+    const int hc = L % a.n_hc;
+    const int n = L / a.n_hc;
+
+    const int t = threadIdx.x;
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
+    const int hs = hc * a.h_chunk;
+    const int he = min(hs + a.h_chunk, H);
+    const int cslab = slab * SC;
+    const int64_t plane_stride = (int64_t)W * D * C;
+    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
+    const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
+
+    // everything that staging never writes must read as zero: positions outside the volume and the
+    // g planes before the chunk
+    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int o = t * 16; o < Cfg::STAGE_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
+
+    // staging assignment, 16-byte chunks (8 channels of one position); lanes without a chunk inside the
+    // volume load the plane's first chunk and write it to the dump slot
+    uint32_t xgo[NLDX], ggo[NLDG];
+    int xls[NLDX], gls[NLDG];
+#pragma unroll
+    for (int j = 0; j < NLDX; ++j) {
+        const int ch = t + j * NT;
+        const int wq = ch / ((TD + 2) * CG);
+        const int rem = ch - wq * ((TD + 2) * CG);
+        const int dq = rem / CG, cq = rem - dq * CG;
+        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
+        const bool ok = (ch < Cfg::NXCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+        xgo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        xls[j] = ok ? Cfg::swz(wq * PDP + dq, cq * 16) : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < NLDG; ++j) {
+        const int ch = t + j * NT;
+        const int wq = ch / (TD * CG);
+        const int rem = ch - wq * (TD * CG);
+        const int dq = rem / CG, cq = rem - dq * CG;
+        const int w = w0 + wq, d = d0 + dq;
+        const bool ok = (ch < Cfg::NGCH) && (w < W) && (d < D);
+        ggo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        gls[j] = ok ? Cfg::swz(wq * TD + dq, cq * 16) : -1;
+    }
+
+    // operand gathering: lane = (block b, index rr); block = (channel pair q, position group sub)
+    const int lane = t % kWave, wave = t / kWave;
+    const int half = wave % Cfg::NHALF, part = wave / Cfg::NHALF;
+    const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RG;  // this wavefront: position group, first g row
+    const int b = lane / 4, rr = lane % 4;
+    const int q = b % NQ, sub = b / NQ;
+    const int r2 = min(rr, 2);  // index 3 repeats index 2: its results are never used
+    const int cb = half * 64 + q * 4;
+    const int pgrp = (gd * NSUB + sub) * 4;  // first position of the lane's group inside a row
+    int aoff[4], boff[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        aoff[k] = Cfg::XOFF + Cfg::swz(ra * PDP + pgrp + r2 + k, cb);  // x row ra (patch row ra-1), window r2
+        boff[k] = Cfg::swz(ra * TD + pgrp + k, cb);                     // g row ra; the slot is added per step
+    }
+
+    float4_t acc[3][2];
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
+    // They are unconditional (plane indices are clamped, values of planes that do not exist or lie
+    // outside the chunk are never used): the compiler's wait-count bookkeeping is exact only on
+    // branch-free paths, and a conservative wait would also wait for the newer set.
+    half8_t xpre0[NLDX], xpre1[NLDX], gpre0[NLDG], gpre1[NLDG];
+    auto prefetch = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {  // x plane hp, g plane hp+1
+        const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
+        const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(hp + 1, hs), he - 1) * plane_stride);
+#pragma unroll
+        for (int j = 0; j < NLDX; ++j) xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
+#pragma unroll
+        for (int j = 0; j < NLDG; ++j)
+            gpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(gplane + ggo[j]));
+    };
+
+    int parity = 0;
+    // step hp: x plane hp meets the g planes hp+1 (kh = 0), hp (kh = 1), hp-1 (kh = 2)
+    auto step = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {
+        const bool xin = (hp >= 0) && (hp < H);  // wavefront-uniform
+        const bool gin = hp + 1 < he;
+        unsigned char* xbuf = smem + Cfg::XOFF + parity * XSLOT;
+        unsigned char* gslot = smem + ((hp + 1) & 3) * GSLOT;
+#pragma unroll
+        for (int j = 0; j < NLDX; ++j) {
+            unsigned char* dst = xls[j] >= 0 ? xbuf + xls[j] : smem + Cfg::DUMP;
+            *reinterpret_cast<half8_t*>(dst) = xpre[j];
+        }
+        // g planes past the chunk read as zero; the slot held a plane that is no longer needed
+#pragma unroll
+        for (int j = 0; j < NLDG; ++j) {
+            unsigned char* dst = gls[j] >= 0 ? gslot + gls[j] : smem + Cfg::DUMP;
+            *reinterpret_cast<half8_t*>(dst) = gin ? gpre[j] : z8;
+        }
+        __syncthreads();
+        prefetch(hp + 2, xpre, gpre);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
+        if (xin) {
+            const int xo = parity * XSLOT;
+            const int go = ((hp + 1 - r2) & 3) * GSLOT;  // lane j reads the slot of plane hp+1-j
+            half4_t G[RG][2];
+#pragma unroll
+            for (int xr = 0; xr < RG + 2; ++xr) {
+                if (xr < RG) {  // the g row first needed by this x row
+                    uint32_t r[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        r[k] = *reinterpret_cast<const uint32_t*>(smem + go + boff[k] + xr * TD * PB);
+                    split_operands(r, G[xr][0], G[xr][1]);
+                }
+                uint32_t r[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    r[k] = *reinterpret_cast<const uint32_t*>(smem + xo + aoff[k] + xr * PDP * PB);
+                half4_t A[2];
+                split_operands(r, A[0], A[1]);
+#pragma unroll
+                for (int kw = 0; kw < 3; ++kw) {
+                    // x patch row ra-1+xr meets g row ra+xr-kw at tap kw
+                    if (xr - kw >= 0 && xr - kw < RG) {
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], G[xr - kw][e], acc[kw][e], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        parity ^= 1;
+    };
+
+    prefetch(hs - 1, xpre0, gpre0);
+    prefetch(hs, xpre1, gpre1);
+    __syncthreads();  // the one-off zero fill is complete before staging writes anything
+    for (int hp = hs - 1;;) {
+        step(hp, xpre0, gpre0);
+        if (++hp > he) break;
+        step(hp, xpre1, gpre1);
+        if (++hp > he) break;
+    }
+
+    // ---- combine: position groups inside a wavefront, then the wavefronts of a half via LDS ----
+    if (NSUB > 1) {
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    float v = acc[kw][e][i];
+#pragma unroll
+                    for (int off = 4 * NQ; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
+                    acc[kw][e][i] = v;
+                }
+    }
+    __syncthreads();  // staging buffers are dead from here on
+    float* red = reinterpret_cast<float*>(smem);  // [NPART][27][SC]
+    if (sub == 0 && rr < 3) {
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    red[(part * 27 + (rr * 3 + kw) * 3 + i) * SC + half * 32 + 2 * q + e] = acc[kw][e][i];
+    }
+    __syncthreads();
+    float* out = a.ws + (int64_t)ws_slot * 27 * SC;
+    for (int o = t; o < 27 * SC; o += NT) {
+        float sacc = 0.0f;
+#pragma unroll
+        for (int pt = 0; pt < Cfg::NPART; ++pt) sacc += red[pt * 27 * SC + o];
+        out[o] = sacc;
+    }
+}
+
 // Second pass, two small kernels, fixed summation order (deterministic).  The workspace holds one
 // row per (n, h-chunk, w-patch, d-patch) of width RW = slabs*27*SC floats.  Pass 1 sums the rows of
 // each of kRedSeg row segments (64 columns x 4 interleaved row slices per workgroup, coalesced
@@ -345,14 +618,14 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     }
     p->cg = C >= 64 ? 8 : C / 8;
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
-        // measured best on MI355X at (1, C, 350, 350, 128)
+        // measured best on MI355X at (1, C, 350, 350, 128): the matrix-core kernels
         switch (p->cg) {
             case 1: tile_w = 8; tile_d = 32; break;
             case 2: tile_w = 8; tile_d = 16; break;
             case 4: tile_w = 4; tile_d = 16; break;
-            default: tile_w = 4; tile_d = 8; break;
+            default: tile_w = 8; tile_d = 8; break;
         }
-        lane_channels = 2;
+        lane_channels = 16;
     }
     p->cl = lane_channels;
     p->tile_w = tile_w;
@@ -383,10 +656,9 @@ static int64_t wgrad_ws_bytes(const WgPlan& p)
     return (p.nblocks * 27 * sc + (int64_t)kRedSeg * p.n_slab * 27 * sc) * (int64_t)sizeof(float);
 }
 
-template <int CG, int TW, int TD, int NT>
-static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
+template <class Cfg, class KernelT>
+static int launch_wgrad_cfg(KernelT kernel, const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
 {
-    using Cfg = WgCfg<CG, TW, TD, NT>;
     WgArgs a = base;
     a.n_wt = p.n_wt;
     a.n_dt = p.n_dt;
@@ -394,7 +666,7 @@ static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStrea
     a.n_slab = p.n_slab;
     a.h_chunk = p.h_chunk;
     a.nblocks = (uint32_t)p.nblocks;
-    hipLaunchKernelGGL(dwconv_wgrad_kernel<Cfg>, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
     int rc = check_launch("dwconv_wgrad");
     if (rc != KEROPS_OK) return rc;
     const int n_rows = (int)(p.nblocks / p.n_slab);
@@ -409,6 +681,20 @@ static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStrea
     hipLaunchKernelGGL(wgrad_reduce2_kernel, dim3(ceil_div(RW, 256)), dim3(256), 0, stream, ws2, gw, nseg, RW, Cfg::SC,
                        a.C);
     return check_launch("dwconv_wgrad_reduce2");
+}
+
+template <int CG, int TW, int TD, int NT>
+static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
+{
+    using Cfg = WgCfg<CG, TW, TD, NT>;
+    return launch_wgrad_cfg<Cfg>(dwconv_wgrad_kernel<Cfg>, base, p, gw, stream);
+}
+
+template <int CG, int TW, int TD, int NT>
+static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
+{
+    using Cfg = WmCfg<CG, TW, TD, NT>;
+    return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg>, base, p, gw, stream);
 }
 
 }  // namespace kerops
@@ -466,6 +752,18 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     KEROPS_WG_CASE(8, 4, 16, 256)
     KEROPS_WG_CASE(8, 4, 8, 256)
 #undef KEROPS_WG_CASE
+    // matrix-core kernels: (channel groups of 8, patch W, patch D, threads)
+#define KEROPS_WM_CASE(CGv, TWv, TDv, NTv)                                   \
+    if (p.cg == CGv && p.tile_w == TWv && p.tile_d == TDv && p.cl == 16) \
+        return launch_wgrad_mfma<CGv, TWv, TDv, NTv>(a, p, gw, s);
+    KEROPS_WM_CASE(1, 8, 32, 256)
+    KEROPS_WM_CASE(2, 8, 16, 256)
+    KEROPS_WM_CASE(4, 4, 16, 256)
+    KEROPS_WM_CASE(4, 8, 16, 256)
+    KEROPS_WM_CASE(8, 4, 8, 256)
+    KEROPS_WM_CASE(8, 8, 8, 512)
+    KEROPS_WM_CASE(8, 4, 16, 512)
+#undef KEROPS_WM_CASE
     set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, p.tile_w, p.tile_d,
               p.cl);
     return KEROPS_E_BADARG;

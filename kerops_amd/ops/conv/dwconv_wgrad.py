@@ -11,9 +11,9 @@ from ... import _lib
 from ...settings import ConfigurableArg, confexc, configure
 from .._common import next_power_of_2, require_cuda
 
-_WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
+_WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
 _TILE_D = {8: 32, 16: 16, 32: 16, 64: 8, 128: 8}
-_TILE_W = {8: 8, 16: 8, 32: 4, 64: 4, 128: 4}
+_TILE_W = {8: 8, 16: 8, 32: 4, 64: 8, 128: 8}
 
 
 @confexc(KeyError)
@@ -45,7 +45,7 @@ def ilp(channels):
     ILP=lambda x: ilp(x.shape[1]),
     W_block=lambda x: wtile(x.shape[1]),
     H_chunk=0,
-    lane_channels=2,
+    lane_channels=16,
     out_dtype=torch.float16,
 )
 def DWConvWGRAD(
@@ -72,7 +72,7 @@ def DWConvWGRAD(
     assert channels == next_power_of_2(channels)
     assert D_block == next_power_of_2(D_block)
     {'float32': None, 'float16': None}[ACCTYPE]
-    assert num_warps == 4, 'the gfx950 kernels are built for 4 wavefronts per workgroup'
+    assert num_warps in (4, 8), 'the gfx950 kernels are built for 4 or 8 wavefronts per workgroup'
     require_cuda(x, grad)
 
     bsize, _, H, W, D = x.shape
