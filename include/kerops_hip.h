@@ -51,6 +51,9 @@ const char* kerops_last_error_string(void);
  * accumulation of all 27 taps, one RNE rounding to fp16:
  *   y[n,h,w,d,c] = sum_{kh,kw,kd} x[n,h+kh-1,w+kw-1,d+kd-1,c] * wt[kh,kw,kd,c]
  * wt is [3][3][3][C] fp16.  C in {8,16,32,64,128}.
+ * lane_channels selects the kernel family: 16 = matrix-core kernels (one 4x4x4
+ * MFMA block per channel; the built-in choice), 2 or 4 = vector kernels with that
+ * many channels per lane.
  * Replaces the `_DWConv_cl3d_impl[grid](...)` launch and its per-sample Python
  * loop: kerops/ops/conv/dwconv.py:47-61 (kernel kerops/kernels/dw_conv.py:6-142). */
 int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W, int32_t D,

@@ -24,6 +24,32 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
+// ---- shared by the matrix-core depthwise kernels (v_mfma_f32_4x4x4_16B_f16, one block per channel) ----
+// LDS patches keep one position in PB = 2*channels bytes; inside a position the channel offset is
+// rotated by 32 bytes per position so that the three or four distinct positions read by half a
+// wavefront (8 channel pairs each) fall into disjoint banks.  p may be taken relative to any multiple of 4.
+template <int PB>
+__device__ constexpr int lds_swizzle(int p, int cb)
+{
+    return p * PB + ((cb + (PB >= 64 ? 32 * (p / (128 / PB)) : 0)) & (PB - 1));
+}
+// dwords holding two channels at consecutive positions -> the even and the odd channel's fp16x4 operand
+__device__ __forceinline__ void split_operands(const uint32_t (&r)[4], half4_t& even, half4_t& odd)
+{
+    const u32x2_t e = {__builtin_amdgcn_perm(r[1], r[0], 0x05040100u), __builtin_amdgcn_perm(r[3], r[2], 0x05040100u)};
+    const u32x2_t o = {__builtin_amdgcn_perm(r[1], r[0], 0x07060302u), __builtin_amdgcn_perm(r[3], r[2], 0x07060302u)};
+    even = __builtin_bit_cast(half4_t, e);
+    odd = __builtin_bit_cast(half4_t, o);
+}
+// same with three positions; the fourth operand element is zero (selector byte 0x0c yields 0x00)
+__device__ __forceinline__ void split_operands3(const uint32_t (&r)[3], half4_t& even, half4_t& odd)
+{
+    const u32x2_t e = {__builtin_amdgcn_perm(r[1], r[0], 0x05040100u), __builtin_amdgcn_perm(0u, r[2], 0x0c0c0100u)};
+    const u32x2_t o = {__builtin_amdgcn_perm(r[1], r[0], 0x07060302u), __builtin_amdgcn_perm(0u, r[2], 0x0c0c0302u)};
+    even = __builtin_bit_cast(half4_t, e);
+    odd = __builtin_bit_cast(half4_t, o);
+}
+
 constexpr int kWave = 64;
 
 // ---- error reporting (host) -------------------------------------------------

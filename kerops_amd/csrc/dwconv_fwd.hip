@@ -401,6 +401,269 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const Fwd
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Matrix-core variant (lane_channels = 16).
+//
+// v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4 blocks, D_b[i][j] += sum_k A_b[i][k] * B_b[k][j];
+// lane 4b+i holds row i of A_b as four fp16 (k = 0..3), lane 4b+j holds column j of B_b, and lane 4b+j
+// receives column j of D_b in four fp32 registers (i = 0..3).  A depthwise convolution never mixes
+// channels, so a block is one channel; the staged input plane hp is scattered, as in the vector
+// kernel, into the output planes hp+1, hp, hp-1:
+//
+//   A_b[i][k] = wt[kh = i][kw][kd = k][c_b]            (weights; row 3 and column 3 are zero)
+//   B_b[k][j] = x[hp][w][d0 + j + k - 1][c_b]           (lane j's window starts j-1 positions in)
+//   D_b[i][j] += ... is the contribution of x row w to out[hp + 1 - i][w - kw + 1][d0 + j][c_b]
+//
+// One accumulator tile per output row w' therefore holds, in its registers i = 0, 1, 2, the partial
+// sums of the output planes hp+1, hp, hp-1 for four D positions; the three x rows around w' add into
+// it with the three kw operands.  After the plane, register 2 is complete (plane hp-1) and is stored;
+// then the registers move up by one (a plane step renames 0 -> 1 -> 2, two moves and a zero).
+// 576 of the 1024 multiply-adds of an instruction are useful; per x row, four positions and 16
+// channels the cost is 3 matrix instructions, the operand comes from LDS as three dwords (two
+// channels per lane and position) split into the even and the odd channel by byte permutes.
+// The arithmetic is a fraction of the memory time; global loads run two planes ahead.
+template <int CG_, int TW_, int TD_, int NT_>
+struct FmCfg {
+    static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, NWAVE = NT_ / 64;
+    static constexpr int SC = CG * 8;                      // channels in the slab
+    static constexpr int PB = SC * 2;                      // bytes of one position
+    static constexpr int NQ = SC >= 32 ? 16 : SC / 2;      // channel pairs per matrix instruction
+    static constexpr int NSUB = 16 / NQ;                   // groups of 4 positions per instruction
+    static constexpr int NHALF = SC / (2 * NQ);            // 32-channel halves of the slab
+    static constexpr int NPART = NWAVE / NHALF;            // wavefronts that share a half split the patch
+    static constexpr int GD = TD / (4 * NSUB);             // position groups along D, one per wavefront
+    static constexpr int RSPLIT = NPART / GD;              // ... and row ranges along W
+    static constexpr int RO = TW / RSPLIT;                 // output rows per wavefront (it reads RO + 2 x rows)
+    static constexpr int R = TW + 2;                       // x rows incl. halo
+    static constexpr int PDP = (TD + 3 + 3) / 4 * 4;       // x positions per row: halo + one over-read, padded to 4
+    static constexpr int XSLOT = R * PDP * PB;
+    static constexpr int DUMP = 2 * XSLOT;
+    static constexpr int LDS_BYTES = DUMP + 16;
+    static constexpr int NXCH = R * (TD + 2) * CG;
+    static constexpr int NLDX = (NXCH + NT - 1) / NT;
+    static_assert(TD % (4 * NSUB) == 0, "a row splits into whole position groups");
+    static_assert(NPART % GD == 0 && NPART >= GD, "one position group per wavefront");
+    static_assert(TW % RSPLIT == 0, "rows split evenly");
+};
+
+template <class Cfg, bool EPI>
+__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mfma_kernel(const FwdArgs a)
+{
+    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
+    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, XSLOT = Cfg::XSLOT, NLDX = Cfg::NLDX;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+
+    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
+    if (L >= a.nblocks) return;
+    const int slab = L % a.n_slab;
+    L /= a.n_slab;
+    const int dt = L % a.n_dt;
+    L /= a.n_dt;
+    const int wt_i = L % a.n_wt;
+    L /= a.n_wt;
+    const int hc = L % a.n_hc;
+    const int n = L / a.n_hc;
+
+    const int t = threadIdx.x;
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
+    const int hs = hc * a.h_chunk;
+    const int he = min(hs + a.h_chunk, H);
+    const int cslab = slab * SC;
+    const int64_t plane_stride = (int64_t)W * D * C;
+    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
+    half_t* yn = a.y + (int64_t)n * H * plane_stride;
+
+    // positions that staging never writes (outside the volume, row padding) must read as zero
+    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int o = t * 16; o < Cfg::LDS_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
+
+    // staging assignment, 16-byte chunks (8 channels of one position); lanes without a chunk inside the
+    // volume load the plane's first chunk and write it to the dump slot
+    uint32_t xgo[NLDX];
+    int xls[NLDX];
+#pragma unroll
+    for (int j = 0; j < NLDX; ++j) {
+        const int ch = t + j * NT;
+        const int wq = ch / ((TD + 2) * CG);
+        const int rem = ch - wq * ((TD + 2) * CG);
+        const int dq = rem / CG, cq = rem - dq * CG;
+        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
+        const bool ok = (ch < Cfg::NXCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+        xgo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        xls[j] = ok ? lds_swizzle<PB>(wq * PDP + dq, cq * 16) : -1;
+    }
+
+    // lane = (block b, index rr); block = (channel pair q, position group sub)
+    const int lane = t % kWave, wave = t / kWave;
+    const int half = wave % Cfg::NHALF, part = wave / Cfg::NHALF;
+    const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RO;  // this wavefront: position group, first output row
+    const int b = lane / 4, rr = lane % 4;
+    const int q = b % NQ, sub = b / NQ;
+    const int cb = half * 64 + q * 4;          // byte offset of the lane's channel pair inside a position
+    const int c0 = cslab + half * 32 + 2 * q;  // its first channel
+    const int pgrp = (gd * NSUB + sub) * 4;    // first output position of the lane's group inside the patch row
+
+    // weight operands: lane rr = kh holds (kd = 0, 1, 2, -) of tap row (kh, kw) for the even / odd channel
+    half4_t wA[3][2];
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+            if (rr < 3) {
+#pragma unroll
+                for (int kd = 0; kd < 3; ++kd) v[kd] = a.wt[((rr * 3 + kw) * 3 + kd) * C + c0 + e];
+            }
+            wA[kw][e] = v;
+        }
+    float esc[2] = {1.0f, 1.0f}, esh[2] = {0.0f, 0.0f};
+    if (EPI) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            esc[e] = a.scale[c0 + e];
+            esh[e] = a.shift[c0 + e];
+        }
+    }
+
+    // x operand: lane rr = j reads the positions pgrp + j + k (patch column = position + 1 - 1), k = 0..2
+    int boff[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) boff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
+    // output: the lane's dword (two channels) of position pgrp + rr in the output rows ra .. ra+RO-1
+    const int od = d0 + pgrp + rr;
+    const bool odv = od < D;
+    uint32_t ooff[RO];
+    bool oval[RO];
+#pragma unroll
+    for (int o = 0; o < RO; ++o) {
+        const int w = w0 + ra + o;
+        oval[o] = odv && (w < W);
+        ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
+    }
+
+    float4_t T[RO][2];
+#pragma unroll
+    for (int o = 0; o < RO; ++o)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
+    // They are unconditional (plane indices are clamped; planes that do not exist are never used):
+    // the compiler's wait-count bookkeeping is exact only on branch-free paths.
+    half8_t xpre0[NLDX], xpre1[NLDX];
+    auto prefetch = [&](int hp, half8_t(&xpre)[NLDX]) {
+        const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
+#pragma unroll
+        for (int j = 0; j < NLDX; ++j) xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
+    };
+
+    int parity = 0;
+    auto step = [&](int hp, half8_t(&xpre)[NLDX]) {
+        const bool xin = (hp >= 0) && (hp < H);  // wavefront-uniform
+        unsigned char* xbuf = smem + parity * XSLOT;
+#pragma unroll
+        for (int j = 0; j < NLDX; ++j) {
+            unsigned char* dst = xls[j] >= 0 ? xbuf + xls[j] : smem + Cfg::DUMP;
+            *reinterpret_cast<half8_t*>(dst) = xpre[j];
+        }
+        __syncthreads();
+        prefetch(hp + 2, xpre);
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
+        if (xin) {
+#pragma unroll
+            for (int xr = 0; xr < RO + 2; ++xr) {
+                uint32_t r[3];
+#pragma unroll
+                for (int k = 0; k < 3; ++k)
+                    r[k] = *reinterpret_cast<const uint32_t*>(xbuf + boff[k] + xr * PDP * PB);
+                half4_t B[2];
+                split_operands3(r, B[0], B[1]);
+#pragma unroll
+                for (int kw = 0; kw < 3; ++kw) {
+                    // x patch row ra+xr (w = w0-1+ra+xr) adds to the output row ra+xr-kw at tap column kw
+                    if (xr - kw >= 0 && xr - kw < RO) {
+#pragma unroll
+                        for (int e = 0; e < 2; ++e)
+                            T[xr - kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(wA[kw][e], B[e], T[xr - kw][e], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // register 2 of every tile is the finished output plane hp-1
+        const int ho = hp - 1;
+        if (ho >= hs) {
+            char* yplane = reinterpret_cast<char*>(yn + ho * plane_stride);  // wavefront-uniform
+#pragma unroll
+            for (int o = 0; o < RO; ++o) {
+                half2_t v;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    float f = T[o][e][2];
+                    if (EPI) f = fmaxf(__builtin_fmaf(f, esc[e], esh[e]), 0.0f);
+                    v[e] = (half_t)f;
+                }
+                // written once, never re-read: streaming hint keeps L2 for the halo rows
+                if (oval[o]) __builtin_nontemporal_store(v, reinterpret_cast<half2_t*>(yplane + ooff[o]));
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < RO; ++o)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                T[o][e][2] = T[o][e][1];
+                T[o][e][1] = T[o][e][0];
+                T[o][e][0] = 0.0f;
+            }
+        parity ^= 1;
+    };
+
+    prefetch(hs - 1, xpre0);
+    prefetch(hs, xpre1);
+    __syncthreads();  // the one-off zero fill is complete before staging writes anything
+    for (int hp = hs - 1;;) {
+        step(hp, xpre0);
+        if (++hp > he) break;
+        step(hp, xpre1);
+        if (++hp > he) break;
+    }
+}
+
+template <int CG, int TW, int TD, int NT>
+static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t stream)
+{
+    using Cfg = FmCfg<CG, TW, TD, NT>;
+    FwdArgs a = base;
+    a.n_slab = a.C / (CG * 8);
+    a.n_wt = ceil_div(a.W, TW);
+    a.n_dt = ceil_div(a.D, TD);
+    if (h_chunk <= 0) {
+        // about 2.75 workgroups per resident slot (256 CUs x 2 workgroups of 512 threads, or x 4 of 256):
+        // measured best; fewer leave a long tail, more pay the two halo planes of a chunk more often
+        const int64_t per_plane = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
+        const int64_t target = NT >= 512 ? 1408 : 2816;
+        const int want_chunks = (int)std::max<int64_t>(1, (target + per_plane / 2) / per_plane);
+        h_chunk = std::max(ceil_div(a.H, want_chunks), std::min(a.H, 24));
+    }
+    h_chunk = std::min(h_chunk, a.H);
+    a.h_chunk = h_chunk;
+    a.n_hc = ceil_div(a.H, h_chunk);
+    const int64_t nb = (int64_t)N * a.n_hc * a.n_wt * a.n_dt * a.n_slab;
+    if (nb > 0x7fffff00LL) {
+        set_error("dwconv_fwd: too many workgroups (%lld)", (long long)nb);
+        return KEROPS_E_BADARG;
+    }
+    a.nblocks = (uint32_t)nb;
+    if (a.scale) {
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+                           stream, a);
+    } else {
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, false>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+                           stream, a);
+    }
+    return check_launch("dwconv_fwd");
+}
+
 template <int CG, int TW, int TD, int CL, int WPE, int NT = 256>
 static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t stream)
 {
@@ -479,12 +742,14 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
     const int cg = C >= 64 ? 8 : C / 8;
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
         // measured best on MI355X at (1, C, 350, 350, 128)
+        // (the matrix-core kernels)
         switch (cg) {
-            case 1: tile_w = 16; tile_d = 32; lane_channels = 2; break;
-            case 2: tile_w = 8; tile_d = 32; lane_channels = 4; break;
-            case 4: tile_w = 8; tile_d = 16; lane_channels = 4; break;
-            default: tile_w = 8; tile_d = 8; lane_channels = 2; break;
+            case 1: tile_w = 8; tile_d = 32; break;
+            case 2: tile_w = 8; tile_d = 16; break;
+            case 4: tile_w = 4; tile_d = 16; break;
+            default: tile_w = 8; tile_d = 8; break;
         }
+        lane_channels = 16;
     }
     // (channel groups of 8, patch W, patch D, channels per lane, wavefronts per SIMD, threads)
 #define KEROPS_FWD_CASE(CGv, TWv, TDv, CLv, WPEv, NTv)                             \
@@ -501,6 +766,17 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
     KEROPS_FWD_CASE(8, 4, 16, 2, 3, 256)
     KEROPS_FWD_CASE(8, 8, 8, 2, 4, 512)
 #undef KEROPS_FWD_CASE
+    // matrix-core kernels: (channel groups of 8, patch W, patch D, threads)
+#define KEROPS_FM_CASE(CGv, TWv, TDv, NTv)                                  \
+    if (cg == CGv && tile_w == TWv && tile_d == TDv && lane_channels == 16) \
+        return launch_fwd_mfma<CGv, TWv, TDv, NTv>(a, N, h_chunk, s);
+    KEROPS_FM_CASE(1, 8, 32, 256)
+    KEROPS_FM_CASE(2, 8, 16, 256)
+    KEROPS_FM_CASE(4, 4, 16, 256)
+    KEROPS_FM_CASE(8, 4, 8, 256)
+    KEROPS_FM_CASE(8, 8, 8, 512)
+    KEROPS_FM_CASE(8, 4, 16, 512)
+#undef KEROPS_FM_CASE
     set_error("dwconv_fwd: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, tile_w, tile_d,
               lane_channels);
     return KEROPS_E_BADARG;

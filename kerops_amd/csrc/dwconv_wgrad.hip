@@ -334,25 +334,8 @@ struct WmCfg {
     static_assert(NPART % GD == 0 && NPART >= GD, "one position group per wavefront");
     static_assert(TW % RSPLIT == 0, "rows split evenly");
     static_assert(STAGE_BYTES % 16 == 0, "16-byte chunks");
-    // byte offset of channel byte cb at position index p (p relative to any multiple of 4)
-    __device__ static constexpr int swz(int p, int cb)
-    {
-        return p * PB + ((cb + (PB >= 64 ? 32 * (p / (128 / PB)) : 0)) & (PB - 1));
-    }
+    __device__ static constexpr int swz(int p, int cb) { return lds_swizzle<PB>(p, cb); }
 };
-
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef float float4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
-
-// four dwords (two channels at four positions) -> the even and the odd channel's operand
-__device__ __forceinline__ void split_operands(const uint32_t (&r)[4], half4_t& even, half4_t& odd)
-{
-    const uint2_t e = {__builtin_amdgcn_perm(r[1], r[0], 0x05040100u), __builtin_amdgcn_perm(r[3], r[2], 0x05040100u)};
-    const uint2_t o = {__builtin_amdgcn_perm(r[1], r[0], 0x07060302u), __builtin_amdgcn_perm(r[3], r[2], 0x07060302u)};
-    even = __builtin_bit_cast(half4_t, e);
-    odd = __builtin_bit_cast(half4_t, o);
-}
 
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_mfma_kernel(const WgArgs a)

@@ -48,7 +48,7 @@ extern "C" int kerops_dwsep_block_f16(const void* x, const void* wt, const float
     const int64_t V = (int64_t)N * H * W * D;
     half_t* t = (half_t*)workspace;
     float* amax_ws = (float*)((char*)workspace + align256(V * Cin * 2));
-    int rc = dwconv_fwd_run(x, wt, t, scale, shift, N, H, W, D, Cin, 8, 8, 0, 2, stream);
+    int rc = dwconv_fwd_run(x, wt, t, scale, shift, N, H, W, D, Cin, 8, 8, 0, 16, stream);
     if (rc != KEROPS_OK) return rc;
     const int blocks = pointwise_blocks(V);
     rc = pointwise_dispatch(t, (const half_t*)Wm, nullptr, (half_t*)y, amax_ws, V, Cin, Cout, false, true, blocks,

@@ -13,9 +13,10 @@ from .._common import cl3d, next_power_of_2, require_cuda
 # (kerops/ops/conv/dwconv.py:10-17): (wavefronts per workgroup, tile extent along D,
 # tile extent along W).  A missing key means "no kernel for this channel count".
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
-_TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
-_TILE_W = {8: 16, 16: 8, 32: 8, 64: 8, 128: 8}
-_LANE_C = {8: 2, 16: 4, 32: 4, 64: 2, 128: 2}
+_TILE_D = {8: 32, 16: 16, 32: 16, 64: 8, 128: 8}
+_TILE_W = {8: 8, 16: 8, 32: 4, 64: 8, 128: 8}
+# 16 = matrix-core kernels (16 channel blocks per MFMA); 2 / 4 = vector kernels (channels per lane)
+_LANE_C = {8: 16, 16: 16, 32: 16, 64: 16, 128: 16}
 
 
 @confexc(KeyError)
@@ -64,8 +65,8 @@ def DWConv(
     64-wide wavefronts per workgroup (fixed per patch shape in the library: 4, or 8 for the
     8x8 patch) and D_block the tile
     extent along D.  W_block (tile extent along W) and H_chunk (rows one workgroup
-    marches over, 0 = automatic) and lane_channels (channels one lane owns: 2, 4 or 8)
-    are additional gfx950 knobs.
+    marches over, 0 = automatic) and lane_channels (16 = matrix-core kernels, the default;
+    2 or 4 = vector kernels with that many channels per lane) are additional gfx950 knobs.
     """
     channels = x.shape[1]
 
