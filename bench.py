@@ -41,8 +41,8 @@ V = H * W * D
 # (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000):
 # profiles/dwconv_fwd_wgrad_c64_readme_shape.md.
 MEASURED_TRAFFIC_BYTES = {
-    ('dwconv_fwd', 64): 4293346969,    # 2.286 GB read + 2.007 GB written (1.070 x algorithmic)
-    ('dwconv_wgrad', 64): 4567850092,  # 4.548 GB read + 0.019 GB written (1.138 x algorithmic)
+    ('dwconv_fwd', 64): 4450765775,    # 2.241 GB read + 2.209 GB written (1.109 x algorithmic)
+    ('dwconv_wgrad', 64): 4413166485,  # 4.399 GB read + 0.015 GB written (1.099 x algorithmic)
 }
 
 
@@ -199,7 +199,7 @@ def main():
     dom_name, dom_avg = ('dwconv_wgrad', wg_avg) if wg_avg >= fwd_avg else ('dwconv_fwd', fwd_avg)
     achieved = nbytes / dom_avg / 1e6
     roofline = {
-        'kernel': 'kerops::dwconv_wgrad_kernel' if dom_name == 'dwconv_wgrad' else 'kerops::dwconv_fwd_kernel',
+        'kernel': 'kerops::' + dom_name + '_mfma_kernel',
         'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
         'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': MEASURED_TRAFFIC_BYTES.get((dom_name, C)),
         'algorithmic_bytes': nbytes, 'avg_launch_ms': round(dom_avg, 4),
@@ -209,7 +209,7 @@ def main():
     other = 'dwconv_fwd' if dom_name == 'dwconv_wgrad' else 'dwconv_wgrad'
     other_avg = fwd_avg if other == 'dwconv_fwd' else wg_avg
     roofline_other = {
-        'kernel': 'kerops::' + other + '_kernel', 'bound': 'hbm', 'achieved': round(nbytes / other_avg / 1e6, 1),
+        'kernel': 'kerops::' + other + '_mfma_kernel', 'bound': 'hbm', 'achieved': round(nbytes / other_avg / 1e6, 1),
         'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(nbytes / other_avg / 1e6 / HBM_PEAK_GBPS, 4),
         'traffic': MEASURED_TRAFFIC_BYTES.get((other, C)), 'algorithmic_bytes': nbytes,
         'avg_launch_ms': round(other_avg, 4),
