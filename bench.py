@@ -265,8 +265,8 @@ def main():
         y5, am5 = DWSepBlock(x5, wk5, sc5, sh5, Wm5)
         ops['config5_int8_pass'] = figures(time_op(torch, lambda: QuantInt8Sym(y5, am5), it, wm)[0], 3 * V5 * 128,
                                            c5_gbps)
-        ops['config5_note'] = ('stage 1 = DWConv with fused BN+ReLU epilogue, then the MFMA 1x1x1 GEMM with fused '
-                               'max|y|; the fp16 intermediate (268 MB) passes through a workspace')
+        ops['config5_note'] = ('stage 1 = one kernel: matrix-core DWConv, BN+ReLU, fp16 tile through LDS into the MFMA '
+                               '1x1x1 GEMM with fused max|y|; the 64-channel intermediate never reaches memory')
         ops['readme_table_note'] = 'C=8 (251 MB) fits the 256 MB Infinity Cache: its rows are not pure HBM numbers'
 
     cpu, cpu_torch = (None, None)

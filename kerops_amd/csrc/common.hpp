@@ -60,6 +60,11 @@ int check_launch(const char* what);
 int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, const float* shift, int32_t N,
                    int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
                    int32_t lane_channels, void* stream);
+// fused depthwise -> affine -> ReLU -> pointwise kernel (64 input channels, Cout in {64,128}); workgroup count of
+// its grid (= floats of amax_ws it writes)
+int dwsep_fused_blocks(int32_t N, int32_t H, int32_t W, int32_t D);
+int dwsep_fused_run(const void* x, const void* wt, const float* scale, const float* shift, const void* pw, void* y2,
+                    float* amax_ws, int32_t N, int32_t H, int32_t W, int32_t D, int32_t Cout, void* stream);
 int pointwise_dispatch(const _Float16* x, const _Float16* Wm, const _Float16* add, _Float16* out, float* amax_ws,
                        int64_t V, int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s);
 int pointwise_blocks(int64_t V);

@@ -50,6 +50,10 @@ struct FwdArgs {
     half_t* y;
     const float* scale;  // optional fused epilogue y = max(acc * scale[c] + shift[c], 0)
     const float* shift;
+    // optional fused pointwise stage (matrix-core kernel only): y2 = fp16(t @ pw), t = the epilogue's fp16 output
+    const half_t* pw;   // [C][cout]
+    half_t* y2;         // [N][H][W][D][cout]
+    float* amax_ws;     // one max|y2| per workgroup
     int H, W, D, C;
     int n_wt, n_dt, n_hc, n_slab, h_chunk;
     uint32_t nblocks;
@@ -446,15 +450,29 @@ struct FmCfg {
     static_assert(TW % RSPLIT == 0, "rows split evenly");
 };
 
-template <class Cfg, bool EPI>
+// MODE 0: y = conv; 1: y = max(conv * scale + shift, 0); 2: that result (fp16) goes through an LDS tile into the
+// pointwise GEMM [TW*TD positions][C] x [C][COUT] on the 32x32x16 matrix instruction (the product is computed
+// transposed as in pointwise_kernel, a wavefront owns 32 positions x 32 output channels; pw^T sits in LDS), the
+// [positions][COUT] result is bounced through LDS and stored as 16-byte chunks with the running max|y| fused in.
+template <class Cfg, int MODE, int COUT = 0>
 __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mfma_kernel(const FwdArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, XSLOT = Cfg::XSLOT, NLDX = Cfg::NLDX;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+    constexpr bool EPI = MODE >= 1;
+    // fused pointwise stage: t tile [NPOS][SC + 8] fp16 and y tile [NPOS][COUT + 4] fp16 behind the staging buffers
+    constexpr int NPOS = Cfg::TW * TD, RT = SC + 8, RY = COUT + 4;
+    constexpr int KS = SC / 16, MT = COUT / 32, NPT = NPOS / 32;  // k = 16 per matrix instruction
+    constexpr int T_OFF = Cfg::LDS_BYTES, Y_OFF = T_OFF + NPOS * RT * 2, A_OFF = Y_OFF + NPOS * RY * 2;
+    constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : Cfg::LDS_BYTES;
+    static_assert(MODE != 2 || (SC == 64 && NPOS % 32 == 0 && COUT % 32 == 0 && MT * NPT <= Cfg::NWAVE),
+                  "fused pointwise stage: 64 input channels, one (32 positions x 32 outputs) tile per wavefront");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+    __shared__ float amax_red[Cfg::NWAVE];
 
     uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
     if (L >= a.nblocks) return;
+    const uint32_t wg_slot = L;
     const int slab = L % a.n_slab;
     L /= a.n_slab;
     const int dt = L % a.n_dt;
@@ -526,6 +544,22 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
         }
     }
 
+    // fused pointwise stage: this wavefront's 32 positions (pt) x 32 output channels (mt); A fragments =
+    // rows of pw^T, k ordered as the 16-byte chunks the B fragments are read in (see pointwise_kernel)
+    const int vl = lane % 32, hl = lane / 32;
+    const int pt = wave % (NPT > 0 ? NPT : 1), mt = wave / (NPT > 0 ? NPT : 1);
+    float amax = 0.0f;
+    if constexpr (MODE == 2) {
+        // pw^T fragments, pre-arranged so that lane l of block mt reads 16 contiguous bytes per k step:
+        // [mt][s][l][8] = pw[16 s + 8 (l / 32) + 0..7][32 mt + l % 32]
+        half_t* pa = reinterpret_cast<half_t*>(smem + A_OFF);
+        for (int i = t; i < MT * KS * 64 * 8; i += NT) {
+            const int jj = i % 8, l = (i / 8) % 64, s2 = (i / 512) % KS, m2 = i / (512 * KS);
+            pa[i] = a.pw[(16 * s2 + 8 * (l / 32) + jj) * COUT + 32 * m2 + l % 32];
+        }
+    }
+    half_t* yn2 = MODE == 2 ? a.y2 + (int64_t)n * H * W * D * COUT : nullptr;
+
     // x operand: lane rr = j reads the positions pgrp + j + k (patch column = position + 1 - 1), k = 0..2
     int boff[3];
 #pragma unroll
@@ -551,6 +585,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
     // They are unconditional (plane indices are clamped; planes that do not exist are never used):
     // the compiler's wait-count bookkeeping is exact only on branch-free paths.
+    // (the fused pointwise mode has no registers to spare for the second set and runs one plane ahead)
+    constexpr int AHEAD = MODE == 2 ? 1 : 2;
     half8_t xpre0[NLDX], xpre1[NLDX];
     auto prefetch = [&](int hp, half8_t(&xpre)[NLDX]) {
         const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
@@ -568,7 +604,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
             *reinterpret_cast<half8_t*>(dst) = xpre[j];
         }
         __syncthreads();
-        prefetch(hp + 2, xpre);
+        prefetch(hp + AHEAD, xpre);
         __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
         if (xin) {
 #pragma unroll
@@ -592,8 +628,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
         }
         // register 2 of every tile is the finished output plane hp-1
         const int ho = hp - 1;
-        if (ho >= hs) {
-            char* yplane = reinterpret_cast<char*>(yn + ho * plane_stride);  // wavefront-uniform
+        if (ho >= hs) {  // workgroup-uniform
+            char* yplane = MODE == 2 ? nullptr : reinterpret_cast<char*>(yn + ho * plane_stride);
+            half_t* tt = reinterpret_cast<half_t*>(smem + T_OFF);
 #pragma unroll
             for (int o = 0; o < RO; ++o) {
                 half2_t v;
@@ -603,8 +640,53 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
                     if (EPI) f = fmaxf(__builtin_fmaf(f, esc[e], esh[e]), 0.0f);
                     v[e] = (half_t)f;
                 }
-                // written once, never re-read: streaming hint keeps L2 for the halo rows
-                if (oval[o]) __builtin_nontemporal_store(v, reinterpret_cast<half2_t*>(yplane + ooff[o]));
+                if constexpr (MODE == 2) {
+                    *reinterpret_cast<half2_t*>(tt + ((ra + o) * TD + pgrp + rr) * RT + half * 32 + 2 * q) = v;
+                } else {
+                    // written once, never re-read: streaming hint keeps L2 for the halo rows
+                    if (oval[o]) __builtin_nontemporal_store(v, reinterpret_cast<half2_t*>(yplane + ooff[o]));
+                }
+            }
+            if constexpr (MODE == 2) {
+                typedef float float16_t __attribute__((ext_vector_type(16)));
+                half_t* yt = reinterpret_cast<half_t*>(smem + Y_OFF);
+                __syncthreads();
+                if (mt < MT) {
+                    const half_t* trow = tt + (32 * pt + vl) * RT;
+                    const half8_t* pa = reinterpret_cast<const half8_t*>(smem + A_OFF) + mt * KS * 64 + lane;
+                    float16_t pacc;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) pacc[i] = 0.0f;
+#pragma unroll
+                    for (int s2 = 0; s2 < KS; ++s2) {
+                        // B fragment: channels 16 s + 8 hl + 0..7 of the lane's position = one 16-byte chunk
+                        const half8_t bfrag = *reinterpret_cast<const half8_t*>(trow + 16 * s2 + 8 * hl);
+                        pacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(pa[s2 * 64], bfrag, pacc, 0, 0, 0);
+                    }
+                    // pacc[i]: output channel 32*mt + 8*(i/4) + 4*hl + i%4 of position 32*pt + vl
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        half4_t o4;
+#pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) o4[jj] = (half_t)pacc[4 * gq + jj];
+                        *reinterpret_cast<half4_t*>(yt + (32 * pt + vl) * RY + 32 * mt + 8 * gq + 4 * hl) = o4;
+                    }
+                }
+                __syncthreads();
+                half_t* y2plane = yn2 + (int64_t)ho * W * D * COUT;
+#pragma unroll
+                for (int c = t; c < NPOS * (COUT / 8); c += NT) {
+                    const int row = c / (COUT / 8), cc = c - row * (COUT / 8);
+                    const int w = w0 + row / TD, d = d0 + row % TD;
+                    if (w < W && d < D) {
+                        const half4_t lo = *reinterpret_cast<const half4_t*>(yt + row * RY + cc * 8);
+                        const half4_t hi = *reinterpret_cast<const half4_t*>(yt + row * RY + cc * 8 + 4);
+                        const half8_t o8 = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+                        for (int jj = 0; jj < 8; ++jj) amax = fmaxf(amax, fabsf((float)o8[jj]));
+                        store_c8_nt(y2plane + ((int64_t)w * D + d) * COUT + cc * 8, o8);
+                    }
+                }
             }
         }
 #pragma unroll
@@ -619,21 +701,33 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     };
 
     prefetch(hs - 1, xpre0);
-    prefetch(hs, xpre1);
+    if (AHEAD == 2) prefetch(hs, xpre1);
     __syncthreads();  // the one-off zero fill is complete before staging writes anything
     for (int hp = hs - 1;;) {
         step(hp, xpre0);
         if (++hp > he) break;
-        step(hp, xpre1);
-        if (++hp > he) break;
+        if (AHEAD == 2) {
+            step(hp, xpre1);
+            if (++hp > he) break;
+        }
+    }
+    if constexpr (MODE == 2) {
+        amax = wave_max(amax);
+        if (lane == 0) amax_red[wave] = amax;
+        __syncthreads();
+        if (t == 0) {
+            float m = amax_red[0];
+#pragma unroll
+            for (int wv = 1; wv < Cfg::NWAVE; ++wv) m = fmaxf(m, amax_red[wv]);
+            a.amax_ws[wg_slot] = m;
+        }
     }
 }
 
+// grid of the matrix-core kernels: fills the n_* fields and nblocks of `a`
 template <int CG, int TW, int TD, int NT>
-static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t stream)
+static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk)
 {
-    using Cfg = FmCfg<CG, TW, TD, NT>;
-    FwdArgs a = base;
     a.n_slab = a.C / (CG * 8);
     a.n_wt = ceil_div(a.W, TW);
     a.n_dt = ceil_div(a.D, TD);
@@ -644,6 +738,7 @@ static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t 
         const int64_t target = NT >= 512 ? 1408 : 2816;
         const int want_chunks = (int)std::max<int64_t>(1, (target + per_plane / 2) / per_plane);
         h_chunk = std::max(ceil_div(a.H, want_chunks), std::min(a.H, 24));
+        h_chunk = ceil_div(a.H, ceil_div(a.H, h_chunk));  // equal chunks, no short last one
     }
     h_chunk = std::min(h_chunk, a.H);
     a.h_chunk = h_chunk;
@@ -654,12 +749,22 @@ static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t 
         return KEROPS_E_BADARG;
     }
     a.nblocks = (uint32_t)nb;
+    return KEROPS_OK;
+}
+
+template <int CG, int TW, int TD, int NT>
+static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t stream)
+{
+    using Cfg = FmCfg<CG, TW, TD, NT>;
+    FwdArgs a = base;
+    int rc = plan_fwd_mfma<CG, TW, TD, NT>(a, N, h_chunk);
+    if (rc != KEROPS_OK) return rc;
     if (a.scale) {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
-                           stream, a);
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 1>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
+                           a);
     } else {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, false>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
-                           stream, a);
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
+                           a);
     }
     return check_launch("dwconv_fwd");
 }
@@ -780,6 +885,50 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
     set_error("dwconv_fwd: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, tile_w, tile_d,
               lane_channels);
     return KEROPS_E_BADARG;
+}
+}  // namespace kerops
+
+namespace kerops {
+// Fused depthwise -> affine -> ReLU -> pointwise block for 64 input channels (8x8 patch, 512 threads).
+int dwsep_fused_blocks(int32_t N, int32_t H, int32_t W, int32_t D)
+{
+    FwdArgs a{};
+    a.H = H;
+    a.W = W;
+    a.D = D;
+    a.C = 64;
+    if (plan_fwd_mfma<8, 8, 8, 512>(a, N, 0) != KEROPS_OK) return -1;
+    return (int)a.nblocks;
+}
+
+int dwsep_fused_run(const void* x, const void* wt, const float* scale, const float* shift, const void* pw, void* y2,
+                    float* amax_ws, int32_t N, int32_t H, int32_t W, int32_t D, int32_t Cout, void* stream)
+{
+    using Cfg = FmCfg<8, 8, 8, 512>;
+    FwdArgs a{};
+    a.x = (const half_t*)x;
+    a.wt = (const half_t*)wt;
+    a.scale = scale;
+    a.shift = shift;
+    a.pw = (const half_t*)pw;
+    a.y2 = (half_t*)y2;
+    a.amax_ws = amax_ws;
+    a.H = H;
+    a.W = W;
+    a.D = D;
+    a.C = 64;
+    int rc = plan_fwd_mfma<8, 8, 8, 512>(a, N, 0);
+    if (rc != KEROPS_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (Cout == 128) {
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 2, 128>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+    } else if (Cout == 64) {
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 2, 64>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+    } else {
+        set_error("dwsep_block: the fused kernel is built for Cout in {64,128}");
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    return check_launch("dwsep_block");
 }
 }  // namespace kerops
 

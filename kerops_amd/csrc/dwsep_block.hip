@@ -4,9 +4,11 @@
 //   t = fp16(max(dwconv(x, wt) * scale[c] + shift[c], 0))   (fp32 accumulate, one rounding)
 //   y = fp16(t @ Wm)                                          (fp32 accumulate, one rounding)
 //
-// Built from the two kernels of this library: the forward depthwise kernel with the affine+ReLU
-// epilogue fused into its store, and the pointwise MFMA kernel with the running max fused into
-// its write-back.  The intermediate t goes through the caller's workspace.
+// Cout in {64, 128}: one kernel.  The matrix-core depthwise kernel hands every finished output plane of
+// its 8x8 patch (64 positions x 64 channels, rounded to fp16) through an LDS tile to the pointwise GEMM
+// on the 32x32x8 matrix instruction; t never reaches memory and the workspace only holds one max|y|
+// per workgroup.  Other Cout: two kernels (depthwise with the affine+ReLU epilogue, then the
+// pointwise kernel with the running max), t goes through the caller's workspace.
 #include "common.hpp"
 
 using namespace kerops;
@@ -23,6 +25,11 @@ extern "C" int64_t kerops_dwsep_block_workspace_bytes(int32_t N, int32_t H, int3
     if (Cin != 64 || !(Cout == 16 || Cout == 32 || Cout == 64 || Cout == 128)) {
         set_error("dwsep_block: built for Cin = 64 and Cout in {16,32,64,128} (got %d -> %d)", Cin, Cout);
         return KEROPS_E_UNSUPPORTED_C;
+    }
+    if (Cout >= 64) {
+        const int nb = dwsep_fused_blocks(N, H, W, D);
+        if (nb < 0) return KEROPS_E_BADARG;
+        return align256((int64_t)nb * 4);
     }
     const int64_t V = (int64_t)N * H * W * D;
     return align256(V * Cin * 2) + align256((int64_t)pointwise_blocks(V) * 4);
@@ -44,6 +51,13 @@ extern "C" int kerops_dwsep_block_f16(const void* x, const void* wt, const float
         set_error("dwsep_block: workspace of %lld bytes required, %lld given", (long long)need,
                   (long long)workspace_bytes);
         return KEROPS_E_WORKSPACE;
+    }
+    if (Cout >= 64) {
+        float* amax_part = (float*)workspace;
+        int rc = dwsep_fused_run(x, wt, scale, shift, Wm, y, amax_part, N, H, W, D, Cout, stream);
+        if (rc != KEROPS_OK) return rc;
+        launch_pw_absmax_final(amax_part, dwsep_fused_blocks(N, H, W, D), absmax, (hipStream_t)stream);
+        return check_launch("dwsep_block");
     }
     const int64_t V = (int64_t)N * H * W * D;
     half_t* t = (half_t*)workspace;
