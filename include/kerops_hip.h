@@ -176,6 +176,17 @@ int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t
 int kerops_pointwise_f16(const void* x, const void* Wm, const void* add, void* out, int64_t V, int32_t Cin,
                          int32_t Cout, int32_t relu_in, void* stream);
 
+/* Backward of the ReLU-linear op, one pass over x and grad on MFMA:
+ *   dx[v, ci] = x[v, ci] > 0 ? fp16(sum_co g[v, co] * Wm[ci, co]) : 0
+ *   dW[ci, co] = sum_v relu(x[v, ci]) * g[v, co]         (fp32, deterministic)
+ * x/dx dense [V][Cin] fp16, g dense [V][Cout] fp16, Wm [Cin][Cout] fp16, dW [Cin][Cout] fp32.
+ * Cin, Cout in {16,32,64,128}.  Replaces the zero-filled partial buffer, the
+ * `_ReLULinearAddBackward[(grid,)](...)` launch and the trailing `weight_grad.sum(dim=0)`:
+ * kerops/ops/linear/relu_linear_backward.py:52-70 (kernel kerops/kernels/linear.py:48-98). */
+int64_t kerops_relu_linear_bwd_workspace_bytes(int64_t V, int32_t Cin, int32_t Cout);
+int kerops_relu_linear_bwd_f16(const void* x, const void* g, const void* Wm, void* dx, float* dW, void* workspace,
+                               int64_t workspace_bytes, int64_t V, int32_t Cin, int32_t Cout, void* stream);
+
 /* Fused depthwise-separable block (no single reference counterpart; composition
  * of DWConv, a folded inference BN, ReLU and the pointwise GEMM above):
  *   t = fp16(relu(dwconv(x, wt) * scale[c] + shift[c]));  y = fp16(t @ Wm)

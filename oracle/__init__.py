@@ -228,6 +228,18 @@ def pointwise(x, weight, add=None, relu_in=False):
     return _from_cl(out)
 
 
+def relu_linear_bwd(x, grad, weight):
+    """x (N,Cin,H,W,D), grad (N,Cout,H,W,D) fp16 cl3d, weight [Cin,Cout] fp16 -> (dx fp16 like x, dW fp64 [Cin,Cout])."""
+    n, cin, h, w, d = x.shape
+    cout = weight.shape[1]
+    xc, gc = _cl(x), _cl(grad)
+    dx = torch.empty_like(xc)
+    dw = torch.empty(cin, cout, dtype=torch.float64)
+    lib().oracle_relu_linear_bwd(_p(xc), _p(gc), _p(weight.contiguous()), _p(dx), _p(dw), _i64(n * h * w * d),
+                                 _i32(cin), _i32(cout))
+    return _from_cl(dx), dw
+
+
 def dwsep_block(x, dw_weight, scale, shift, pw_weight, return_mid=False):
     n, cin, h, w, d = x.shape
     cout = pw_weight.shape[1]

@@ -551,6 +551,37 @@ void oracle_pointwise(const uint16_t *x, const uint16_t *Wm, const uint16_t *add
     }
 }
 
+/* Backward of the ReLU-linear op: kerops/kernels/linear.py:48-98 (dot products with fp32 accumulate;
+ * input_grad rounded to fp16 then masked by input > 0 at :92; weight_grad accumulated over voxels at
+ * :89-91).  fp64 accumulate here; dW is returned in fp64.
+ *   dx[v,ci] = x[v,ci] > 0 ? fp16(sum_co g[v,co] * Wm[ci,co]) : 0
+ *   dW[ci,co] = sum_v relu(x[v,ci]) * g[v,co]
+ */
+void oracle_relu_linear_bwd(const uint16_t *x, const uint16_t *g, const uint16_t *Wm, uint16_t *dx, double *dW,
+                            int64_t V, int Cin, int Cout)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t v = 0; v < V; ++v) {
+        for (int ci = 0; ci < Cin; ++ci) {
+            double s = 0.0;
+            for (int co = 0; co < Cout; ++co)
+                s += (double)h2f(g[v * Cout + co]) * (double)h2f(Wm[(int64_t)ci * Cout + co]);
+            dx[v * Cin + ci] = h2f(x[v * Cin + ci]) > 0.0f ? f2h((float)s) : (uint16_t)0;
+        }
+    }
+#pragma omp parallel for schedule(static)
+    for (int ci = 0; ci < Cin; ++ci) {
+        for (int co = 0; co < Cout; ++co) {
+            double s = 0.0;
+            for (int64_t v = 0; v < V; ++v) {
+                const float xv = h2f(x[v * Cin + ci]);
+                if (xv > 0.0f) s += (double)xv * (double)h2f(g[v * Cout + co]);
+            }
+            dW[(int64_t)ci * Cout + co] = s;
+        }
+    }
+}
+
 /* Fused depthwise-separable block of config 5 (composition of the pieces above;
  * no single reference counterpart): t = fp16(relu(dwconv(x) * scale[c] +
  * shift[c])) with the depthwise sum and the affine step in fp32; y = fp16(t @ Wm).

@@ -9,8 +9,8 @@ from torch.nn import functional as F
 import oracle
 from conftest import cpu_gen, rand_cl3d, rand_dw_weight
 from kerops_amd.ops.fused import DWSepBlock, DWSepBlockInt8, PointwiseLinear
-from kerops_amd.ops.linear import ReLULinearAdd
-from kerops_amd.utils import allclose_two_stage
+from kerops_amd.ops.linear import ReLULinearAdd, ReLULinearBackward
+from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda'
@@ -41,6 +41,53 @@ def test_relu_linear_add_matches_oracle(cin, cout, spatial):
     # the reference's own ground truth: 1x1x1 conv3d of relu(x) plus the residual
     conv = F.conv3d(F.relu(x.float()), Wm.float().t().reshape(cout, cin, 1, 1, 1)).half() + add
     assert torch.allclose(out.float(), conv.float(), rtol=1e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize('cin,cout', [(16, 16), (16, 32), (32, 16), (32, 32), (32, 64), (64, 64), (64, 128),
+                                      (128, 128), (128, 32), (16, 128), (128, 16), (64, 16)])
+@pytest.mark.parametrize('spatial', [(1, 3, 5, 7), (2, 4, 4, 4), (1, 1, 1, 1), (3, 5, 13, 37)])
+def test_relu_linear_backward_matches_oracle(cin, cout, spatial):
+    g = cpu_gen(cin * 1000 + cout + 1)
+    n, h, w, d = spatial
+    x = rand_cl3d(g, n, cin, h, w, d)
+    grad = rand_cl3d(g, n, cout, h, w, d)
+    Wm = rand_pw(g, cin, cout)
+    dx, dw = ReLULinearBackward(x.to(DEV), grad.to(DEV), Wm.to(DEV), out_dtype=torch.float32)
+    dx, dw = dx.cpu(), dw.cpu()
+    ref_dx, ref_dw = oracle.relu_linear_bwd(x, grad, Wm)
+    assert dx.shape == x.shape and dx.stride() == x.stride() and dw.shape == (cin, cout)
+    # the mask is exact; the values are fp32 MFMA sums vs the oracle's fp64, one rounding to fp16 each
+    assert torch.equal(dx == 0, ref_dx == 0) or ((dx == 0) != (ref_dx == 0)).float().mean() < 1e-3
+    assert torch.equal(dx[x <= 0], torch.zeros_like(dx[x <= 0]))
+    assert (dx.float() - ref_dx.float()).abs().max() <= 2.0 ** -9 * max(1.0, ref_dx.abs().max().item())
+    same = (dx.contiguous().view(torch.int16) == ref_dx.contiguous().view(torch.int16)).float().mean().item()
+    assert same > 0.99, same
+    rel = ((dw.double() - ref_dw).norm() / max(ref_dw.norm().item(), 1e-30)).item()
+    assert rel < 2e-6, rel
+    # the reference's own criteria (tests/ops/test_linear.py:60-78)
+    assert allclose_two_stage(ref_dx.contiguous(), dx.contiguous(), rtol_strict=1e-4, atol_strict=1e-4,
+                              rtol_narrow=1e-3, atol_narrow=1e-3)
+    if ref_dw.norm() > 0:
+        assert weight_grad_similarity(ref_dw.float(), dw, rtol_cos=1e-4, atol_cos=1e-4, rtol_len=1e-3, atol_len=1e-3)
+
+
+def test_relu_linear_backward_default_dtype_determinism_and_large():
+    g = cpu_gen(77)
+    x = rand_cl3d(g, 2, 32, 37, 53, 16)   # V = 62 752: many tiles per workgroup, ragged last tile
+    grad = rand_cl3d(g, 2, 16, 37, 53, 16)
+    Wm = rand_pw(g, 32, 16)
+    xd, gd, wd = x.to(DEV), grad.to(DEV), Wm.to(DEV)
+    dx1, dw1 = ReLULinearBackward(xd, gd, wd)
+    dx2, dw2 = ReLULinearBackward(xd, gd, wd)
+    assert dw1.dtype == torch.float16 and dx1.dtype == torch.float16
+    assert torch.equal(dx1, dx2) and torch.equal(dw1, dw2)  # no atomics: bit-reproducible
+    ref_dx, ref_dw = oracle.relu_linear_bwd(x, grad, Wm)
+    same = (dx1.cpu().contiguous().view(torch.int16) == ref_dx.contiguous().view(torch.int16)).float().mean().item()
+    assert same > 0.99, same
+    _, dw32 = ReLULinearBackward(xd, gd, wd, out_dtype=torch.float32)
+    assert ((dw32.cpu().double() - ref_dw).norm() / ref_dw.norm()).item() < 2e-6
+    with pytest.raises(AssertionError):
+        ReLULinearBackward(xd, gd, wd.t().contiguous())
 
 
 def test_pointwise_identity_and_no_relu():

@@ -377,3 +377,30 @@ def test_pointwise_and_block_vs_torch():
     assert (mid.float() - t.float()).abs().max() <= 2.0 ** -10 * max(1.0, t.abs().max().item())
     ref_y = oracle.pointwise(mid, Wm)
     assert torch.equal(y, ref_y)
+
+
+def test_relu_linear_bwd_vs_torch_autograd():
+    """Pinned by autograd of the 1x1x1 conv3d of relu(x) in fp64 (the ground truth of the reference's
+    own test, tests/ops/test_linear.py:40-78) and by closed forms."""
+    g = cpu_gen(23)
+    n, cin, cout, h, w, d = 2, 16, 32, 3, 5, 4
+    x = rand_cl3d(g, n, cin, h, w, d)
+    grad = rand_cl3d(g, n, cout, h, w, d)
+    Wm = (torch.randn(cin, cout, generator=g) / math.sqrt(cin)).half()
+    dx, dw = oracle.relu_linear_bwd(x, grad, Wm)
+    xd = x.double().requires_grad_(True)
+    wd = Wm.double().requires_grad_(True)
+    out = F.conv3d(F.relu(xd), wd.t().reshape(cout, cin, 1, 1, 1))
+    out.backward(grad.double())
+    assert torch.equal(dx, xd.grad.half())
+    assert dx.stride() == x.stride()
+    assert torch.allclose(dw, wd.grad, rtol=1e-12, atol=1e-12)
+    # closed forms: identity weight passes grad through the mask; an all-negative x has no gradient at all
+    eye = torch.eye(cin, dtype=torch.float16)
+    grad_c = rand_cl3d(g, n, cin, h, w, d)
+    dx, dw = oracle.relu_linear_bwd(x, grad_c, eye)
+    assert torch.equal(dx, torch.where(x > 0, grad_c, torch.zeros_like(grad_c)))
+    ref_dw = torch.einsum('nihwd,nohwd->io', F.relu(x.double()), grad_c.double())
+    assert torch.allclose(dw, ref_dw, rtol=1e-12, atol=1e-12)
+    dx, dw = oracle.relu_linear_bwd(-x.abs(), grad, Wm)
+    assert dx.abs().max() == 0 and dw.abs().max() == 0
