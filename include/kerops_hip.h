@@ -187,6 +187,14 @@ int64_t kerops_relu_linear_bwd_workspace_bytes(int64_t V, int32_t Cin, int32_t C
 int kerops_relu_linear_bwd_f16(const void* x, const void* g, const void* Wm, void* dx, float* dW, void* workspace,
                                int64_t workspace_bytes, int64_t V, int32_t Cin, int32_t Cout, void* stream);
 
+/* Inverted-bottleneck pointwise block on MFMA, the hidden activation stays in registers:
+ *   hid = relu(fp16(x @ Wup) + bias);  out = fp16(hid @ Wdown) + add       (fp16 adds)
+ * x/add/out dense [V][C] fp16, Wup [C][2C], Wdown [2C][C], bias [2C] fp16.  C in {16,32,64}.
+ * Replaces `_LinBReLULinAdd[(grid,)](...)`: kerops/ops/linear/linear_bias_relu_linear_add.py:58-71
+ * (kernel kerops/kernels/linear.py:102-146). */
+int kerops_lin_brelu_lin_add_f16(const void* x, const void* Wup, const void* Wdown, const void* bias, const void* add,
+                                 void* out, int64_t V, int32_t C, void* stream);
+
 /* Fused depthwise-separable block (no single reference counterpart; composition
  * of DWConv, a folded inference BN, ReLU and the pointwise GEMM above):
  *   t = fp16(relu(dwconv(x, wt) * scale[c] + shift[c]));  y = fp16(t @ Wm)

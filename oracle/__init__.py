@@ -240,6 +240,19 @@ def relu_linear_bwd(x, grad, weight):
     return _from_cl(dx), dw
 
 
+def lin_brelu_lin_add(x, weight_up, weight_down, bias, add, return_hidden=False):
+    """x, add (N,C,H,W,D) fp16 cl3d; weight_up [C,2C], weight_down [2C,C], bias [2C] fp16 -> (N,C,H,W,D) fp16."""
+    n, c, h, w, d = x.shape
+    xc, ac = _cl(x), _cl(add)
+    out = torch.empty_like(xc)
+    hid = torch.empty(n, h, w, d, 2 * c, dtype=torch.float16)
+    lib().oracle_lin_brelu_lin_add(_p(xc), _p(weight_up.contiguous()), _p(weight_down.contiguous()),
+                                   _p(bias.contiguous()), _p(ac), _p(hid), _p(out), _i64(n * h * w * d), _i32(c))
+    if return_hidden:
+        return _from_cl(out), _from_cl(hid)
+    return _from_cl(out)
+
+
 def dwsep_block(x, dw_weight, scale, shift, pw_weight, return_mid=False):
     n, cin, h, w, d = x.shape
     cout = pw_weight.shape[1]

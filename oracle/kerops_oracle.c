@@ -582,6 +582,34 @@ void oracle_relu_linear_bwd(const uint16_t *x, const uint16_t *g, const uint16_t
     }
 }
 
+/* Inverted-bottleneck pointwise block: kerops/kernels/linear.py:102-146.
+ *   hid = relu(fp16(x @ Wup) + bias)   (dot with wide accumulate, cast to fp16, fp16 add at :139, ReLU :140)
+ *   out = fp16(hid @ Wdown) + add      (:141)
+ * fp64 accumulate here; hid16 (optional) receives the hidden activation [V][2C].
+ */
+void oracle_lin_brelu_lin_add(const uint16_t *x, const uint16_t *Wup, const uint16_t *Wdown, const uint16_t *bias,
+                              const uint16_t *add, uint16_t *hid16, uint16_t *out, int64_t V, int C)
+{
+    const int HID = 2 * C;
+#pragma omp parallel for schedule(static)
+    for (int64_t v = 0; v < V; ++v) {
+        float hid[256];
+        for (int hcn = 0; hcn < HID; ++hcn) {
+            double s = 0.0;
+            for (int ci = 0; ci < C; ++ci) s += (double)h2f(x[v * C + ci]) * (double)h2f(Wup[(int64_t)ci * HID + hcn]);
+            float hv = h2f(f2h(h2f(f2h((float)s)) + h2f(bias[hcn])));
+            if (!(hv > 0.0f)) hv = 0.0f;
+            hid[hcn] = hv;
+            if (hid16) hid16[v * HID + hcn] = f2h(hv);
+        }
+        for (int co = 0; co < C; ++co) {
+            double s = 0.0;
+            for (int hcn = 0; hcn < HID; ++hcn) s += (double)hid[hcn] * (double)h2f(Wdown[(int64_t)hcn * C + co]);
+            out[v * C + co] = f2h(h2f(f2h((float)s)) + h2f(add[v * C + co]));
+        }
+    }
+}
+
 /* Fused depthwise-separable block of config 5 (composition of the pieces above;
  * no single reference counterpart): t = fp16(relu(dwconv(x) * scale[c] +
  * shift[c])) with the depthwise sum and the affine step in fp32; y = fp16(t @ Wm).

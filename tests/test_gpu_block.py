@@ -9,7 +9,7 @@ from torch.nn import functional as F
 import oracle
 from conftest import cpu_gen, rand_cl3d, rand_dw_weight
 from kerops_amd.ops.fused import DWSepBlock, DWSepBlockInt8, PointwiseLinear
-from kerops_amd.ops.linear import ReLULinearAdd, ReLULinearBackward
+from kerops_amd.ops.linear import LinBReLULinAdd, ReLULinearAdd, ReLULinearBackward
 from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
 
 pytestmark = pytest.mark.gpu
@@ -88,6 +88,49 @@ def test_relu_linear_backward_default_dtype_determinism_and_large():
     assert ((dw32.cpu().double() - ref_dw).norm() / ref_dw.norm()).item() < 2e-6
     with pytest.raises(AssertionError):
         ReLULinearBackward(xd, gd, wd.t().contiguous())
+
+
+@pytest.mark.parametrize('c', [16, 32, 64])
+@pytest.mark.parametrize('spatial', [(1, 3, 5, 7), (2, 4, 4, 4), (1, 1, 1, 1), (3, 5, 13, 37), (1, 37, 53, 16)])
+def test_lin_brelu_lin_add_matches_oracle(c, spatial):
+    g = cpu_gen(c * 77 + spatial[1])
+    n, h, w, d = spatial
+    x, add = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    Wup, Wdown = rand_pw(g, c, 2 * c), rand_pw(g, 2 * c, c)
+    bias = (torch.randn(2 * c, generator=g) * 0.5).half()
+    out = LinBReLULinAdd(x.to(DEV), Wup.to(DEV), Wdown.to(DEV), bias.to(DEV), add.to(DEV)).cpu()
+    ref = oracle.lin_brelu_lin_add(x, Wup, Wdown, bias, add)
+    assert out.shape == x.shape and out.stride() == x.stride()
+    # fp32 MFMA sums vs the oracle's fp64: a hidden value may round differently once in a while
+    assert allclose_two_stage(ref.contiguous(), out.contiguous(), rtol_strict=1e-4, atol_strict=5e-4,
+                              rtol_narrow=1e-3, atol_narrow=2e-3)
+    assert (out.float() - ref.float()).abs().max() <= 2.0 ** -8 * max(1.0, ref.abs().max().item())
+    same = (out.contiguous().view(torch.int16) == ref.contiguous().view(torch.int16)).float().mean().item()
+    assert same > 0.98, same
+    # the reference's own ground truth (tests/ops/test_linear.py:101-116)
+    base = F.conv3d(x.float(), Wup.float().t().reshape(2 * c, c, 1, 1, 1), bias.float())
+    base = F.conv3d(F.relu(base), Wdown.float().t().reshape(c, 2 * c, 1, 1, 1)) + add.float()
+    assert allclose_two_stage(base.half().contiguous(), out.contiguous(), rtol_strict=1e-4, atol_strict=5e-4,
+                              rtol_narrow=1e-3, atol_narrow=2e-3) or torch.allclose(out.float(), base, rtol=2e-3,
+                                                                                    atol=4e-3)
+
+
+def test_lin_brelu_lin_add_closed_form_and_contract():
+    g = cpu_gen(31)
+    c = 32
+    x, add = rand_cl3d(g, 1, c, 5, 6, 7), rand_cl3d(g, 1, c, 5, 6, 7)
+    eye_up = torch.cat([torch.eye(c), torch.zeros(c, c)], 1).half()
+    eye_dn = torch.cat([torch.eye(c), torch.zeros(c, c)], 0).half()
+    zero_b = torch.zeros(2 * c, dtype=torch.float16)
+    out = LinBReLULinAdd(x.to(DEV), eye_up.to(DEV), eye_dn.to(DEV), zero_b.to(DEV), add.to(DEV)).cpu()
+    assert torch.equal(out, (F.relu(x).float() + add.float()).half())  # one nonzero product per sum: exact
+    with pytest.raises(AssertionError):
+        LinBReLULinAdd(x.to(DEV), eye_dn.to(DEV), eye_up.to(DEV), zero_b.to(DEV), add.to(DEV))
+    from kerops_amd.settings import CongiguratorError
+    x128 = rand_cl3d(g, 1, 128, 2, 2, 2)
+    with pytest.raises(CongiguratorError):
+        LinBReLULinAdd(x128.to(DEV), rand_pw(g, 128, 256).to(DEV), rand_pw(g, 256, 128).to(DEV),
+                       torch.zeros(256, dtype=torch.float16, device=DEV), x128.to(DEV))
 
 
 def test_pointwise_identity_and_no_relu():

@@ -404,3 +404,25 @@ def test_relu_linear_bwd_vs_torch_autograd():
     assert torch.allclose(dw, ref_dw, rtol=1e-12, atol=1e-12)
     dx, dw = oracle.relu_linear_bwd(-x.abs(), grad, Wm)
     assert dx.abs().max() == 0 and dw.abs().max() == 0
+
+
+def test_lin_brelu_lin_add_vs_torch():
+    """Pinned by the two 1x1x1 conv3d calls of the reference's own test (tests/ops/test_linear.py:101-106),
+    with the fp16 roundings of the kernel (kerops/kernels/linear.py:139-141) made explicit."""
+    g = cpu_gen(29)
+    n, c, h, w, d = 2, 16, 3, 5, 4
+    x, add = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    Wup = (torch.randn(c, 2 * c, generator=g) / math.sqrt(c)).half()
+    Wdown = (torch.randn(2 * c, c, generator=g) / math.sqrt(2 * c)).half()
+    bias = (torch.randn(2 * c, generator=g) * 0.5).half()
+    out, hid = oracle.lin_brelu_lin_add(x, Wup, Wdown, bias, add, return_hidden=True)
+    up = F.conv3d(x.double(), Wup.double().t().reshape(2 * c, c, 1, 1, 1)).half()
+    hid_ref = F.relu((up.float() + bias.float().view(1, -1, 1, 1, 1)).half())
+    assert torch.equal(hid, hid_ref)
+    down = F.conv3d(hid_ref.double(), Wdown.double().t().reshape(c, 2 * c, 1, 1, 1)).half()
+    assert torch.equal(out, (down.float() + add.float()).half())
+    # closed form: Wup = [I 0], bias = 0, Wdown = [I; 0]  ->  out = relu(x) + add
+    eye_up = torch.cat([torch.eye(c), torch.zeros(c, c)], 1).half()
+    eye_dn = torch.cat([torch.eye(c), torch.zeros(c, c)], 0).half()
+    out = oracle.lin_brelu_lin_add(x, eye_up, eye_dn, torch.zeros(2 * c, dtype=torch.float16), add)
+    assert torch.equal(out, (F.relu(x).float() + add.float()).half())
