@@ -195,6 +195,18 @@ int kerops_relu_linear_bwd_f16(const void* x, const void* g, const void* Wm, voi
 int kerops_lin_brelu_lin_add_f16(const void* x, const void* Wup, const void* Wdown, const void* bias, const void* add,
                                  void* out, int64_t V, int32_t C, void* stream);
 
+/* Backward of the inverted-bottleneck block, one pass over x and grad on MFMA:
+ *   linup = fp16(x @ Wup) + bias;  lg = linup > 0 ? fp16(g @ Wdown^T) : 0
+ *   dx = fp16(lg @ Wup^T);  dWup = x^T lg;  dWdown = relu(linup)^T g;  dbias = sum_v lg   (fp32, deterministic)
+ * x/g/dx dense [V][C] fp16; dWup [C][2C], dWdown [2C][C], dbias [2C] fp32.  C in {16,32,64}.
+ * Replaces the zero-filled partial buffers, the `_LinBReLULinBackward[(grid,)](...)` launch and the three
+ * trailing `.sum(dim=0)`: kerops/ops/linear/linear_bias_relu_linear_backward.py:48-71
+ * (kernel kerops/kernels/linear.py:149-230). */
+int64_t kerops_lin_brelu_lin_bwd_workspace_bytes(int64_t V, int32_t C);
+int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const void* Wup, const void* Wdown, const void* bias,
+                                 void* dx, float* dWup, float* dWdown, float* dbias, void* workspace,
+                                 int64_t workspace_bytes, int64_t V, int32_t C, void* stream);
+
 /* Fused depthwise-separable block (no single reference counterpart; composition
  * of DWConv, a folded inference BN, ReLU and the pointwise GEMM above):
  *   t = fp16(relu(dwconv(x, wt) * scale[c] + shift[c]));  y = fp16(t @ Wm)

@@ -50,6 +50,8 @@ SIGNATURES = {
     'kerops_quant_i8_sym_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p]),
     'kerops_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p]),
     'kerops_lin_brelu_lin_add_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _p]),
+    'kerops_lin_brelu_lin_bwd_workspace_bytes': (_i64, [_i64, _i32]),
+    'kerops_lin_brelu_lin_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _p]),
     'kerops_relu_linear_bwd_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'kerops_relu_linear_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p]),
     'kerops_dwsep_block_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),

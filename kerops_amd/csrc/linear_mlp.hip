@@ -192,3 +192,373 @@ extern "C" int kerops_lin_brelu_lin_add_f16(const void* x, const void* Wup, cons
     set_error("lin_brelu_lin_add: built for C in {16,32,64} (got %d)", C);
     return KEROPS_E_UNSUPPORTED_C;
 }
+
+// =============================================================================================
+// Backward of the block above, one pass over x and grad:
+//
+//   linup = fp16(x @ Wup) + bias (fp16 add);  hid = relu(linup)
+//   dWdown[h, c] = sum_v hid[v, h] * g[v, c]
+//   lg[v, h]     = linup[v, h] > 0 ? fp16(sum_c Wdown[h, c] * g[v, c]) : 0
+//   dWup[c, h]   = sum_v x[v, c] * lg[v, h];   dbias[h] = sum_v lg[v, h]
+//   dx[v, c]     = fp16(sum_h Wup[c, h] * lg[v, h])
+//
+// A workgroup of four wavefronts loops over tiles of 64 voxels; x and g tiles are staged through LDS.
+// Phase A: per (32 voxels, 32 hidden channels) block a wavefront computes linup^T and (Wdown g^T) with the
+// same output layout, applies bias / ReLU / mask in registers and writes the hid and lg tiles to LDS.
+// Phase B: dx^T = Wup lg^T from the lg tile (bounced through LDS for 16-byte stores), and the three
+// reductions over voxels: the 32x32 blocks of dWdown = hid^T g and dWup = x^T lg take their fragments
+// (8 consecutive voxels of one channel) from the LDS tiles with 2-byte reads and stay in fp32 registers
+// for all tiles of the workgroup; dbias is a per-thread column sum of the lg tile.  Partials go to the
+// workspace, a second kernel adds them in a fixed order (fp64): deterministic, no atomics.
+namespace kerops {
+
+constexpr int kMbTile = 64;
+
+template <int C>
+struct MbCfg {
+    static constexpr int H = 2 * C;
+    static constexpr int MH = H / 32, MO = (C + 31) / 32;  // 32-channel blocks of hidden / in-out channels
+    static constexpr int KC = C / 16, KH = H / 16;         // k steps over C / over H
+    static constexpr int KV = kMbTile / 16;                // k steps over the voxels of a tile
+    static constexpr int XP = C + 8, HP = H + 8, DP = C + 4;  // LDS row pitches in halves
+    static constexpr int NBA = 2 * MH;                     // phase A blocks (vt, mh)
+    static constexpr int NB6 = 2 * MO;                     // dx blocks (vt, mo)
+    static constexpr int NU = 2 * MH * MO;                 // reduction blocks: (type, mh, mc)
+    static constexpr int KSPL = NU >= kMlpWaves ? 1 : kMlpWaves / NU;
+    static constexpr int UPW = NU >= kMlpWaves ? NU / kMlpWaves : 1;
+    static constexpr int NXC = kMbTile * C / 8;            // 16-byte chunks of an x / g / dx tile
+    static constexpr int NLX = (NXC + kMlpThreads - 1) / kMlpThreads;
+    static constexpr int BPARTS = kMlpThreads / H;         // threads per hidden channel in the bias sum
+    static constexpr int RW = 2 * C * H + H;               // floats of one partial: dWup, dWdown, dbias
+    static constexpr int XS_OFF = 0;
+    static constexpr int GS_OFF = XS_OFF + kMbTile * XP * 2;
+    static constexpr int HS_OFF = GS_OFF + kMbTile * XP * 2;
+    static constexpr int LS_OFF = HS_OFF + kMbTile * HP * 2;
+    static constexpr int DS_OFF = LS_OFF + kMbTile * HP * 2;
+    static constexpr int A1_OFF = (DS_OFF + kMbTile * DP * 2 + 15) / 16 * 16;
+    static constexpr int A3_OFF = A1_OFF + MH * KC * 64 * 16;
+    static constexpr int A6_OFF = A3_OFF + MH * KC * 64 * 16;
+    static constexpr int BS_OFF = A6_OFF + MO * KH * 64 * 16;
+    static constexpr int BH_OFF = BS_OFF + kMlpThreads * 4;  // fp16 copy of the bias
+    static constexpr int LDS_BYTES = BH_OFF + H * 2;
+    static_assert(C == 16 || C == 32 || C == 64, "C in {16,32,64}");
+    static_assert(KV % KSPL == 0 && kMbTile % BPARTS == 0, "even splits");
+};
+
+template <int C>
+__global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_bwd_kernel(const half_t* __restrict__ x,
+                                                                        const half_t* __restrict__ g,
+                                                                        const half_t* __restrict__ Wup,
+                                                                        const half_t* __restrict__ Wdown,
+                                                                        const half_t* __restrict__ bias,
+                                                                        half_t* __restrict__ dx, float* __restrict__ ws,
+                                                                        int64_t V)
+{
+    using Cfg = MbCfg<C>;
+    constexpr int H = Cfg::H, MH = Cfg::MH, MO = Cfg::MO, KC = Cfg::KC, KH = Cfg::KH, KV = Cfg::KV;
+    constexpr int XP = Cfg::XP, HP = Cfg::HP, DP = Cfg::DP, NLX = Cfg::NLX, KSPL = Cfg::KSPL, UPW = Cfg::UPW;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+    half_t* xs = reinterpret_cast<half_t*>(smem + Cfg::XS_OFF);
+    half_t* gs = reinterpret_cast<half_t*>(smem + Cfg::GS_OFF);
+    half_t* hs = reinterpret_cast<half_t*>(smem + Cfg::HS_OFF);
+    half_t* ls = reinterpret_cast<half_t*>(smem + Cfg::LS_OFF);
+    half_t* ds = reinterpret_cast<half_t*>(smem + Cfg::DS_OFF);
+    half_t* a1 = reinterpret_cast<half_t*>(smem + Cfg::A1_OFF);
+    half8_t* a3 = reinterpret_cast<half8_t*>(smem + Cfg::A3_OFF);
+    half8_t* a6 = reinterpret_cast<half8_t*>(smem + Cfg::A6_OFF);
+    float* bred = reinterpret_cast<float*>(smem + Cfg::BS_OFF);
+    half_t* bsh = reinterpret_cast<half_t*>(smem + Cfg::BH_OFF);
+
+    const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
+    const int il = lane % 32, hl = lane / 32;
+    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // fragments of the three per-voxel products (lane l: row l%32 of the block, k = 16 s + 8 (l/32) + 0..7)
+    // a1: linup^T = Wup^T x^T     -> Wup[k][32 mh + l%32]
+    for (int i = t; i < MH * KC * 64 * 8; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, s = (i / 512) % KC, mh = i / (512 * KC);
+        a1[i] = Wup[(16 * s + 8 * (l / 32) + j) * H + 32 * mh + l % 32];
+    }
+    // a3: (Wdown g^T)             -> Wdown[32 mh + l%32][k .. k+7]
+    for (int i = t; i < MH * KC * 64; i += kMlpThreads) {
+        const int l = i % 64, s = (i / 64) % KC, mh = i / (64 * KC);
+        a3[i] = load_c8(Wdown + (32 * mh + l % 32) * C + 16 * s + 8 * (l / 32));
+    }
+    // a6: dx^T = Wup lg^T         -> Wup[32 mo + l%32][k .. k+7]
+    for (int i = t; i < MO * KH * 64; i += kMlpThreads) {
+        const int l = i % 64, s = (i / 64) % KH, mo = i / (64 * KH);
+        const int c = 32 * mo + l % 32;
+        a6[i] = c < C ? load_c8(Wup + c * H + 16 * s + 8 * (l / 32)) : z8;
+    }
+    for (int i = t; i < H; i += kMlpThreads) bsh[i] = bias[i];
+    const half8_t* a1f = reinterpret_cast<const half8_t*>(a1);
+
+    // reduction blocks of this wavefront: unit u = (type = u % 2, mh = (u / 2) % MH, mc = u / (2 MH));
+    // type 0: dWdown[h, c] = hid^T g, type 1: dWup[c, h] = x^T lg
+    const int u0 = Cfg::NU >= kMlpWaves ? wave : wave % Cfg::NU;
+    const int kpart = Cfg::NU >= kMlpWaves ? 0 : wave / Cfg::NU;
+    float16_t wacc[UPW];
+#pragma unroll
+    for (int uu = 0; uu < UPW; ++uu)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wacc[uu][i] = 0.0f;
+    float bacc = 0.0f;  // dbias: hidden channel t % H, voxels t / H + BPARTS * n
+    const int bh = t % H, bp = t / H;
+
+    const int64_t ntiles = (V + kMbTile - 1) / kMbTile;
+    half8_t xpre[NLX], gpre[NLX];
+    auto prefetch = [&](int64_t tile) {
+        const int64_t v0 = tile * kMbTile;
+#pragma unroll
+        for (int j = 0; j < NLX; ++j) {
+            const int c = t + j * kMlpThreads;
+            const int64_t v = v0 + c / (C / 8);
+            const bool ok = (c < Cfg::NXC) && (v < V);
+            xpre[j] = ok ? load_c8_nt(x + v * C + (c % (C / 8)) * 8) : z8;
+            gpre[j] = ok ? load_c8_nt(g + v * C + (c % (C / 8)) * 8) : z8;
+        }
+    };
+
+    int64_t tile = blockIdx.x;
+    if (tile < ntiles) prefetch(tile);
+    for (; tile < ntiles; tile += gridDim.x) {
+        const int64_t v0 = tile * kMbTile;
+        // ---- stage the tile (rows past V are zero: they add nothing to the reductions) ----
+#pragma unroll
+        for (int j = 0; j < NLX; ++j) {
+            const int c = t + j * kMlpThreads;
+            if (c < Cfg::NXC) {
+                *reinterpret_cast<half8_t*>(xs + (c / (C / 8)) * XP + (c % (C / 8)) * 8) = xpre[j];
+                *reinterpret_cast<half8_t*>(gs + (c / (C / 8)) * XP + (c % (C / 8)) * 8) = gpre[j];
+            }
+        }
+        __syncthreads();
+        if (tile + gridDim.x < ntiles) prefetch(tile + gridDim.x);
+
+        // ---- phase A: hid and lg tiles, blocks (vt, mh) of 32 voxels x 32 hidden channels ----
+#pragma unroll
+        for (int ba = 0; ba < (Cfg::NBA + kMlpWaves - 1) / kMlpWaves; ++ba) {
+            const int blk = wave + ba * kMlpWaves;
+            if (blk < Cfg::NBA) {  // wavefront-uniform
+                const int vt = blk % 2, mh = blk / 2;
+                const int row = 32 * vt + il;
+                float16_t up, dn;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) up[i] = dn[i] = 0.0f;
+#pragma unroll
+                for (int s = 0; s < KC; ++s) {
+                    const half8_t xb = *reinterpret_cast<const half8_t*>(xs + row * XP + 16 * s + 8 * hl);
+                    const half8_t gb = *reinterpret_cast<const half8_t*>(gs + row * XP + 16 * s + 8 * hl);
+                    up = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1f[(mh * KC + s) * 64 + lane], xb, up, 0, 0, 0);
+                    dn = __builtin_amdgcn_mfma_f32_32x32x16_f16(a3[(mh * KC + s) * 64 + lane], gb, dn, 0, 0, 0);
+                }
+                // up[i], dn[i]: hidden channel 32 mh + 8 (i/4) + 4 hl + i%4 of voxel row
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int hc = 32 * mh + 8 * gq + 4 * hl;
+                    const half4_t b4 = *reinterpret_cast<const half4_t*>(bsh + hc);
+                    half4_t hv, lv;
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const half_t lin = (half_t)((float)(half_t)up[4 * gq + jj] + (float)b4[jj]);  // fp16 add
+                        const bool pos = lin > (half_t)0;
+                        hv[jj] = pos ? lin : (half_t)0;
+                        lv[jj] = pos ? (half_t)dn[4 * gq + jj] : (half_t)0;
+                    }
+                    // rows past V hold x = g = 0: hid = relu(bias) there, which must not reach dWdown ... but
+                    // it is multiplied by g = 0; lg = fp16(0) = 0, so dWup and dbias are unaffected as well
+                    *reinterpret_cast<half4_t*>(hs + row * HP + hc) = hv;
+                    *reinterpret_cast<half4_t*>(ls + row * HP + hc) = lv;
+                }
+            }
+        }
+        __syncthreads();
+
+        // ---- phase B1: dx^T blocks (vt, mo) from the lg tile ----
+#pragma unroll
+        for (int b6 = 0; b6 < (Cfg::NB6 + kMlpWaves - 1) / kMlpWaves; ++b6) {
+            const int blk = wave + b6 * kMlpWaves;
+            if (blk < Cfg::NB6) {  // wavefront-uniform
+                const int vt = blk % 2, mo = blk / 2;
+                const int row = 32 * vt + il;
+                float16_t acc;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+                for (int s = 0; s < KH; ++s) {
+                    const half8_t lb = *reinterpret_cast<const half8_t*>(ls + row * HP + 16 * s + 8 * hl);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a6[(mo * KH + s) * 64 + lane], lb, acc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int c = 32 * mo + 8 * gq + 4 * hl;
+                    if (c < C) {
+                        half4_t o;
+#pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)acc[4 * gq + jj];
+                        *reinterpret_cast<half4_t*>(ds + row * DP + c) = o;
+                    }
+                }
+            }
+        }
+        // ---- phase B2: the reductions over the voxels of the tile ----
+#pragma unroll
+        for (int uu = 0; uu < UPW; ++uu) {
+            const int u = u0 + uu * kMlpWaves;
+            const int type = u % 2, mh = (u / 2) % MH, mc = u / (2 * MH);
+            const int cc = min(32 * mc + il, C - 1), hh = 32 * mh + il;
+            // A rows / B columns: type 0: (hid[:, hh], g[:, cc]); type 1: (x[:, cc], lg[:, hh])
+            const half_t* ap = type == 0 ? hs + hh : xs + cc;
+            const half_t* bp2 = type == 0 ? gs + cc : ls + hh;
+            const int apitch = type == 0 ? HP : XP, bpitch = type == 0 ? XP : HP;
+#pragma unroll
+            for (int sp = 0; sp < KV / KSPL; ++sp) {
+                const int s = kpart + sp * KSPL;
+                half8_t af, bf;
+#pragma unroll
+                for (int jj = 0; jj < 8; ++jj) {
+                    af[jj] = ap[(16 * s + 8 * hl + jj) * apitch];
+                    bf[jj] = bp2[(16 * s + 8 * hl + jj) * bpitch];
+                }
+                wacc[uu] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, wacc[uu], 0, 0, 0);
+            }
+        }
+        // dbias: column sums of the lg tile
+#pragma unroll
+        for (int n = 0; n < kMbTile / Cfg::BPARTS; ++n) bacc += (float)ls[(bp + Cfg::BPARTS * n) * HP + bh];
+        __syncthreads();
+
+        // ---- phase C: dx write-back, 16-byte chunks ----
+#pragma unroll
+        for (int j = 0; j < NLX; ++j) {
+            const int c = t + j * kMlpThreads;
+            const int row = c / (C / 8), cc = c % (C / 8);
+            if (c < Cfg::NXC && v0 + row < V) {
+                const half4_t lo = *reinterpret_cast<const half4_t*>(ds + row * DP + cc * 8);
+                const half4_t hi = *reinterpret_cast<const half4_t*>(ds + row * DP + cc * 8 + 4);
+                const half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                store_c8_nt(dx + (v0 + row) * C + cc * 8, o);
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- partials of this workgroup: row (blockIdx, kpart) = [dWup C*H][dWdown H*C][dbias H] ----
+    float* out = ws + ((int64_t)blockIdx.x * KSPL + kpart) * Cfg::RW;
+#pragma unroll
+    for (int uu = 0; uu < UPW; ++uu) {
+        const int u = u0 + uu * kMlpWaves;
+        const int type = u % 2, mh = (u / 2) % MH, mc = u / (2 * MH);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int ri = 8 * (i / 4) + 4 * hl + i % 4;  // row of the block held in register i
+            if (type == 0) {  // D[i = h][j = c]
+                const int h = 32 * mh + ri, c = 32 * mc + il;
+                if (c < C) out[C * H + h * C + c] = wacc[uu][i];
+            } else {  // D[i = c][j = h]
+                const int c = 32 * mc + ri, h = 32 * mh + il;
+                if (c < C) out[c * H + h] = wacc[uu][i];
+            }
+        }
+    }
+    bred[t] = bacc;
+    __syncthreads();
+    if (t < H) {
+        float s = 0.0f;
+#pragma unroll
+        for (int p = 0; p < Cfg::BPARTS; ++p) s += bred[p * H + t];
+        ws[((int64_t)blockIdx.x * KSPL) * Cfg::RW + 2 * C * H + t] = s;
+        for (int kp = 1; kp < KSPL; ++kp) ws[((int64_t)blockIdx.x * KSPL + kp) * Cfg::RW + 2 * C * H + t] = 0.0f;
+    }
+}
+
+// sums the rows of the partial buffer in a fixed order and scatters the three results
+__global__ __launch_bounds__(256) void mlp_reduce_kernel(const float* __restrict__ ws, int nrows, int RW, int n_up,
+                                                         int n_down, float* __restrict__ d_up,
+                                                         float* __restrict__ d_down, float* __restrict__ d_bias)
+{
+    __shared__ double part[16][17];
+    const int lo = threadIdx.x % 16, sl = threadIdx.x / 16;
+    const int j = blockIdx.x * 16 + lo;
+    double s = 0.0;
+    if (j < RW) {
+        for (int r = sl; r < nrows; r += 16) s += (double)ws[(int64_t)r * RW + j];
+    }
+    part[sl][lo] = s;
+    __syncthreads();
+    if (sl == 0 && j < RW) {
+        double v = 0.0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v += part[i][lo];
+        if (j < n_up) d_up[j] = (float)v;
+        else if (j < n_up + n_down) d_down[j - n_up] = (float)v;
+        else d_bias[j - n_up - n_down] = (float)v;
+    }
+}
+
+static int mb_blocks(int64_t V)
+{
+    const int64_t ntiles = (V + kMbTile - 1) / kMbTile;
+    return (int)std::max<int64_t>(1, std::min<int64_t>(ntiles, 512));
+}
+
+static int mb_kspl(int C)
+{
+    const int nu = 2 * (2 * C / 32) * ((C + 31) / 32);
+    return nu >= kMlpWaves ? 1 : kMlpWaves / nu;
+}
+
+}  // namespace kerops
+
+extern "C" int64_t kerops_lin_brelu_lin_bwd_workspace_bytes(int64_t V, int32_t C)
+{
+    if (V <= 0) {
+        set_error("lin_brelu_lin_bwd: non-positive size");
+        return KEROPS_E_BADARG;
+    }
+    if (!(C == 16 || C == 32 || C == 64)) {
+        set_error("lin_brelu_lin_bwd: built for C in {16,32,64} (got %d)", C);
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    return (int64_t)mb_blocks(V) * mb_kspl(C) * (4 * C * C + 2 * C) * (int64_t)sizeof(float);
+}
+
+extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const void* Wup, const void* Wdown,
+                                            const void* bias, void* dx, float* dWup, float* dWdown, float* dbias,
+                                            void* workspace, int64_t workspace_bytes, int64_t V, int32_t C,
+                                            void* stream)
+{
+    const int64_t need = kerops_lin_brelu_lin_bwd_workspace_bytes(V, C);
+    if (need < 0) return (int)need;
+    if (!x || !g || !Wup || !Wdown || !bias || !dx || !dWup || !dWdown || !dbias || !aligned16(x) || !aligned16(g) ||
+        !aligned16(Wup) || !aligned16(Wdown) || !aligned16(dx)) {
+        set_error("lin_brelu_lin_bwd: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
+        set_error("lin_brelu_lin_bwd: workspace of %lld bytes required, %lld given", (long long)need,
+                  (long long)workspace_bytes);
+        return KEROPS_E_WORKSPACE;
+    }
+    const int blocks = mb_blocks(V);
+    hipStream_t s = (hipStream_t)stream;
+    float* ws = (float*)workspace;
+#define KEROPS_MB_CASE(CV)                                                                                        \
+    if (C == CV) {                                                                                                \
+        hipLaunchKernelGGL((lin_brelu_lin_bwd_kernel<CV>), dim3(blocks), dim3(kMlpThreads), 0, s,                \
+                           (const half_t*)x, (const half_t*)g, (const half_t*)Wup, (const half_t*)Wdown,         \
+                           (const half_t*)bias, (half_t*)dx, ws, V);                                             \
+        int rc = check_launch("lin_brelu_lin_bwd");                                                               \
+        if (rc != KEROPS_OK) return rc;                                                                           \
+        const int RW = MbCfg<CV>::RW;                                                                             \
+        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(256), 0, s, ws,                       \
+                           blocks * MbCfg<CV>::KSPL, RW, 2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);          \
+        return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
+    }
+    KEROPS_MB_CASE(16)
+    KEROPS_MB_CASE(32)
+    KEROPS_MB_CASE(64)
+#undef KEROPS_MB_CASE
+    set_error("lin_brelu_lin_bwd: built for C in {16,32,64} (got %d)", C);
+    return KEROPS_E_UNSUPPORTED_C;
+}

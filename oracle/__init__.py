@@ -253,6 +253,20 @@ def lin_brelu_lin_add(x, weight_up, weight_down, bias, add, return_hidden=False)
     return _from_cl(out)
 
 
+def lin_brelu_lin_bwd(x, grad, weight_up, weight_down, bias):
+    """-> (dx fp16 like x, dWup fp64 [C,2C], dWdown fp64 [2C,C], dbias fp64 [2C])."""
+    n, c, h, w, d = x.shape
+    xc, gc = _cl(x), _cl(grad)
+    dx = torch.empty_like(xc)
+    dup = torch.empty(c, 2 * c, dtype=torch.float64)
+    ddn = torch.empty(2 * c, c, dtype=torch.float64)
+    db = torch.empty(2 * c, dtype=torch.float64)
+    lib().oracle_lin_brelu_lin_bwd(_p(xc), _p(gc), _p(weight_up.contiguous()), _p(weight_down.contiguous()),
+                                   _p(bias.contiguous()), _p(dx), _p(dup), _p(ddn), _p(db), _i64(n * h * w * d),
+                                   _i32(c))
+    return _from_cl(dx), dup, ddn, db
+
+
 def dwsep_block(x, dw_weight, scale, shift, pw_weight, return_mid=False):
     n, cin, h, w, d = x.shape
     cout = pw_weight.shape[1]

@@ -610,6 +610,59 @@ void oracle_lin_brelu_lin_add(const uint16_t *x, const uint16_t *Wup, const uint
     }
 }
 
+/* Backward of the inverted-bottleneck block: kerops/kernels/linear.py:149-230.
+ *   linup = fp16(x @ Wup) + bias (fp16 add, :196-198); hid = relu(linup) (:199)
+ *   dWdown[h,c] = sum_v hid[v,h] g[v,c] (:201-203)
+ *   lg[v,h] = linup > 0 ? fp16(sum_c Wdown[h,c] g[v,c]) : 0 (:205-207)
+ *   dWup[c,h] = sum_v x[v,c] lg[v,h] (:208-210);  dbias[h] = sum_v lg[v,h] (:211)
+ *   dx[v,c] = fp16(sum_h Wup[c,h] lg[v,h]) (:213-214)
+ * fp64 accumulate here; the weight / bias gradients are returned in fp64.
+ */
+void oracle_lin_brelu_lin_bwd(const uint16_t *x, const uint16_t *g, const uint16_t *Wup, const uint16_t *Wdown,
+                              const uint16_t *bias, uint16_t *dx, double *dWup, double *dWdown, double *dbias,
+                              int64_t V, int C)
+{
+    const int H = 2 * C;
+    float *hid = (float *)malloc((size_t)V * H * sizeof(float));
+    float *lg = (float *)malloc((size_t)V * H * sizeof(float));
+#pragma omp parallel for schedule(static)
+    for (int64_t v = 0; v < V; ++v) {
+        for (int h = 0; h < H; ++h) {
+            double s = 0.0, d = 0.0;
+            for (int c = 0; c < C; ++c) {
+                s += (double)h2f(x[v * C + c]) * (double)h2f(Wup[(int64_t)c * H + h]);
+                d += (double)h2f(g[v * C + c]) * (double)h2f(Wdown[(int64_t)h * C + c]);
+            }
+            const float lin = h2f(f2h(h2f(f2h((float)s)) + h2f(bias[h])));
+            const int pos = lin > 0.0f;
+            hid[v * H + h] = pos ? lin : 0.0f;
+            lg[v * H + h] = pos ? h2f(f2h((float)d)) : 0.0f;
+        }
+        for (int c = 0; c < C; ++c) {
+            double s = 0.0;
+            for (int h = 0; h < H; ++h) s += (double)h2f(Wup[(int64_t)c * H + h]) * (double)lg[v * H + h];
+            dx[v * C + c] = f2h((float)s);
+        }
+    }
+#pragma omp parallel for schedule(static)
+    for (int h = 0; h < H; ++h) {
+        double sb = 0.0;
+        for (int64_t v = 0; v < V; ++v) sb += (double)lg[v * H + h];
+        dbias[h] = sb;
+        for (int c = 0; c < C; ++c) {
+            double sd = 0.0, su = 0.0;
+            for (int64_t v = 0; v < V; ++v) {
+                sd += (double)hid[v * H + h] * (double)h2f(g[v * C + c]);
+                su += (double)h2f(x[v * C + c]) * (double)lg[v * H + h];
+            }
+            dWdown[(int64_t)h * C + c] = sd;
+            dWup[(int64_t)c * H + h] = su;
+        }
+    }
+    free(hid);
+    free(lg);
+}
+
 /* Fused depthwise-separable block of config 5 (composition of the pieces above;
  * no single reference counterpart): t = fp16(relu(dwconv(x) * scale[c] +
  * shift[c])) with the depthwise sum and the affine step in fp32; y = fp16(t @ Wm).

@@ -9,7 +9,7 @@ from torch.nn import functional as F
 import oracle
 from conftest import cpu_gen, rand_cl3d, rand_dw_weight
 from kerops_amd.ops.fused import DWSepBlock, DWSepBlockInt8, PointwiseLinear
-from kerops_amd.ops.linear import LinBReLULinAdd, ReLULinearAdd, ReLULinearBackward
+from kerops_amd.ops.linear import LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd, ReLULinearBackward
 from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
 
 pytestmark = pytest.mark.gpu
@@ -131,6 +131,54 @@ def test_lin_brelu_lin_add_closed_form_and_contract():
     with pytest.raises(CongiguratorError):
         LinBReLULinAdd(x128.to(DEV), rand_pw(g, 128, 256).to(DEV), rand_pw(g, 256, 128).to(DEV),
                        torch.zeros(256, dtype=torch.float16, device=DEV), x128.to(DEV))
+
+
+@pytest.mark.parametrize('c', [16, 32, 64])
+@pytest.mark.parametrize('spatial', [(1, 3, 5, 7), (2, 4, 4, 4), (1, 1, 1, 1), (3, 5, 13, 37), (1, 37, 53, 16)])
+def test_lin_brelu_lin_backward_matches_oracle(c, spatial):
+    g = cpu_gen(c * 91 + spatial[1])
+    n, h, w, d = spatial
+    x, grad = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    Wup, Wdown = rand_pw(g, c, 2 * c), rand_pw(g, 2 * c, c)
+    bias = (torch.randn(2 * c, generator=g) * 0.5).half()
+    dev = [t_.to(DEV) for t_ in (x, grad, Wup, Wdown, bias)]
+    dx, dup, ddn, db = (t_.cpu() for t_ in LinBReLULinBackward(*dev, out_dtype=torch.float32))
+    rdx, rup, rdn, rdb = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
+    assert dx.shape == x.shape and dx.stride() == x.stride()
+    assert dup.shape == (c, 2 * c) and ddn.shape == (2 * c, c) and db.shape == (2 * c,)
+    # fp32 MFMA sums vs the oracle's fp64: an intermediate fp16 value may round (or its ReLU mask flip at a
+    # linup within one rounding of zero) differently once in a while
+    assert (dx.float() - rdx.float()).abs().max() <= 2.0 ** -7 * max(1.0, rdx.abs().max().item())
+    same = (dx.contiguous().view(torch.int16) == rdx.contiguous().view(torch.int16)).float().mean().item()
+    assert same > 0.97, same
+    for got, ref in ((dup, rup), (ddn, rdn), (db, rdb)):
+        rel = ((got.double() - ref).norm() / max(ref.norm().item(), 1e-30)).item()
+        assert rel < 1e-3, rel
+    # the reference's own criteria (tests/ops/test_linear.py:153-200)
+    assert weight_grad_similarity(rdn.float(), ddn, rtol_cos=1e-4, atol_cos=1e-4, rtol_len=1e-3, atol_len=1e-3)
+    assert weight_grad_similarity(rup.float(), dup, rtol_cos=1e-4, atol_cos=1e-4, rtol_len=2e-3, atol_len=1e-3)
+    assert weight_grad_similarity(rdb.float(), db, rtol_cos=1e-3, atol_cos=1e-3, rtol_len=2e-3, atol_len=1e-3)
+    assert allclose_two_stage(rdx.contiguous(), dx.contiguous(), rtol_strict=1e-4, atol_strict=1e-3,
+                              rtol_narrow=1e-3, atol_narrow=4e-3)
+
+
+def test_lin_brelu_lin_backward_defaults_and_determinism():
+    g = cpu_gen(41)
+    c = 32
+    x, grad = rand_cl3d(g, 2, c, 37, 53, 16), rand_cl3d(g, 2, c, 37, 53, 16)
+    Wup, Wdown = rand_pw(g, c, 2 * c), rand_pw(g, 2 * c, c)
+    bias = (torch.randn(2 * c, generator=g) * 0.5).half()
+    dev = [t_.to(DEV) for t_ in (x, grad, Wup, Wdown, bias)]
+    r1 = LinBReLULinBackward(*dev)
+    r2 = LinBReLULinBackward(*dev)
+    assert all(t_.dtype == torch.float16 for t_ in r1)
+    assert all(torch.equal(a_, b_) for a_, b_ in zip(r1, r2))  # no atomics: bit-reproducible
+    rdx, rup, rdn, rdb = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
+    got = LinBReLULinBackward(*dev, out_dtype=torch.float32)
+    for a_, b_ in zip(got[1:], (rup, rdn, rdb)):
+        assert ((a_.cpu().double() - b_).norm() / b_.norm()).item() < 1e-3
+    with pytest.raises(AssertionError):
+        LinBReLULinBackward(dev[0], dev[1], dev[3], dev[2], dev[4])
 
 
 def test_pointwise_identity_and_no_relu():

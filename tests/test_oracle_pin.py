@@ -426,3 +426,34 @@ def test_lin_brelu_lin_add_vs_torch():
     eye_dn = torch.cat([torch.eye(c), torch.zeros(c, c)], 0).half()
     out = oracle.lin_brelu_lin_add(x, eye_up, eye_dn, torch.zeros(2 * c, dtype=torch.float16), add)
     assert torch.equal(out, (F.relu(x).float() + add.float()).half())
+
+
+def test_lin_brelu_lin_bwd_vs_torch():
+    """Pinned by a torch restatement with the kernel's fp16 roundings made explicit
+    (kerops/kernels/linear.py:196-214) and, loosely, by fp64 autograd of the two conv3d calls
+    (the ground truth of tests/ops/test_linear.py:146-151)."""
+    g = cpu_gen(37)
+    n, c, h, w, d = 2, 16, 3, 5, 4
+    x, grad = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    Wup = (torch.randn(c, 2 * c, generator=g) / math.sqrt(c)).half()
+    Wdown = (torch.randn(2 * c, c, generator=g) / math.sqrt(2 * c)).half()
+    bias = (torch.randn(2 * c, generator=g) * 0.5).half()
+    dx, dup, ddn, db = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
+    X = x.permute(0, 2, 3, 4, 1).reshape(-1, c).double()
+    G = grad.permute(0, 2, 3, 4, 1).reshape(-1, c).double()
+    lin = ((X @ Wup.double()).half().float() + bias.float()).half()
+    hid = F.relu(lin).double()
+    lg = torch.where(lin > 0, (G @ Wdown.double().t()).half(), torch.zeros_like(lin)).double()
+    assert torch.allclose(ddn, hid.t() @ G, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(dup, X.t() @ lg, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(db, lg.sum(0), rtol=1e-12, atol=1e-12)
+    ref_dx = (lg @ Wup.double().t()).half().reshape(n, h, w, d, c).permute(0, 4, 1, 2, 3)
+    assert torch.equal(dx, ref_dx) and dx.stride() == x.stride()
+    # fp64 autograd without the intermediate roundings agrees to fp16 accuracy
+    xd = x.double().requires_grad_(True)
+    wu, wd_, bd = (t_.double().requires_grad_(True) for t_ in (Wup, Wdown, bias))
+    y = F.conv3d(F.relu(F.conv3d(xd, wu.t().reshape(2 * c, c, 1, 1, 1), bd)), wd_.t().reshape(c, 2 * c, 1, 1, 1))
+    y.backward(grad.double())
+    for a_, b_ in ((dup, wu.grad), (ddn, wd_.grad), (db, bd.grad)):
+        assert ((a_ - b_).norm() / b_.norm()).item() < 2e-3
+    assert (dx.double() - xd.grad).abs().max() < 2e-2
