@@ -265,6 +265,27 @@ def main():
         y5, am5 = DWSepBlock(x5, wk5, sc5, sh5, Wm5)
         ops['config5_int8_pass'] = figures(time_op(torch, lambda: QuantInt8Sym(y5, am5), it, wm)[0], 3 * V5 * 128,
                                            c5_gbps)
+        # pointwise ops of the reference's linear family at (1,32,350,350,128) (its tests use 32 channels)
+        from kerops_amd.ops.linear import LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd, ReLULinearBackward
+        del y5
+        cl = 32
+        xl = torch.randn(1, 350, 350, 128, cl, device=dev, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+        gl = torch.randn(1, 350, 350, 128, cl, device=dev, dtype=torch.float16, generator=gen).permute(0, 4, 1, 2, 3)
+        Wl = (torch.randn(cl, cl, device=dev, generator=gen) / math.sqrt(cl)).half()
+        Wu = (torch.randn(cl, 2 * cl, device=dev, generator=gen) / math.sqrt(cl)).half()
+        Wd = (torch.randn(2 * cl, cl, device=dev, generator=gen) / math.sqrt(2 * cl)).half()
+        bl = (torch.randn(2 * cl, device=dev, generator=gen) * 0.5).half()
+        cl_ms = time_op(torch, lambda: xl.clone(), it, wm)[0]
+        cl_gbps = 4 * V * cl / cl_ms / 1e6
+        ops['ReLULinearAdd_32_32'] = figures(time_op(torch, lambda: ReLULinearAdd(xl, Wl, gl), it, wm)[0],
+                                             6 * V * cl, cl_gbps)
+        ops['ReLULinearBackward_32_32'] = figures(time_op(torch, lambda: ReLULinearBackward(xl, gl, Wl), it, wm)[0],
+                                                  6 * V * cl, cl_gbps)
+        ops['LinBReLULinAdd_32'] = figures(time_op(torch, lambda: LinBReLULinAdd(xl, Wu, Wd, bl, gl), it, wm)[0],
+                                           6 * V * cl, cl_gbps)
+        ops['LinBReLULinBackward_32'] = figures(
+            time_op(torch, lambda: LinBReLULinBackward(xl, gl, Wu, Wd, bl), it, wm)[0], 6 * V * cl, cl_gbps)
+        del xl, gl
         ops['config5_note'] = ('stage 1 = one kernel: matrix-core DWConv, BN+ReLU, fp16 tile through LDS into the MFMA '
                                '1x1x1 GEMM with fused max|y|; the 64-channel intermediate never reaches memory')
         ops['readme_table_note'] = 'C=8 (251 MB) fits the 256 MB Infinity Cache: its rows are not pure HBM numbers'
