@@ -13,6 +13,7 @@ from .ops.addition import AddStats, AddStatsBackward
 from .ops.avgpool import AvgPoolCeilStats, AvgPoolCeilStatsBackward
 from .ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
 from .ops.conv import DWConv, DWConvWGRAD
+from .ops.linear import LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd, ReLULinearBackward
 from .ops.stats import Stats, StatsBackward
 
 
@@ -101,3 +102,36 @@ class AvgPoolCeilStatsFn(torch.autograd.Function):
         (pooled,) = ctx.saved_tensors
         return AvgPoolCeilStatsBackward(_cl3d(grad_pooled), grad_mean.float().contiguous(),
                                         grad_sqmean.float().contiguous(), _cl3d(pooled), ctx.in_shape)
+
+
+class ReLULinearAddFn(torch.autograd.Function):
+    """out = fp16(relu(x) @ weight) + add_other; weight is [Cin, Cout] fp16."""
+
+    @staticmethod
+    def forward(ctx, x, weight, add_other):
+        ctx.save_for_backward(x, weight)
+        return ReLULinearAdd(x, weight, add_other)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weight = ctx.saved_tensors
+        grad_out = _cl3d(grad_out)
+        grad_x, grad_w = ReLULinearBackward(x, grad_out, weight, out_dtype=weight.dtype)
+        return grad_x, grad_w, grad_out  # the residual passes the gradient through
+
+
+class LinBReLULinAddFn(torch.autograd.Function):
+    """out = fp16(relu(fp16(x @ weight_up) + bias) @ weight_down) + add_other."""
+
+    @staticmethod
+    def forward(ctx, x, weight_up, weight_down, bias, add_other):
+        ctx.save_for_backward(x, weight_up, weight_down, bias)
+        return LinBReLULinAdd(x, weight_up, weight_down, bias, add_other)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, weight_up, weight_down, bias = ctx.saved_tensors
+        grad_out = _cl3d(grad_out)
+        grad_x, grad_up, grad_down, grad_bias = LinBReLULinBackward(x, grad_out, weight_up, weight_down, bias,
+                                                                    out_dtype=weight_up.dtype)
+        return grad_x, grad_up, grad_down, grad_bias, grad_out

@@ -93,3 +93,45 @@ def test_stats_fn_gradient():
     ((mean * um.to(DEV)).sum() + (sq * us.to(DEV)).sum()).backward()
     assert torch.equal(xd.grad.cpu().contiguous().view(torch.int16),
                        oracle.stats_bwd(x, um, us).contiguous().view(torch.int16))
+
+
+def test_linear_family_gradients_against_torch_autograd():
+    """ReLULinearAddFn and LinBReLULinAddFn against fp32 torch autograd of the 1x1x1 convolutions they stand for
+    (the ground truth of the reference's tests/ops/test_linear.py)."""
+    from kerops_amd.autograd import LinBReLULinAddFn, ReLULinearAddFn
+    g = cpu_gen(53)
+    n, c, co, h, w, d = 2, 32, 16, 5, 6, 7
+    x, add = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, co, h, w, d)
+    Wm = (torch.randn(c, co, generator=g) / math.sqrt(c)).half()
+    up = rand_cl3d(g, n, co, h, w, d)
+    xd, ad, wd = (t_.to(DEV).requires_grad_(True) for t_ in (x, add, Wm))
+    out = ReLULinearAddFn.apply(xd, wd, ad)
+    out.backward(up.to(DEV))
+    xr, ar, wr = (t_.float().requires_grad_(True) for t_ in (x, add, Wm))
+    ref = F.conv3d(F.relu(xr), wr.t().reshape(co, c, 1, 1, 1)) + ar
+    ref.backward(up.float())
+    assert torch.allclose(out.float().cpu(), ref, rtol=2e-3, atol=4e-3)
+    assert torch.allclose(xd.grad.float().cpu(), xr.grad, rtol=2e-3, atol=4e-3)
+    assert torch.equal(ad.grad.cpu(), up)
+    assert ((wd.grad.float().cpu() - wr.grad).norm() / wr.grad.norm()).item() < 2e-3
+
+    add2, up2 = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    Wu = (torch.randn(c, 2 * c, generator=g) / math.sqrt(c)).half()
+    Wd = (torch.randn(2 * c, c, generator=g) / math.sqrt(2 * c)).half()
+    b = (torch.randn(2 * c, generator=g) * 0.5).half()
+    dev = [t_.to(DEV).requires_grad_(True) for t_ in (x, Wu, Wd, b, add2)]
+    out = LinBReLULinAddFn.apply(*dev)
+    out.backward(up2.to(DEV))
+    refs = [t_.float().requires_grad_(True) for t_ in (x, Wu, Wd, b, add2)]
+    hid = F.relu(F.conv3d(refs[0], refs[1].t().reshape(2 * c, c, 1, 1, 1), refs[3]))
+    ref = F.conv3d(hid, refs[2].t().reshape(c, 2 * c, 1, 1, 1)) + refs[4]
+    ref.backward(up2.float())
+    assert torch.allclose(out.float().cpu(), ref, rtol=4e-3, atol=8e-3)
+    # a hidden unit whose pre-activation is within one fp16 rounding of zero may take the other side of the
+    # ReLU: rare, but it moves that voxel's input gradient by a whole weight row
+    bad = (dev[0].grad.float().cpu() - refs[0].grad).abs() > 2e-2 + 1e-2 * refs[0].grad.abs()
+    assert bad.float().mean().item() < 2e-2
+    for got, want in zip(dev[1:4], refs[1:4]):
+        # (the same flips reach the weight gradients; the strict comparison is the one against the oracle)
+        assert ((got.grad.float().cpu() - want.grad).norm() / want.grad.norm()).item() < 3e-2
+    assert torch.equal(dev[4].grad.cpu(), up2)
