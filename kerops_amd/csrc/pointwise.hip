@@ -7,12 +7,11 @@
 // matrix cores are used so that the arithmetic never shows up next to the memory stream.
 //
 // Each wavefront owns tiles of 32 voxels.  The product is computed transposed,
-// out^T[co, v] = Wm^T[co, :] . x^T[:, v], with v_mfma_f32_32x32x8_f16: the A operand is a
-// 32-row block of Wm^T (held in registers for the whole kernel), the B operand is x^T, whose
-// per-lane fragment "4 consecutive k of voxel lane%32" is simply 8 contiguous bytes of the
-// voxel's channel vector.  Any permutation of k is allowed as long as A and B agree, so a lane
-// loads whole 16-byte chunks: lane half h = lane/32 takes chunks 2q+h, MFMA step s uses half
-// s%2 of chunk 2*(s/2)+h.  The fp32 result fragment of a lane is 4 consecutive output channels
+// out^T[co, v] = Wm^T[co, :] . x^T[:, v], with v_mfma_f32_32x32x16_f16: the A operand is a
+// 32-row block of Wm^T (16-byte fragments pre-arranged in LDS, one ds_read_b128 per instruction), the
+// B operand is x^T, whose per-lane fragment "8 consecutive k of voxel lane%32" is simply one 16-byte
+// chunk of the voxel's channel vector: lane half h = lane/32 takes chunk 2s+h in step s.
+// The fp32 result fragment of a lane is 4 consecutive output channels
 // of one voxel (x 4 row groups x COUT/32 blocks); it is rounded to fp16, bounced through a
 // wavefront-private LDS tile [32][COUT] and written back as 16-byte chunks, coalesced, with
 // the optional fp16 residual add and the optional running max|out| fused into that pass.
@@ -28,8 +27,7 @@ constexpr int kPwWaves = kPwThreads / kWave;
 template <int CIN, int COUT>
 struct PwCfg {
     static constexpr int MT = (COUT + 31) / 32;      // 32-row blocks of output channels
-    static constexpr int KS = CIN / 8;               // MFMA steps (k = 8 each)
-    static constexpr int NQ = CIN / 16;              // 16-byte chunks a lane loads per voxel
+    static constexpr int KS = CIN / 16;              // MFMA steps (k = 16 each) = 16-byte chunks a lane loads per voxel
     static constexpr int ROW_HALVES = COUT + 4;      // LDS row pitch: +8 bytes staggers the banks
     static constexpr int TILE_HALVES = 32 * ROW_HALVES;
     static constexpr int OUT_CHUNKS = 32 * COUT / 8; // 16-byte chunks of one output tile
@@ -45,25 +43,22 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                                                                int64_t V)
 {
     using Cfg = PwCfg<CIN, COUT>;
-    constexpr int MT = Cfg::MT, KS = Cfg::KS, NQ = Cfg::NQ, RH = Cfg::ROW_HALVES;
+    constexpr int MT = Cfg::MT, KS = Cfg::KS, RH = Cfg::ROW_HALVES;
     __shared__ __attribute__((aligned(16))) half_t tile[kPwWaves][Cfg::TILE_HALVES];
+    __shared__ __attribute__((aligned(16))) half_t wfrag[MT * KS * 64 * 8];
     __shared__ float red[kPwWaves];
 
     const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
     const int vl = lane % 32, hl = lane / 32;
 
-    // A fragments: Wm^T[32*mt + vl][k], k = channels of (chunk 2*(s/2)+hl, half s%2)
-    half4_t wa[MT][KS];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int co = 32 * mt + vl;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            const int k0 = 8 * (2 * (s / 2) + hl) + 4 * (s % 2);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) wa[mt][s][j] = (co < COUT) ? Wm[(k0 + j) * COUT + co] : (half_t)0;
-        }
+    // A fragments: wfrag[((mt*KS + s)*64 + l)*8 + j] = Wm[16 s + 8 (l/32) + j][32 mt + l%32]
+    for (int i = t; i < MT * KS * 64 * 8; i += kPwThreads) {
+        const int j = i % 8, l = (i / 8) % 64, s = (i / 512) % KS, mt = i / (512 * KS);
+        const int co = 32 * mt + l % 32;
+        wfrag[i] = (co < COUT) ? Wm[(16 * s + 8 * (l / 32) + j) * COUT + co] : (half_t)0;
     }
+    __syncthreads();
+    const half8_t* wa = reinterpret_cast<const half8_t*>(wfrag) + lane;
 
     float amax = 0.0f;
     const int64_t ntiles = (V + 31) / 32;
@@ -79,12 +74,12 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
             // B fragments: this lane's voxel, chunks 2q+hl
             int64_t v = v0 + vl;
             if (v >= V) v = V - 1;  // ragged last tile: clamp the read, the write is masked
-            half8_t xb[NQ];
+            half8_t xb[KS];
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) xb[q] = load_c8(x + v * CIN + 8 * (2 * q + hl));
+            for (int q = 0; q < KS; ++q) xb[q] = load_c8(x + v * CIN + 8 * (2 * q + hl));
             if (RELU_IN) {
 #pragma unroll
-                for (int q = 0; q < NQ; ++q)
+                for (int q = 0; q < KS; ++q)
 #pragma unroll
                     for (int j = 0; j < 8; ++j) xb[q][j] = xb[q][j] > (half_t)0 ? xb[q][j] : (half_t)0;
             }
@@ -95,11 +90,9 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                 for (int i = 0; i < 16; ++i) acc[mt][i] = 0.0f;
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
-                half4_t b;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) b[j] = xb[s / 2][4 * (s % 2) + j];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_32x32x8f16(wa[mt][s], b, acc[mt], 0, 0, 0);
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wa[(mt * KS + s) * 64], xb[s], acc[mt], 0, 0, 0);
             }
             // acc[mt][i]: output channel 32*mt + 8*(i/4) + 4*hl + i%4 of voxel vl
 #pragma unroll
