@@ -850,8 +850,8 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
         // (the matrix-core kernels)
         switch (cg) {
             case 1: tile_w = 8; tile_d = 32; break;
-            case 2: tile_w = 8; tile_d = 16; break;
-            case 4: tile_w = 4; tile_d = 16; break;
+            case 2: tile_w = 8; tile_d = 32; break;
+            case 4: tile_w = 8; tile_d = 16; break;
             default: tile_w = 8; tile_d = 8; break;
         }
         lane_channels = 16;
@@ -878,6 +878,9 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
     KEROPS_FM_CASE(1, 8, 32, 256)
     KEROPS_FM_CASE(2, 8, 16, 256)
     KEROPS_FM_CASE(4, 4, 16, 256)
+    KEROPS_FM_CASE(1, 8, 64, 512)
+    KEROPS_FM_CASE(2, 8, 32, 512)
+    KEROPS_FM_CASE(4, 8, 16, 512)
     KEROPS_FM_CASE(8, 4, 8, 256)
     KEROPS_FM_CASE(8, 8, 8, 512)
     KEROPS_FM_CASE(8, 4, 16, 512)

@@ -12,9 +12,9 @@ from .._common import cl3d, next_power_of_2, require_cuda
 # gfx950 launch table, keyed by channel count like the reference's `warps` / `dblock`
 # (kerops/ops/conv/dwconv.py:10-17): (wavefronts per workgroup, tile extent along D,
 # tile extent along W).  A missing key means "no kernel for this channel count".
-_WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
-_TILE_D = {8: 32, 16: 16, 32: 16, 64: 8, 128: 8}
-_TILE_W = {8: 8, 16: 8, 32: 4, 64: 8, 128: 8}
+_WAVES = {8: 4, 16: 8, 32: 8, 64: 8, 128: 8}
+_TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
+_TILE_W = {8: 8, 16: 8, 32: 8, 64: 8, 128: 8}
 # 16 = matrix-core kernels (16 channel blocks per MFMA); 2 / 4 = vector kernels (channels per lane)
 _LANE_C = {8: 16, 16: 16, 32: 16, 64: 16, 128: 16}
 
