@@ -224,6 +224,10 @@ def main():
         ops['ApplyBNReLU'] = figures(time_op(torch, lambda: ApplyBNReLU(x, Wv, Bv), it, wm)[0], 4 * V * C, clone_gbps)
         ops['AvgPoolCeilStats'] = figures(time_op(torch, lambda: AvgPoolCeilStats(x), it, wm)[0],
                                           2 * V * C + 2 * (V // 8) * C, clone_gbps)
+        from kerops_amd.ops.avgpool import ApplyBNReLUAvgPoolCeilStats
+        ops['ApplyBNReLU+AvgPoolCeilStats_fused'] = figures(
+            time_op(torch, lambda: ApplyBNReLUAvgPoolCeilStats(x, Wv, Bv), it, wm)[0], 2 * V * C * (1 + 1 / 8),
+            clone_gbps)
         ops['QuantUint8Window'] = figures(time_op(torch, lambda: QuantUint8Window(x, 3.0), it, wm)[0], 3 * V * C,
                                           clone_gbps)
         table = {}

@@ -130,6 +130,15 @@ int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sq
                                   int32_t D, int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks,
                                   void* stream);
 
+/* ApplyBNReLU and AvgPoolCeilStats in one pass (no single reference counterpart; the reference composes
+ * the two ops, tests/ops/test_bn_relu.py:26-30 and tests/ops/test_avgpool.py): every existing voxel is
+ * mapped to fp16(max(x * weight[c] + bias[c], 0)) before the pool, so the result equals the composition
+ * bit for bit while the full-size intermediate never reaches memory.  Workspace as for
+ * kerops_avgpool_ceil_stats_f16. */
+int kerops_bnrelu_avgpool_ceil_stats_f16(const void* x, const float* weight, const float* bias, void* y, float* mean,
+                                         float* sqmean, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
+                                         void* workspace, int64_t workspace_bytes, int32_t blocks, void* stream);
+
 /* dx[every existing voxel of a window] =
  *   fp16((inpgrad + meangrad[c]/Mo + 2*output*sqmeangrad[c]/Mo) / count),
  * Mo = N*ceil(H/2)*ceil(W/2)*ceil(D/2); (N,H,W,D) is the shape of dx.

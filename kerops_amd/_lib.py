@@ -42,6 +42,8 @@ SIGNATURES = {
     'kerops_avgpool_ceil_stats_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_avgpool_ceil_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _i64, _i32,
                                                      _p]),
+    'kerops_bnrelu_avgpool_ceil_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _i64, _i32,
+                                                     _p]),
     'kerops_avgpool_ceil_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_quant_u8_window': (ctypes.c_int, [_p, _i32, _p, _i64, _f32, _i32, _p]),
     'kerops_dequant_u8_window': (ctypes.c_int, [_p, _p, _i32, _i64, _f32, _i32, _p]),

@@ -16,8 +16,13 @@ struct PoolDims {
     int N, H, W, D, Ho, Wo, Do, C, CG;
 };
 
-template <int V>
+// BNRELU: every voxel that exists is first mapped to fp16(max(x * bw[c] + bb[c], 0)), exactly what
+// bnrelu_fwd_kernel would have stored, so the fused op equals ApplyBNReLU followed by the pool bit for bit
+// while the full-size intermediate is neither written nor read.
+template <int V, bool BNRELU>
 __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_t* __restrict__ x,
+                                                                     const float* __restrict__ bw,
+                                                                     const float* __restrict__ bb,
                                                                      half_t* __restrict__ y, float* __restrict__ ws,
                                                                      const PoolDims p, int64_t nchunks)
 {
@@ -27,6 +32,16 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
     float acc[2][V];
 #pragma unroll
     for (int j = 0; j < V; ++j) acc[0][j] = acc[1][j] = 0.0f;
+    // the grid stride is a multiple of the number of channel groups: a thread keeps its channel group
+    float cw[V], cb[V];
+    if (BNRELU) {
+        const int cg0 = (int)(((int64_t)blockIdx.x * kStreamThreads + threadIdx.x) % p.CG);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            cw[j] = bw[cg0 * V + j];
+            cb[j] = bb[cg0 * V + j];
+        }
+    }
     const int64_t sD = p.CG, sW = (int64_t)p.D * p.CG, sH = (int64_t)p.W * sW, sN = (int64_t)p.H * sH;  // in chunks
 
     for (int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x; i < nchunks; i += T) {
@@ -55,6 +70,22 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
                     if (ok) t = ld_stream<V>(x, base + a * sH + b * sW + e * sD);
                     v[a][b][e] = t;
                 }
+        if (BNRELU) {
+            // a second pass, so that all eight loads are in flight before the first value is touched
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
+#pragma unroll
+                        for (int j = 0; j < V; ++j) {
+                            const half_t r = (half_t)fmaxf(__builtin_fmaf((float)v[a][b][e][j], cw[j], cb[j]), 0.0f);
+                            v[a][b][e][j] = ok ? r : (half_t)0;
+                        }
+                    }
+        }
         const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
         hv o;
 #pragma unroll
@@ -168,34 +199,61 @@ extern "C" int64_t kerops_avgpool_ceil_stats_workspace_bytes(int32_t N, int32_t 
     return rc != KEROPS_OK ? rc : need;
 }
 
-extern "C" int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H,
-                                             int32_t W, int32_t D, int32_t C, void* workspace,
-                                             int64_t workspace_bytes, int32_t blocks, void* stream)
+static int pool_fwd_run(const char* op, const void* x, const float* bw, const float* bb, void* y, float* mean,
+                        float* sqmean, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, void* workspace,
+                        int64_t workspace_bytes, int32_t blocks, void* stream)
 {
     PoolDims p;
     int64_t nchunks = 0, need = 0;
-    int rc = pool_plan("avgpool_ceil_stats", N, H, W, D, C, &blocks, &p, &nchunks, &need);
+    int rc = pool_plan(op, N, H, W, D, C, &blocks, &p, &nchunks, &need);
     if (rc != KEROPS_OK) return rc;
     if (!x || !y || !mean || !sqmean || !aligned16(x) || !aligned16(y)) {
-        set_error("avgpool_ceil_stats: null or misaligned pointer");
+        set_error("%s: null or misaligned pointer", op);
         return KEROPS_E_BADARG;
     }
     if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
-        set_error("avgpool_ceil_stats: workspace of %lld bytes required, %lld given", (long long)need,
-                  (long long)workspace_bytes);
+        set_error("%s: workspace of %lld bytes required, %lld given", op, (long long)need, (long long)workspace_bytes);
         return KEROPS_E_WORKSPACE;
     }
     hipStream_t s = (hipStream_t)stream;
     float* ws = (float*)workspace;
-    KEROPS_DISPATCH_V(C, {
-        hipLaunchKernelGGL((avgpool_fwd_kernel<V>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x,
-                           (half_t*)y, ws, p, nchunks);
-    });
-    rc = check_launch("avgpool_ceil_stats");
+    if (bw) {
+        KEROPS_DISPATCH_V(C, {
+            hipLaunchKernelGGL((avgpool_fwd_kernel<V, true>), dim3(blocks), dim3(kStreamThreads), 0, s,
+                               (const half_t*)x, bw, bb, (half_t*)y, ws, p, nchunks);
+        });
+    } else {
+        KEROPS_DISPATCH_V(C, {
+            hipLaunchKernelGGL((avgpool_fwd_kernel<V, false>), dim3(blocks), dim3(kStreamThreads), 0, s,
+                               (const half_t*)x, bw, bb, (half_t*)y, ws, p, nchunks);
+        });
+    }
+    rc = check_launch(op);
     if (rc != KEROPS_OK) return rc;
     const double Mo = (double)N * p.Ho * p.Wo * p.Do;
     launch_reduce_rows(ws, blocks, 2 * C, mean, sqmean, C, 1.0 / Mo, s);
-    return check_launch("avgpool_ceil_stats");
+    return check_launch(op);
+}
+
+extern "C" int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H,
+                                             int32_t W, int32_t D, int32_t C, void* workspace,
+                                             int64_t workspace_bytes, int32_t blocks, void* stream)
+{
+    return pool_fwd_run("avgpool_ceil_stats", x, nullptr, nullptr, y, mean, sqmean, N, H, W, D, C, workspace,
+                        workspace_bytes, blocks, stream);
+}
+
+extern "C" int kerops_bnrelu_avgpool_ceil_stats_f16(const void* x, const float* weight, const float* bias, void* y,
+                                                    float* mean, float* sqmean, int32_t N, int32_t H, int32_t W,
+                                                    int32_t D, int32_t C, void* workspace, int64_t workspace_bytes,
+                                                    int32_t blocks, void* stream)
+{
+    if (!weight || !bias) {
+        set_error("bnrelu_avgpool_ceil_stats: null weight or bias");
+        return KEROPS_E_BADARG;
+    }
+    return pool_fwd_run("bnrelu_avgpool_ceil_stats", x, weight, bias, y, mean, sqmean, N, H, W, D, C, workspace,
+                        workspace_bytes, blocks, stream);
 }
 
 extern "C" int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad, const float* sqmeangrad,

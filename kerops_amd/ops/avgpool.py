@@ -41,6 +41,34 @@ def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: Configura
     return output, mean, sqmean
 
 
+@configure(blocks=0)
+def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg):
+    """ApplyBNReLU(x, weight, bias) followed by AvgPoolCeilStats in one pass over x (no reference counterpart:
+    the reference composes kerops/ops/bnrelu.py:11-41 and kerops/ops/avgpool.py:11-60).  Bit-identical to the
+    composition; the full-size activation is neither written nor read.  Returns (pooled, mean, sqmean)."""
+    num_channels = x.shape[1]
+    assert num_channels == next_power_of_2(num_channels)
+    assert x.ndim == 5
+    assert x.dtype == torch.float16
+    assert x.is_contiguous(memory_format=torch.channels_last_3d)
+    assert weight.numel() == bias.numel() == num_channels
+    require_cuda(x, weight, bias)
+
+    n, _, h, w, d = x.shape
+    weight = weight.float().contiguous()
+    bias = bias.float().contiguous()
+    out_shape = [n] + [ceil(sh / 2) for sh in x.shape[2:]] + [num_channels]
+    output = torch.empty(out_shape, dtype=torch.float16, device=x.device).permute(0, 4, 1, 2, 3)
+    mean = torch.empty(num_channels, device=x.device, dtype=torch.float32)
+    sqmean = torch.empty(num_channels, device=x.device, dtype=torch.float32)
+    ws_bytes = _lib.query('kerops_avgpool_ceil_stats_workspace_bytes', n, h, w, d, num_channels, int(blocks))
+    ws = _lib.workspace(ws_bytes, x.device)
+    _lib.call('kerops_bnrelu_avgpool_ceil_stats_f16', x.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+              output.data_ptr(), mean.data_ptr(), sqmean.data_ptr(), n, h, w, d, num_channels, ws.data_ptr(),
+              ws_bytes, int(blocks), _lib.stream_of(x))
+    return output, mean, sqmean
+
+
 @configure(l1_cache_bytes=get_l1_cache, num_warps=4, blocks=0)
 def AvgPoolCeilStatsBackward(
     inpgrad,

@@ -13,7 +13,7 @@ import torch
 import oracle
 from conftest import cpu_gen, from_bits, rand_cl3d
 from kerops_amd.ops.addition import AddStats, AddStatsBackward
-from kerops_amd.ops.avgpool import AvgPoolCeilStats, AvgPoolCeilStatsBackward
+from kerops_amd.ops.avgpool import ApplyBNReLUAvgPoolCeilStats, AvgPoolCeilStats, AvgPoolCeilStatsBackward
 from kerops_amd.ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
 from kerops_amd.ops.quantization import AbsMax, DequantUint8Window, QuantInt8Sym, QuantUint8Window
 from kerops_amd.ops.stats import Stats, StatsBackward
@@ -120,6 +120,24 @@ def test_avgpool_and_backward(shape):
     dx = AvgPoolCeilStatsBackward(ig.to(DEV), mg.to(DEV), sg.to(DEV), ypc, x.shape)
     assert list(dx.shape) == list(x.shape)
     assert bits_equal(dx, oracle.avgpool_ceil_stats_bwd(ig, mg, sg, ryp, x.shape))
+
+
+@pytest.mark.parametrize('shape', SHAPES + [(2, 16, 2, 3, 2), (1, 64, 13, 7, 128), (1, 4, 5, 5, 5)])
+def test_bnrelu_avgpool_fused_equals_composition(shape):
+    """One pass = ApplyBNReLU then AvgPoolCeilStats, bit for bit: against the oracle's composition and
+    against the two separate GPU ops."""
+    g = cpu_gen(6)
+    c = shape[1]
+    x = rand_cl3d(g, *shape)
+    wv, bv = torch.rand(c, generator=g) + 0.5, torch.randn(c, generator=g) * 0.3
+    yp, mean, sq = ApplyBNReLUAvgPoolCeilStats(x.to(DEV), wv.to(DEV), bv.to(DEV))
+    ryp, rm, rs = oracle.avgpool_ceil_stats(oracle.bnrelu_fwd(x, wv, bv))
+    assert list(yp.shape) == [shape[0], c] + [math.ceil(s / 2) for s in shape[2:]]
+    assert yp.permute(0, 2, 3, 4, 1).is_contiguous()
+    assert bits_equal(yp, ryp)
+    assert close64(mean, rm) and close64(sq, rs)
+    y2, m2, s2 = AvgPoolCeilStats(ApplyBNReLU(x.to(DEV), wv.to(DEV), bv.to(DEV)))
+    assert torch.equal(yp, y2) and torch.equal(mean, m2) and torch.equal(sq, s2)
 
 
 def test_avgpool_golden(golden):
