@@ -464,9 +464,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     constexpr int NPOS = Cfg::TW * TD, RT = SC + 8, RY = COUT + 4;
     constexpr int KS = SC / 16, MT = COUT / 32, NPT = NPOS / 32;  // k = 16 per matrix instruction
     constexpr int T_OFF = Cfg::LDS_BYTES, Y_OFF = T_OFF + NPOS * RT * 2, A_OFF = Y_OFF + NPOS * RY * 2;
-    constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : Cfg::LDS_BYTES;
-    static_assert(MODE != 2 || (SC == 64 && NPOS % 32 == 0 && COUT % 32 == 0 && MT * NPT <= Cfg::NWAVE),
-                  "fused pointwise stage: 64 input channels, one (32 positions x 32 outputs) tile per wavefront");
+    // modes 0 and 1 with a 64-channel slab: two output tiles [NPOS][PB] behind the staging buffers.  A wavefront
+    // owns 32 channels, i.e. 64-byte halves of the 128-byte positions; written directly they cost 10 % more HBM
+    // write traffic than the tensor holds.  So a finished plane is written to the tile as dwords and leaves one
+    // step later, behind that step's barrier, as one 16-byte chunk per thread: whole lines, one store instruction
+    // instead of RO.  Narrower slabs write runs of 256 contiguous bytes anyway and store directly.
+    constexpr bool BOUNCE = MODE != 2 && SC == 64;
+    constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
+    static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
+    constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);
     __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
     __shared__ float amax_red[Cfg::NWAVE];
 
@@ -564,15 +570,35 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     int boff[3];
 #pragma unroll
     for (int k = 0; k < 3; ++k) boff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
-    // output: the lane's dword (two channels) of position pgrp + rr in the output rows ra .. ra+RO-1
+    // output tile: the halves of odd positions are swapped so that the four positions of a write spread over all banks
+    auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
+    int owr[RO];  // the lane's dword (two channels) of position pgrp + rr in the output rows ra .. ra+RO-1
+#pragma unroll
+    for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
+    // the thread's 16-byte chunk of the tile: position t / CG, channels 8 (t % CG) ..
+    const int opos = t / CG, ocq = t % CG;
+    const int ord = ot_swz(opos, ocq * 16);
+    const int ow = w0 + opos / TD, odd = d0 + opos % TD;
+    const bool ovalid = (ow < W) && (odd < D);
+    const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
+    int pending_row = -1;
+    auto flush_row = [&](int par) {  // stores the plane that the previous step left in output tile par
+        if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
+            const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + OT_OFF + par * OT_BYTES + ord);
+            // written once, never re-read: streaming hint keeps L2 for the halo rows
+            if (ovalid)
+                __builtin_nontemporal_store(
+                    o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(yn + pending_row * plane_stride) + ogo));
+        }
+    };
+    // direct stores (narrow slabs): the lane's dword of position pgrp + rr in the output rows ra .. ra+RO-1
     const int od = d0 + pgrp + rr;
-    const bool odv = od < D;
     uint32_t ooff[RO];
     bool oval[RO];
 #pragma unroll
     for (int o = 0; o < RO; ++o) {
         const int w = w0 + ra + o;
-        oval[o] = odv && (w < W);
+        oval[o] = (od < D) && (w < W);
         ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
     }
 
@@ -604,6 +630,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
             *reinterpret_cast<half8_t*>(dst) = xpre[j];
         }
         __syncthreads();
+        flush_row(parity ^ 1);
         prefetch(hp + AHEAD, xpre);
         __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
         if (xin) {
@@ -628,8 +655,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
         }
         // register 2 of every tile is the finished output plane hp-1
         const int ho = hp - 1;
+        pending_row = (ho >= hs) ? ho : -1;
         if (ho >= hs) {  // workgroup-uniform
-            char* yplane = MODE == 2 ? nullptr : reinterpret_cast<char*>(yn + ho * plane_stride);
+            unsigned char* otile = smem + OT_OFF + parity * OT_BYTES;
             half_t* tt = reinterpret_cast<half_t*>(smem + T_OFF);
 #pragma unroll
             for (int o = 0; o < RO; ++o) {
@@ -642,9 +670,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
                 }
                 if constexpr (MODE == 2) {
                     *reinterpret_cast<half2_t*>(tt + ((ra + o) * TD + pgrp + rr) * RT + half * 32 + 2 * q) = v;
+                } else if constexpr (BOUNCE) {
+                    *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
                 } else {
-                    // written once, never re-read: streaming hint keeps L2 for the halo rows
-                    if (oval[o]) __builtin_nontemporal_store(v, reinterpret_cast<half2_t*>(yplane + ooff[o]));
+                    if (oval[o])
+                        __builtin_nontemporal_store(
+                            v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(yn + ho * plane_stride) + ooff[o]));
                 }
             }
             if constexpr (MODE == 2) {
@@ -710,6 +741,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
             step(hp, xpre1);
             if (++hp > he) break;
         }
+    }
+    if constexpr (BOUNCE) {
+        __syncthreads();
+        flush_row(parity ^ 1);
     }
     if constexpr (MODE == 2) {
         amax = wave_max(amax);
