@@ -41,8 +41,8 @@ V = H * W * D
 # (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000):
 # profiles/dwconv_fwd_wgrad_c64_readme_shape.md.
 MEASURED_TRAFFIC_BYTES = {
-    ('dwconv_fwd', 64): 4450765775,    # 2.241 GB read + 2.209 GB written (1.109 x algorithmic)
-    ('dwconv_wgrad', 64): 4413166485,  # 4.399 GB read + 0.015 GB written (1.099 x algorithmic)
+    ('dwconv_fwd', 64): 4360563514,    # 2.354 GB read + 2.007 GB written (1.086 x algorithmic)
+    ('dwconv_wgrad', 64): 4392326091,  # 4.383 GB read + 0.010 GB written (1.094 x algorithmic)
 }
 
 
