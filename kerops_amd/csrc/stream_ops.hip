@@ -111,24 +111,29 @@ __global__ __launch_bounds__(kStreamThreads) void stats_bwd_kernel(const half_t*
         sg[j] = sqmean_grad[cg * V + j];
         mg[j] = __fdiv_rn(mean_grad[cg * V + j], fm);
     }
+    auto one = [&](const hv& v, const hv& g) {
+        hv o;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const float a = __fdiv_rn(__fmul_rn(__fmul_rn(2.0f, (float)v[j]), sg[j]), fm);
+            o[j] = ADD ? (half_t)__fadd_rn(__fadd_rn((float)g[j], a), mg[j]) : (half_t)__fadd_rn(a, mg[j]);
+        }
+        return o;
+    };
+    constexpr int U = ADD ? 2 : 4;  // chunks in flight per lane and input stream
+    for (; i + (U - 1) * T < nchunks; i += U * T) {
+        hv v[U], g[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v[u] = ld_stream<V>(x, i + u * T);
+            g[u] = ADD ? ld_stream<V>(add_grad, i + u * T) : v[u];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) st_stream<V>(dx, i + u * T, one(v[u], g[u]));
+    }
     for (; i < nchunks; i += T) {
         const hv v = ld_stream<V>(x, i);
-        hv o;
-        if (ADD) {
-            const hv g = ld_stream<V>(add_grad, i);
-#pragma unroll
-            for (int j = 0; j < V; ++j) {
-                const float a = __fdiv_rn(__fmul_rn(__fmul_rn(2.0f, (float)v[j]), sg[j]), fm);
-                o[j] = (half_t)__fadd_rn(__fadd_rn((float)g[j], a), mg[j]);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < V; ++j) {
-                const float a = __fdiv_rn(__fmul_rn(__fmul_rn(2.0f, (float)v[j]), sg[j]), fm);
-                o[j] = (half_t)__fadd_rn(a, mg[j]);
-            }
-        }
-        st_stream<V>(dx, i, o);
+        st_stream<V>(dx, i, one(v, ADD ? ld_stream<V>(add_grad, i) : v));
     }
 }
 

@@ -140,6 +140,41 @@ def test_bnrelu_avgpool_fused_equals_composition(shape):
     assert torch.equal(yp, y2) and torch.equal(mean, m2) and torch.equal(sq, s2)
 
 
+def _same_bits_or_nan(a, b):
+    a, b = a.cpu().contiguous(), b.contiguous()
+    both_nan = torch.isnan(a) & torch.isnan(b)
+    eq = a.view(torch.int16) == b.view(torch.int16)
+    return bool((eq | both_nan).all())
+
+
+@pytest.mark.parametrize('grad_scale', [1.0, 1e-30, 1e30, 3e38])
+def test_backward_ops_bit_exact_on_special_values(grad_scale):
+    """The divisions of StatsBackward / AddStatsBackward / AvgPoolCeilStatsBackward must give the oracle's
+    (IEEE) bits for every operand: signed zeros, infinities, NaNs, subnormals, huge and tiny gradients."""
+    g = cpu_gen(61)
+    shape = (1, 8, 6, 5, 16)
+    x = rand_cl3d(g, *shape)
+    flat = x.permute(0, 2, 3, 4, 1).reshape(-1)  # a view of the channels_last memory
+    special = torch.tensor([0.0, -0.0, float('inf'), -float('inf'), float('nan'), 65504.0, -65504.0, 6e-8, -6e-8,
+                            6.1e-5], dtype=torch.float16)
+    flat[torch.randperm(flat.numel(), generator=g)[:200]] = special.repeat(20)
+    c = shape[1]
+    mg = torch.randn(c, generator=g) * grad_scale
+    sg = torch.randn(c, generator=g) * grad_scale
+    sg[0], sg[1], mg[2], mg[3] = 0.0, -0.0, -0.0, 0.0
+    dx = StatsBackward(x.to(DEV), mg.to(DEV), sg.to(DEV))
+    assert _same_bits_or_nan(dx, oracle.stats_bwd(x, mg, sg))
+    ag = rand_cl3d(g, *shape)
+    out = AddStatsBackward(ag.to(DEV), mg.to(DEV), sg.to(DEV), x.to(DEV))
+    assert _same_bits_or_nan(out, oracle.add_stats_bwd(ag, mg, sg, x))
+    pooled_shape = (1, 8, 3, 3, 8)
+    ig, outp = rand_cl3d(g, *pooled_shape), rand_cl3d(g, *pooled_shape)
+    pf = outp.permute(0, 2, 3, 4, 1).reshape(-1)
+    pf[torch.randperm(pf.numel(), generator=g)[:100]] = special.repeat(10)
+    dxp = AvgPoolCeilStatsBackward(ig.to(DEV), mg.to(DEV), sg.to(DEV), outp.to(DEV), shape)
+    assert _same_bits_or_nan(dxp, oracle.avgpool_ceil_stats_bwd(ig, mg, sg, outp, shape))
+
+
 def test_avgpool_golden(golden):
     x = from_bits(golden['x']).to(memory_format=torch.channels_last_3d).to(DEV)
     yp, mean, sq = AvgPoolCeilStats(x)
