@@ -97,7 +97,7 @@ def cpu_baseline(torch, C):
     wk = wt[:, 0].permute(1, 2, 3, 0).contiguous()
     oracle.dwconv_fwd(x[:, :, :8], wk, wide=False)  # load the library, warm the thread pool
 
-    reps_f, reps_w = 3, 1
+    reps_f, reps_w = 12, 8  # about 10 s of CPU work on 16 cores
     t0 = time.perf_counter()
     for _ in range(reps_f):
         oracle.dwconv_fwd(x, wk, wide=False)
@@ -109,7 +109,7 @@ def cpu_baseline(torch, C):
     scale = V / vox
     port = {
         'value': round((t_f + t_w) * 1e3 * scale, 1), 'unit': 'ms', 'cores': oracle.num_threads(), 'kind': 'port',
-        'sample': f'oracle DWConv fwd (fp32, {reps_f} runs) + wgrad (fp64, {reps_w} run) on the leading crop '
+        'sample': f'oracle DWConv fwd (fp32, {reps_f} runs) + wgrad (fp64, {reps_w} runs) on the leading crop '
                   f'(1,{C},176,176,128), time scaled by the voxel ratio {scale:.2f} to (1,{C},350,350,128)',
         'fwd_ms_scaled': round(t_f * 1e3 * scale, 1), 'wgrad_ms_scaled': round(t_w * 1e3 * scale, 1),
         'host_cpus': os.cpu_count(),
