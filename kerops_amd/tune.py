@@ -1,0 +1,112 @@
+"""Measure the built launch shapes of DWConv / DWConvWGRAD on the GPU at hand and install the winners.
+
+The reference ships static per-channel tables tuned for one card (kerops/ops/conv/dwconv.py:10-17,
+kerops/ops/conv/dwconv_wgrad.py:10-22); the tables in kerops_amd/ops/conv were measured on an MI355X at
+(1, C, 350, 350, 128).  For another shape or part:
+
+    python -m kerops_amd.tune --shape 1 64 350 350 128          # print the timings
+    python -m kerops_amd.tune --channels 32 64 --apply          # and reconfigure the ops of this process
+
+`tune(...)` returns {op: {C: (W_block, D_block, lane_channels, H_chunk, ms)}}; `apply(result)` installs the
+choices through the ops' `reconfigure`, the same mechanism a user of the reference has for overriding its tables.
+"""
+import argparse
+import math
+
+import torch
+
+from .ops.conv import DWConv, DWConvWGRAD
+from .ops.conv.variants import FWD_VARIANTS, WGRAD_VARIANTS, threads_per_workgroup
+
+
+def _time(fn, iters, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return ts[len(ts) // 2]
+
+
+def tune(shape=(1, 64, 350, 350, 128), channels=None, h_chunks=(0,), iters=10, warmup=3, device='cuda', verbose=False):
+    """Times every built launch shape for the given (N, C, H, W, D) (C replaced by each entry of `channels`)."""
+    n, c0, h, w, d = shape
+    result = {'DWConv': {}, 'DWConvWGRAD': {}}
+    for c in (channels or [c0]):
+        x = torch.randn(n, h, w, d, c, device=device, dtype=torch.float16).permute(0, 4, 1, 2, 3)
+        g = torch.randn(n, h, w, d, c, device=device, dtype=torch.float16).permute(0, 4, 1, 2, 3)
+        wk = (torch.randn(3, 3, 3, c, device=device) / math.sqrt(27)).half()
+        for name, table, run in (
+            ('DWConv', FWD_VARIANTS, lambda kw: DWConv(x, wk, **kw)),
+            ('DWConvWGRAD', WGRAD_VARIANTS, lambda kw: DWConvWGRAD(x, g, **kw)),
+        ):
+            best = None
+            for (tw, td, cl) in table[c]:
+                for hc in h_chunks:
+                    kw = dict(W_block=tw, D_block=td, lane_channels=cl, H_chunk=hc,
+                              num_warps=threads_per_workgroup(c, tw, td, cl) // 64)
+                    ms = _time(lambda: run(kw), iters, warmup)
+                    if verbose:
+                        print(f'{name:12s} C={c:3d} patch {tw}x{td} lane_channels {cl:2d} H_chunk {hc:3d}: {ms:.3f} ms',
+                              flush=True)
+                    if best is None or ms < best[4]:
+                        best = (tw, td, cl, hc, ms)
+            result[name][c] = best
+        del x, g
+    return result
+
+
+def _picker(table, idx, fallback):
+    def pick(x):
+        c = x.shape[1]
+        return table[c][idx] if c in table else fallback(c)
+
+    return pick
+
+
+def _warps_picker(table, fallback):
+    def pick(x):
+        c = x.shape[1]
+        return threads_per_workgroup(c, *table[c][:3]) // 64 if c in table else fallback(c)
+
+    return pick
+
+
+def apply(result):
+    """Installs the measured winners as the ops' defaults (channel counts not measured keep the built-in table)."""
+    from .ops.conv import dwconv as fwd_mod, dwconv_wgrad as wg_mod
+    for op, mod, key in ((DWConv, fwd_mod, 'DWConv'), (DWConvWGRAD, wg_mod, 'DWConvWGRAD')):
+        table = result.get(key, {})
+        if not table:
+            continue
+        conf = dict(op.configurators)
+        conf['W_block'] = _picker(table, 0, mod.wtile)
+        conf['D_block'] = _picker(table, 1, mod.dblock)
+        conf['lane_channels'] = _picker(table, 2, getattr(mod, 'lanec', lambda c: 16))
+        conf['H_chunk'] = _picker(table, 3, lambda c: 0)
+        conf['num_warps'] = _warps_picker(table, mod.warps)
+        op.reconfigure(**conf)
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__.split('\n')[0])
+    ap.add_argument('--shape', type=int, nargs=5, default=[1, 64, 350, 350, 128], metavar=('N', 'C', 'H', 'W', 'D'))
+    ap.add_argument('--channels', type=int, nargs='*', default=None)
+    ap.add_argument('--h-chunks', type=int, nargs='*', default=[0])
+    ap.add_argument('--apply', action='store_true')
+    args = ap.parse_args()
+    res = tune(tuple(args.shape), args.channels, tuple(args.h_chunks), verbose=True)
+    for op, table in res.items():
+        for c, (tw, td, cl, hc, ms) in table.items():
+            print(f'best {op:12s} C={c:3d}: W_block={tw} D_block={td} lane_channels={cl} H_chunk={hc}  {ms:.3f} ms')
+    if args.apply:
+        apply(res)
+
+
+if __name__ == '__main__':
+    main()

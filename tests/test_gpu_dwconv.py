@@ -65,17 +65,7 @@ def test_dwconv_wgrad_matches_oracle(shape):
                                       rtol_len=1e-3 * shape[0], atol_len=1e-3)
 
 
-FWD_VARIANTS = {8: [(16, 32, 4), (16, 32, 2), (8, 32, 16), (8, 64, 16)],
-                16: [(8, 32, 4), (8, 32, 2), (8, 16, 16), (8, 32, 16)],
-                32: [(8, 16, 4), (8, 16, 2), (4, 16, 16), (8, 16, 16)],
-                64: [(4, 8, 4), (4, 8, 2), (4, 16, 2), (8, 8, 2), (4, 8, 16), (8, 8, 16), (4, 16, 16)],
-                128: [(4, 8, 4), (4, 8, 2), (4, 16, 2), (8, 8, 2), (4, 8, 16), (8, 8, 16), (4, 16, 16)]}
-# lane_channels 2: vector dot-product kernels; 16: matrix-core kernels (16 channel blocks per instruction)
-WG_VARIANTS = {8: [(16, 32, 2), (8, 32, 2), (8, 32, 16), (8, 64, 16)],
-               16: [(8, 32, 2), (8, 16, 2), (8, 16, 16), (8, 32, 16)],
-               32: [(8, 16, 2), (4, 16, 2), (4, 16, 16), (8, 16, 16)],
-               64: [(8, 8, 2), (4, 16, 2), (4, 8, 2), (4, 8, 16), (8, 8, 16), (4, 16, 16)],
-               128: [(8, 8, 2), (4, 16, 2), (4, 8, 2), (4, 8, 16), (8, 8, 16), (4, 16, 16)]}
+from kerops_amd.ops.conv.variants import FWD_VARIANTS, WGRAD_VARIANTS as WG_VARIANTS  # noqa: E402
 
 
 @pytest.mark.parametrize('c', [8, 16, 32, 64, 128])

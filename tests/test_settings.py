@@ -105,3 +105,35 @@ def test_confexc_passes_other_exceptions():
 
     with pytest.raises(ValueError):
         c(1)
+
+
+def test_tuner_apply_installs_and_falls_back():
+    """kerops_amd.tune.apply reconfigures the conv ops through the settings mechanism; channel counts that were
+    not measured keep the built-in tables (no GPU needed: only the configurators are evaluated)."""
+    import torch
+
+    from kerops_amd import tune
+    from kerops_amd.ops.conv import DWConv, DWConvWGRAD
+    from kerops_amd.ops.conv.variants import FWD_VARIANTS, WGRAD_VARIANTS, threads_per_workgroup
+
+    saved = dict(DWConv.configurators), dict(DWConvWGRAD.configurators)
+    try:
+        tune.apply({'DWConv': {64: (4, 8, 16, 88, 0.9)}, 'DWConvWGRAD': {64: (4, 16, 2, 0, 0.9)}})
+        x64, x32 = torch.empty(1, 64, 2, 2, 2), torch.empty(1, 32, 2, 2, 2)
+        got = {k: (c(x64) if callable(c) else c) for k, c in DWConv.configurators.items()}
+        assert (got['W_block'], got['D_block'], got['lane_channels'], got['H_chunk'], got['num_warps']) == (4, 8, 16, 88, 4)
+        got = {k: (c(x32) if callable(c) else c) for k, c in DWConv.configurators.items()}
+        assert (got['W_block'], got['D_block'], got['lane_channels'], got['H_chunk']) == (8, 16, 16, 0)
+        got = {k: (c(x64) if callable(c) else c) for k, c in DWConvWGRAD.configurators.items()}
+        assert (got['W_block'], got['D_block'], got['lane_channels'], got['num_warps']) == (4, 16, 2, 4)
+    finally:
+        DWConv.reconfigure(**saved[0])
+        DWConvWGRAD.reconfigure(**saved[1])
+    # the built-in defaults are entries of the variant tables, with the workgroup size the library uses
+    for c in (8, 16, 32, 64, 128):
+        x = torch.empty(1, c, 2, 2, 2)
+        for op, table in ((DWConv, FWD_VARIANTS), (DWConvWGRAD, WGRAD_VARIANTS)):
+            conf = {k: (f(x) if callable(f) else f) for k, f in op.configurators.items()}
+            shape = (conf['W_block'], conf['D_block'], conf['lane_channels'])
+            assert shape in table[c], (op, c, shape)
+            assert conf['num_warps'] * 64 == threads_per_workgroup(c, *shape)
