@@ -228,6 +228,9 @@ def main():
         ops['ApplyBNReLU+AvgPoolCeilStats_fused'] = figures(
             time_op(torch, lambda: ApplyBNReLUAvgPoolCeilStats(x, Wv, Bv), it, wm)[0], 2 * V * C * (1 + 1 / 8),
             clone_gbps)
+        from kerops_amd.ops.conv import DWConvBackward
+        ops['DWConvBackward_fused'] = figures(time_op(torch, lambda: DWConvBackward(x, g, wk), it, wm)[0], 6 * V * C,
+                                              clone_gbps)
         ops['QuantUint8Window'] = figures(time_op(torch, lambda: QuantUint8Window(x, 3.0), it, wm)[0], 3 * V * C,
                                           clone_gbps)
         table = {}

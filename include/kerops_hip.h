@@ -76,6 +76,18 @@ int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* works
                             int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d,
                             int32_t h_chunk, int32_t lane_channels, void* stream);
 
+/* Backward of the depthwise convolution in one pass over x and g (no reference counterpart: the reference has
+ * no input gradient, TODO at kerops/kernels/dw_conv.py:145, and computes the weight gradient separately,
+ * kerops/ops/conv/dwconv_wgrad.py:25-79):
+ *   dx[n,h,w,d,c] = sum_{kh,kw,kd} g[n,h-kh+1,w-kw+1,d-kd+1,c] * wt[kh,kw,kd,c]      (fp16, one rounding)
+ *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]        (fp32, deterministic)
+ * Every plane of g is staged once and feeds both products, which saves one of the two reads of g that
+ * kerops_dwconv_fwd_f16(g, flipped wt) + kerops_dwconv_wgrad_f16 need.  C in {8,16,32,64,128}. */
+int64_t kerops_dwconv_bwd_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t h_chunk);
+int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* wt, void* dx, float* gw, void* workspace,
+                          int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
+                          int32_t h_chunk, void* stream);
+
 /* Per-channel mean and mean of squares over M = numel / C voxels, fp32.
  * Replaces the zero-fill of mean/sqmean and the `_Stats_cl3d_impl[(grid,)](...)`
  * launch: kerops/ops/stats.py:27-31 (kernel kerops/kernels/stats.py:6-23).

@@ -1,2 +1,3 @@
 from .dwconv import DWConv
+from .dwconv_backward import DWConvBackward
 from .dwconv_wgrad import DWConvWGRAD

@@ -195,3 +195,31 @@ def test_readme_shape_properties(c):
         # halo removes exactly those rows from the comparison
         assert torch.allclose(got.float(), ref32[sl], rtol=1e-2, atol=1e-2)  # BASELINE config 2 tolerance
         assert (got.float() - ref32[sl]).abs().max() <= 2.0 ** -11 * max(1.0, ref32.abs().max().item()) * 1.01
+
+
+@pytest.mark.parametrize('c', [8, 16, 32, 64, 128])
+@pytest.mark.parametrize('shape_hc', [((2, 11, 19, 37), 0), ((1, 5, 3, 2), 0), ((1, 13, 9, 70), 4), ((1, 9, 8, 8), 1),
+                                      ((1, 7, 20, 130), 100)])
+def test_fused_backward_matches_oracle_and_separate_ops(c, shape_hc):
+    """DWConvBackward = (DWConv(grad, flipped weight), DWConvWGRAD(x, grad)), every plane of grad staged once."""
+    from kerops_amd.ops.conv import DWConvBackward
+    (n, h, w, d), hc = shape_hc
+    g = cpu_gen(c + h)
+    x, grad = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    _, wk = rand_dw_weight(g, c)
+    xd, gd, wd = x.to(DEV), grad.to(DEV), wk.to(DEV)
+    dx, gw = DWConvBackward(xd, gd, wd, H_chunk=hc, out_dtype=torch.float32)
+    assert dx.shape == x.shape and dx.stride() == x.stride() and gw.shape == (3, 3, 3, c)
+    ref_gw = oracle.dwconv_wgrad(x, grad)
+    rel = ((gw.cpu().double() - ref_gw).norm() / ref_gw.norm()).item()
+    assert rel < 2e-6, rel
+    wflip = torch.flip(wk, dims=(0, 1, 2)).contiguous()
+    check_fwd(grad, wflip, dx)
+    # same arithmetic as the separate matrix-core kernels: the input gradient agrees to the last bit
+    dx2 = DWConv(gd, wflip.to(DEV))
+    assert torch.equal(dx, dx2)
+    gw2 = DWConvWGRAD(xd, gd, out_dtype=torch.float32)
+    assert ((gw - gw2).norm() / gw2.norm()).item() < 2e-6  # other patch shape, other summation order
+    # determinism
+    dx3, gw3 = DWConvBackward(xd, gd, wd, H_chunk=hc, out_dtype=torch.float32)
+    assert torch.equal(dx, dx3) and torch.equal(gw, gw3)
