@@ -238,7 +238,9 @@ def main():
             if c == C:
                 table[str(c)] = {'clone_ms': round(clone_ms, 4), 'dwconv_ms': fwd['ms'], 'wgrad_ms': wg['ms'],
                                  'dwconv_frac_of_clone': fwd['frac_of_clone'],
-                                 'wgrad_frac_of_clone': wg['frac_of_clone']}
+                                 'wgrad_frac_of_clone': wg['frac_of_clone'],
+                                 'dwconv_frac_hbm_peak': fwd['frac_hbm_peak'],
+                                 'wgrad_frac_hbm_peak': wg['frac_hbm_peak']}
                 continue
             x = g = None
             torch.cuda.empty_cache()

@@ -324,7 +324,9 @@ struct WmCfg {
     static constexpr int R = TW + 2;                       // x rows incl. halo
     static constexpr int PDP = (TD + 2 + 3) / 4 * 4;       // x positions per row incl. halo, padded to 4
     static constexpr int XSLOT = R * PDP * PB;
-    static constexpr int GSLOT = TW * TD * PB + 32;
+    // lanes j read different slots: shift their banks apart (with 8 channels a half wavefront reads two
+    // position groups 16 banks apart, so the shift is 4 banks there, 8 otherwise)
+    static constexpr int GSLOT = TW * TD * PB + (SC == 8 ? 16 : 32);
     static constexpr int XOFF = 4 * GSLOT;                 // [4 g slots][2 x slots][dump]
     static constexpr int DUMP = XOFF + 2 * XSLOT;
     static constexpr int STAGE_BYTES = DUMP + 16;
@@ -564,7 +566,7 @@ struct BwCfg {
     static constexpr int R = TW + 2;                  // rows incl. halo
     static constexpr int PDP = (TD + 3 + 3) / 4 * 4;  // positions per row: halo + one over-read, padded to 4
     static constexpr int SLOT = R * PDP * PB;
-    static constexpr int GSLOT = SLOT + 32;           // lanes j read different slots: shift their banks apart
+    static constexpr int GSLOT = SLOT + (SC == 8 ? 16 : 32);  // lanes j read different slots: shift their banks apart
     static constexpr int XOFF = 4 * GSLOT;            // [4 g slots][2 x slots][2 output tiles][dump]
     static constexpr int NPOS = TW * TD, OT_BYTES = NPOS * PB;
     static constexpr int OT_OFF = XOFF + 2 * SLOT;
