@@ -202,6 +202,9 @@ extern "C" int kerops_lin_brelu_lin_add_f16(const void* x, const void* Wup, cons
 //   dWup[c, h]   = sum_v x[v, c] * lg[v, h];   dbias[h] = sum_v lg[v, h]
 //   dx[v, c]     = fp16(sum_h Wup[c, h] * lg[v, h])
 //
+// Two kernels: C <= 32 (one block of in / out channels) runs lin_brelu_lin_bwd_wave_kernel further down,
+// where a wavefront needs no LDS tiles and no workgroup barrier per tile; C = 64 runs the kernel below.
+//
 // A workgroup of four wavefronts loops over tiles of 64 voxels; x and g tiles are staged through LDS.
 // Phase A: per (32 voxels, 32 hidden channels) block a wavefront computes linup^T and (Wdown g^T) with the
 // same output layout, applies bias / ReLU / mask in registers and writes the hid and lg tiles to LDS.
@@ -472,6 +475,314 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_bwd_kernel(const ha
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// C <= 32: every wavefront works alone on tiles of 32 voxels, no workgroup barrier inside the loop.
+//
+// The per-voxel products want "voxel per lane" results (lane = voxel, registers = channels: the B operand
+// of the next per-voxel product), the reductions over voxels want "channel per lane" operands (lane =
+// channel, registers = 8 voxels).  A 32x32 matrix-core block D = A B holds column j in lane j%32, so the
+// second form of a tile M[v][c] is the product M I with an identity B fragment: exact, since every sum has
+// one non-zero term.  Fragments of x and g come straight from global memory (16-byte chunk 2 s + l/32 of
+// voxel l%32: the same registers serve as A operand of the transposing product and B operand of the
+// per-voxel products); hid and lg are transposed from their packed fp16 registers, whose reduction index
+// runs over the hidden channels in the order the accumulator leaves them, with a matching permuted
+// identity.  Weight and identity fragments sit in LDS (one 16-byte read per lane and use).  The
+// accumulators of dWup, dWdown and dbias stay in registers for all tiles of the wavefront; at the end the
+// four wavefronts add theirs in LDS in a fixed order and the workgroup writes one partial row.
+template <int C>
+struct MtCfg {
+    static constexpr int H = 2 * C;
+    static constexpr int MH = H / 32;   // 32-channel blocks of the hidden channels
+    static constexpr int KC = C / 16;   // k steps over the in / out channels
+    static constexpr int DP = C + 4;    // row pitch of the dx tile (halves)
+    static constexpr int RW = 2 * C * H + H;
+    static constexpr int F1_OFF = 0;                              // Wup^T rows   [mh][s]
+    static constexpr int F2_OFF = F1_OFF + MH * KC * 1024;        // Wdown rows   [mh][s]
+    static constexpr int F3_OFF = F2_OFF + MH * KC * 1024;        // Wup rows, hidden order of the accumulator
+    static constexpr int IP_OFF = F3_OFF + 2 * MH * 1024;         // identity in that order [half]
+    static constexpr int ID_OFF = IP_OFF + 2 * 1024;              // identity [s]
+    static constexpr int BH_OFF = ID_OFF + KC * 1024;             // bias
+    static constexpr int DS_OFF = (BH_OFF + H * 2 + 15) / 16 * 16;
+    static constexpr int LOOP_BYTES = DS_OFF + kMlpWaves * 32 * DP * 2;
+    static constexpr int LDS_BYTES = LOOP_BYTES > RW * 4 ? LOOP_BYTES : RW * 4;
+    static_assert(C == 16 || C == 32, "one 32-channel block of in / out channels");
+};
+
+// fp32 accumulator -> the two packed fp16 operands (registers 0..7 and 8..15)
+__device__ __forceinline__ void pack_acc(const float16_t& a, half8_t& lo, half8_t& hi)
+{
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        lo[i] = (half_t)a[i];
+        hi[i] = (half_t)a[8 + i];
+    }
+}
+
+typedef short i16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+
+// Two neighbouring accumulator registers of both products -> packed (hid, lg), 16-bit packed operations only:
+// lin = fp16(up) + bias (fp16 add);  hid = relu(lin) as the signed integer maximum of the bit pattern with 0
+// (negative values and -0 have the sign bit set, positive ones compare like integers);  lg = fp16(dn) where
+// hid has a non-zero bit pattern, i.e. where lin > 0.
+__device__ __forceinline__ void hid_lg_pair(float u0, float u1, float d0, float d1, half2_t b, half2_t& hid,
+                                            half2_t& lg)
+{
+    const half2_t up2 = {(half_t)u0, (half_t)u1};
+    const half2_t dn2 = {(half_t)d0, (half_t)d1};
+    const half2_t lin = up2 + b;
+    const i16x2_t hb = __builtin_elementwise_max(__builtin_bit_cast(i16x2_t, lin), i16x2_t{0, 0});
+    hid = __builtin_bit_cast(half2_t, hb);
+    const u16x2_t one = {1, 1}, zero = {0, 0};
+    uint32_t nz;  // written out: the compiler would turn the minimum into two compares and selects
+    asm("v_pk_min_u16 %0, %1, %2" : "=v"(nz) : "v"(__builtin_bit_cast(uint32_t, hb)), "v"(__builtin_bit_cast(uint32_t, one)));
+    const u16x2_t m = zero - __builtin_bit_cast(u16x2_t, nz);  // 0 or 0xffff per half
+    lg = __builtin_bit_cast(half2_t, __builtin_bit_cast(uint32_t, dn2) & __builtin_bit_cast(uint32_t, m));
+}
+
+template <int C>
+__global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
+    const half_t* __restrict__ x, const half_t* __restrict__ g, const half_t* __restrict__ Wup,
+    const half_t* __restrict__ Wdown, const half_t* __restrict__ bias, half_t* __restrict__ dx,
+    float* __restrict__ ws, int64_t V)
+{
+    using Cfg = MtCfg<C>;
+    constexpr int H = Cfg::H, MH = Cfg::MH, KC = Cfg::KC, DP = Cfg::DP;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+    half_t* f1w = reinterpret_cast<half_t*>(smem + Cfg::F1_OFF);
+    half_t* f3w = reinterpret_cast<half_t*>(smem + Cfg::F3_OFF);
+    half_t* ipw = reinterpret_cast<half_t*>(smem + Cfg::IP_OFF);
+    half_t* idw = reinterpret_cast<half_t*>(smem + Cfg::ID_OFF);
+    half_t* bsh = reinterpret_cast<half_t*>(smem + Cfg::BH_OFF);
+
+    const int t = threadIdx.x, lane = t % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(t / kWave);  // scalar: tile indices stay wavefront-uniform
+    const int il = lane % 32, hl = lane / 32;
+    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // hidden channel (within a block of 32) that element j of reduction group `half` of lane half hl holds
+    auto hperm = [](int half, int hl_, int j) { return 16 * half + 8 * (j / 4) + 4 * hl_ + j % 4; };
+
+    for (int i = t; i < MH * KC * 512; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, s = (i / 512) % KC, mh = i / (512 * KC);
+        f1w[i] = Wup[(16 * s + 8 * (l / 32) + j) * H + 32 * mh + l % 32];
+    }
+    for (int i = t; i < MH * KC * 64; i += kMlpThreads) {
+        const int l = i % 64, s = (i / 64) % KC, mh = i / (64 * KC);
+        reinterpret_cast<half8_t*>(smem + Cfg::F2_OFF)[i] = load_c8(Wdown + (32 * mh + l % 32) * C + 16 * s + 8 * (l / 32));
+    }
+    for (int i = t; i < 2 * MH * 512; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, f = i / 512;
+        const int c = l % 32, h = 32 * (f / 2) + hperm(f % 2, l / 32, j);
+        f3w[i] = c < C ? Wup[c * H + h] : (half_t)0;
+    }
+    for (int i = t; i < 2 * 512; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, half = i / 512;
+        ipw[i] = hperm(half, l / 32, j) == l % 32 ? (half_t)1 : (half_t)0;
+    }
+    for (int i = t; i < KC * 512; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, s = i / 512;
+        idw[i] = 16 * s + 8 * (l / 32) + j == l % 32 ? (half_t)1 : (half_t)0;
+    }
+    for (int i = t; i < H; i += kMlpThreads) bsh[i] = bias[i];
+    __syncthreads();
+
+    const half8_t* f1 = reinterpret_cast<const half8_t*>(smem + Cfg::F1_OFF) + lane;
+    const half8_t* f2 = reinterpret_cast<const half8_t*>(smem + Cfg::F2_OFF) + lane;
+    const half8_t* f3 = reinterpret_cast<const half8_t*>(smem + Cfg::F3_OFF) + lane;
+    const half8_t* ip = reinterpret_cast<const half8_t*>(smem + Cfg::IP_OFF) + lane;
+    const half8_t* id = reinterpret_cast<const half8_t*>(smem + Cfg::ID_OFF) + lane;
+    half_t* my = reinterpret_cast<half_t*>(smem + Cfg::DS_OFF) + wave * 32 * DP;
+
+    float16_t wdn[MH], wup[MH];  // dWdown block: D[h][c];  dWup block: D[c][h]
+    float bacc[MH];
+#pragma unroll
+    for (int mh = 0; mh < MH; ++mh) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wdn[mh][i] = wup[mh][i] = 0.0f;
+        bacc[mh] = 0.0f;
+    }
+
+    const int64_t ntiles = (V + 31) / 32;
+    const int64_t stride = (int64_t)gridDim.x * kMlpWaves;
+    half8_t xn[KC], gn[KC];
+    auto fetch = [&](int64_t tile) {  // rows past V read the last voxel and are zeroed before use
+        int64_t v = tile * 32 + il;
+        v = v < V ? v : V - 1;
+#pragma unroll
+        for (int s = 0; s < KC; ++s) {
+            xn[s] = load_c8_nt(x + v * C + 16 * s + 8 * hl);
+            gn[s] = load_c8_nt(g + v * C + 16 * s + 8 * hl);
+        }
+    };
+
+    // dx leaves one tile late: the wait for the operands of a tile then only covers stores issued a whole
+    // tile earlier (the memory counter retires loads and stores in issue order)
+    auto flush = [&](int64_t pv0, bool ragged) {
+#pragma unroll
+        for (int c0 = 0; c0 < 32 * C / 8; c0 += kWave) {
+            const int c = c0 + lane;
+            const int row = c / (C / 8), cc = c % (C / 8);
+            if (!ragged || pv0 + row < V) {
+                const half4_t lo = *reinterpret_cast<const half4_t*>(my + row * DP + cc * 8);
+                const half4_t hi = *reinterpret_cast<const half4_t*>(my + row * DP + cc * 8 + 4);
+                const half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                store_c8_nt(dx + (pv0 + row) * C + cc * 8, o);
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    const int64_t first = (int64_t)blockIdx.x * kMlpWaves + wave;
+    int64_t tile = first;
+    if (tile < ntiles) fetch(tile);
+    for (; tile < ntiles; tile += stride) {
+        const int64_t v0 = tile * 32;
+        half8_t xc[KC], gc[KC];
+#pragma unroll
+        for (int s = 0; s < KC; ++s) {
+            xc[s] = xn[s];
+            gc[s] = gn[s];
+        }
+        if (v0 + 32 > V) {  // ragged last tile (wavefront-uniform)
+            const bool ok = v0 + il < V;
+#pragma unroll
+            for (int s = 0; s < KC; ++s) {
+                xc[s] = ok ? xc[s] : z8;
+                gc[s] = ok ? gc[s] : z8;
+            }
+        }
+        if (tile != first) flush(v0 - stride * 32, false);  // an earlier tile of this wavefront is never ragged
+        {
+            const int64_t nt = tile + stride;
+            fetch(nt < ntiles ? nt : tile);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // x^T, g^T: lane = channel, registers = voxels 8 (i/4) + 4 hl + i%4
+        half8_t xT[2], gT[2];
+        {
+            float16_t tx, tg;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tx[i] = tg[i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KC; ++s) {
+                const half8_t e = id[s * 64];
+                tx = __builtin_amdgcn_mfma_f32_32x32x16_f16(xc[s], e, tx, 0, 0, 0);
+                tg = __builtin_amdgcn_mfma_f32_32x32x16_f16(gc[s], e, tg, 0, 0, 0);
+            }
+            pack_acc(tx, xT[0], xT[1]);
+            pack_acc(tg, gT[0], gT[1]);
+        }
+
+        float16_t dacc;  // dx^T: D[c][v]
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dacc[i] = 0.0f;
+
+#pragma unroll
+        for (int mh = 0; mh < MH; ++mh) {
+            float16_t up, dn;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) up[i] = dn[i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KC; ++s) {
+                up = __builtin_amdgcn_mfma_f32_32x32x16_f16(f1[(mh * KC + s) * 64], xc[s], up, 0, 0, 0);
+                dn = __builtin_amdgcn_mfma_f32_32x32x16_f16(f2[(mh * KC + s) * 64], gc[s], dn, 0, 0, 0);
+            }
+            // up[i], dn[i]: hidden channel 32 mh + 8 (i/4) + 4 hl + i%4 of voxel il
+            half8_t hv[2], lv[2];
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const half4_t b4 = *reinterpret_cast<const half4_t*>(bsh + 32 * mh + 8 * gq + 4 * hl);
+#pragma unroll
+                for (int jp = 0; jp < 2; ++jp) {
+                    const int i = 4 * gq + 2 * jp, e = 4 * (gq % 2) + 2 * jp;
+                    half2_t hid, lg;
+                    hid_lg_pair(up[i], up[i + 1], dn[i], dn[i + 1], half2_t{b4[2 * jp], b4[2 * jp + 1]}, hid, lg);
+                    hv[gq / 2][e] = hid[0];
+                    hv[gq / 2][e + 1] = hid[1];
+                    lv[gq / 2][e] = lg[0];
+                    lv[gq / 2][e + 1] = lg[1];
+                }
+            }
+            // rows past V hold x = g = 0: hid = relu(bias) there meets g = 0 in dWdown, lg = 0 everywhere else
+            dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(f3[(2 * mh) * 64], lv[0], dacc, 0, 0, 0);
+            dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(f3[(2 * mh + 1) * 64], lv[1], dacc, 0, 0, 0);
+
+            // hid^T, lg^T: lane = hidden channel 32 mh + il, registers = voxels
+            half8_t hT[2], lT[2];
+            {
+                float16_t th, tl;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) th[i] = tl[i] = 0.0f;
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    const half8_t e = ip[hf * 64];
+                    th = __builtin_amdgcn_mfma_f32_32x32x16_f16(hv[hf], e, th, 0, 0, 0);
+                    tl = __builtin_amdgcn_mfma_f32_32x32x16_f16(lv[hf], e, tl, 0, 0, 0);
+                }
+                pack_acc(th, hT[0], hT[1]);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) bacc[mh] += tl[i];
+                pack_acc(tl, lT[0], lT[1]);
+            }
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                wdn[mh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hT[hf], gT[hf], wdn[mh], 0, 0, 0);
+                wup[mh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xT[hf], lT[hf], wup[mh], 0, 0, 0);
+            }
+        }
+
+        // ---- dx: into the wavefront's own LDS tile; the LDS operations of one wavefront complete in issue
+        // order, so no workgroup barrier is needed ----
+#pragma unroll
+        for (int gq = 0; gq < C / 8; ++gq) {
+            half4_t o;
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)dacc[4 * gq + jj];
+            *reinterpret_cast<half4_t*>(my + il * DP + 8 * gq + 4 * hl) = o;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if (first < ntiles) flush((tile - stride) * 32, true);
+
+    // ---- the four wavefronts add their partials in LDS, wavefront 0 first: [dWup C*H][dWdown H*C][dbias H] ----
+    float* red = reinterpret_cast<float*>(smem);
+    __syncthreads();  // every wavefront is done with the fragments
+#pragma unroll 1
+    for (int w = 0; w < kMlpWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int mh = 0; mh < MH; ++mh) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int ri = 8 * (i / 4) + 4 * hl + i % 4;  // row of the block held in register i
+                    if (il < C) {  // dWdown[h = 32 mh + ri][c = il]
+                        float* p = red + C * H + (32 * mh + ri) * C + il;
+                        *p = w == 0 ? wdn[mh][i] : *p + wdn[mh][i];
+                    }
+                    if (ri < C) {  // dWup[c = ri][h = 32 mh + il]
+                        float* p = red + ri * H + 32 * mh + il;
+                        *p = w == 0 ? wup[mh][i] : *p + wup[mh][i];
+                    }
+                }
+                const float b = bacc[mh] + __shfl_xor(bacc[mh], 32);  // both lane halves hold 16 voxels each
+                if (hl == 0) {
+                    float* p = red + 2 * C * H + 32 * mh + il;
+                    *p = w == 0 ? b : *p + b;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = ws + (int64_t)blockIdx.x * Cfg::RW;
+    for (int i = t; i < Cfg::RW; i += kMlpThreads) out[i] = red[i];
+}
+
 // sums the rows of the partial buffer in a fixed order and scatters the three results
 __global__ __launch_bounds__(256) void mlp_reduce_kernel(const float* __restrict__ ws, int nrows, int RW, int n_up,
                                                          int n_down, float* __restrict__ d_up,
@@ -496,14 +807,20 @@ __global__ __launch_bounds__(256) void mlp_reduce_kernel(const float* __restrict
     }
 }
 
-static int mb_blocks(int64_t V)
+// workgroups and partial rows per workgroup
+static int mb_blocks(int64_t V, int C)
 {
+    if (C <= 32) {  // wavefront-per-tile kernel: as many workgroups per compute unit as its registers allow
+        const int64_t ntiles = (V + 31) / 32;
+        return (int)std::max<int64_t>(1, std::min<int64_t>((ntiles + kMlpWaves - 1) / kMlpWaves, C == 16 ? 768 : 512));
+    }
     const int64_t ntiles = (V + kMbTile - 1) / kMbTile;
     return (int)std::max<int64_t>(1, std::min<int64_t>(ntiles, 512));
 }
 
 static int mb_kspl(int C)
 {
+    if (C <= 32) return 1;
     const int nu = 2 * (2 * C / 32) * ((C + 31) / 32);
     return nu >= kMlpWaves ? 1 : kMlpWaves / nu;
 }
@@ -520,7 +837,7 @@ extern "C" int64_t kerops_lin_brelu_lin_bwd_workspace_bytes(int64_t V, int32_t C
         set_error("lin_brelu_lin_bwd: built for C in {16,32,64} (got %d)", C);
         return KEROPS_E_UNSUPPORTED_C;
     }
-    return (int64_t)mb_blocks(V) * mb_kspl(C) * (4 * C * C + 2 * C) * (int64_t)sizeof(float);
+    return (int64_t)mb_blocks(V, C) * mb_kspl(C) * (4 * C * C + 2 * C) * (int64_t)sizeof(float);
 }
 
 extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const void* Wup, const void* Wdown,
@@ -540,9 +857,24 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
                   (long long)workspace_bytes);
         return KEROPS_E_WORKSPACE;
     }
-    const int blocks = mb_blocks(V);
+    const int blocks = mb_blocks(V, C);
     hipStream_t s = (hipStream_t)stream;
     float* ws = (float*)workspace;
+#define KEROPS_MT_CASE(CV)                                                                                        \
+    if (C == CV) {                                                                                                \
+        hipLaunchKernelGGL((lin_brelu_lin_bwd_wave_kernel<CV>), dim3(blocks), dim3(kMlpThreads), 0, s,           \
+                           (const half_t*)x, (const half_t*)g, (const half_t*)Wup, (const half_t*)Wdown,         \
+                           (const half_t*)bias, (half_t*)dx, ws, V);                                             \
+        int rc = check_launch("lin_brelu_lin_bwd");                                                               \
+        if (rc != KEROPS_OK) return rc;                                                                           \
+        const int RW = MtCfg<CV>::RW;                                                                             \
+        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(256), 0, s, ws, blocks, RW,           \
+                           2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);                                        \
+        return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
+    }
+    KEROPS_MT_CASE(16)
+    KEROPS_MT_CASE(32)
+#undef KEROPS_MT_CASE
 #define KEROPS_MB_CASE(CV)                                                                                        \
     if (C == CV) {                                                                                                \
         hipLaunchKernelGGL((lin_brelu_lin_bwd_kernel<CV>), dim3(blocks), dim3(kMlpThreads), 0, s,                \
@@ -555,8 +887,6 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
                            blocks * MbCfg<CV>::KSPL, RW, 2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);          \
         return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
     }
-    KEROPS_MB_CASE(16)
-    KEROPS_MB_CASE(32)
     KEROPS_MB_CASE(64)
 #undef KEROPS_MB_CASE
     set_error("lin_brelu_lin_bwd: built for C in {16,32,64} (got %d)", C);

@@ -162,6 +162,50 @@ def test_lin_brelu_lin_backward_matches_oracle(c, spatial):
                               rtol_narrow=1e-3, atol_narrow=4e-3)
 
 
+@pytest.mark.parametrize('c', [16, 32])
+def test_lin_brelu_lin_backward_several_tiles_per_wavefront(c):
+    # more 32-voxel tiles than resident wavefronts, ragged end: the loop-carried prefetch, the store of a tile
+    # one iteration late and the accumulation over tiles are all on the path
+    g = cpu_gen(1000 + c)
+    n, h, w, d = 1, 61, 67, 29
+    x, grad = rand_cl3d(g, n, c, h, w, d), rand_cl3d(g, n, c, h, w, d)
+    Wup, Wdown = rand_pw(g, c, 2 * c), rand_pw(g, 2 * c, c)
+    bias = (torch.randn(2 * c, generator=g) * 0.5).half()
+    dev = [t_.to(DEV) for t_ in (x, grad, Wup, Wdown, bias)]
+    dx, dup, ddn, db = (t_.cpu() for t_ in LinBReLULinBackward(*dev, out_dtype=torch.float32))
+    rdx, rup, rdn, rdb = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
+    assert (dx.float() - rdx.float()).abs().max() <= 2.0 ** -7 * max(1.0, rdx.abs().max().item())
+    same = (dx.contiguous().view(torch.int16) == rdx.contiguous().view(torch.int16)).float().mean().item()
+    assert same > 0.97, same
+    for got, ref in ((dup, rup), (ddn, rdn), (db, rdb)):
+        rel = ((got.double() - ref).norm() / max(ref.norm().item(), 1e-30)).item()
+        assert rel < 1e-3, rel
+
+
+@pytest.mark.parametrize('c', [16, 32, 64])
+def test_lin_brelu_lin_backward_mask_at_zero(c):
+    # linup == 0 exactly (x = 0, bias = +0 or -0) must not pass the gradient, a positive bias must
+    g = cpu_gen(7 + c)
+    n, h, w, d = 1, 5, 6, 7
+    x = torch.zeros(n, c, h, w, d, dtype=torch.float16).contiguous(memory_format=torch.channels_last_3d)
+    grad = rand_cl3d(g, n, c, h, w, d)
+    Wup, Wdown = rand_pw(g, c, 2 * c), rand_pw(g, 2 * c, c)
+    bias = torch.zeros(2 * c, dtype=torch.float16)
+    bias[1::4] = -0.0
+    bias[2::4] = 0.25
+    bias[3::4] = -0.25
+    dev = [t_.to(DEV) for t_ in (x, grad, Wup, Wdown, bias)]
+    dx, dup, ddn, db = (t_.cpu() for t_ in LinBReLULinBackward(*dev, out_dtype=torch.float32))
+    rdx, rup, rdn, rdb = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
+    assert torch.all(db[0::4] == 0) and torch.all(db[1::4] == 0) and torch.all(db[3::4] == 0)
+    assert torch.all(db[2::4] != 0)
+    assert torch.all(dup == 0)  # x = 0
+    assert torch.all(ddn[0::4] == 0) and torch.all(ddn[1::4] == 0) and torch.all(ddn[3::4] == 0)
+    for got, ref in ((ddn, rdn), (db, rdb)):
+        assert ((got.double() - ref).norm() / ref.norm()).item() < 1e-3
+    assert (dx.float() - rdx.float()).abs().max() <= 2.0 ** -7 * max(1.0, rdx.abs().max().item())
+
+
 def test_lin_brelu_lin_backward_defaults_and_determinism():
     g = cpu_gen(41)
     c = 32
