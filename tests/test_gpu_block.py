@@ -206,6 +206,30 @@ def test_lin_brelu_lin_backward_mask_at_zero(c):
     assert (dx.float() - rdx.float()).abs().max() <= 2.0 ** -7 * max(1.0, rdx.abs().max().item())
 
 
+def _spatial_sample(n, seed, max_voxels=200_000):
+    """Deterministic sample of the spatial grid of the reference's linear tests (tests/conftest.py:14-36)."""
+    import random
+    rng = random.Random(seed)
+    extents = [2, 3, 7, 13, 16, 32, 37, 53, 111, 128]
+    out = []
+    while len(out) < n:
+        sp = (rng.choice([1, 2, 3, 4]), rng.choice(extents), rng.choice(extents), rng.choice(extents))
+        if sp[0] * sp[1] * sp[2] * sp[3] <= max_voxels and sp not in out:
+            out.append(sp)
+    return out
+
+
+@pytest.mark.parametrize('spatial', _spatial_sample(12, seed=322))
+@pytest.mark.parametrize('cout', [16, 32])
+def test_linear_family_on_reference_fixture_grid_sample(cout, spatial):
+    # the reference's parameters: 32 input channels, channels_out in {16, 32} (tests/ops/test_linear.py:11-78) and
+    # channels in {16, 32} for the bottleneck block (:81-200)
+    test_relu_linear_add_matches_oracle(32, cout, spatial)
+    test_relu_linear_backward_matches_oracle(32, cout, spatial)
+    test_lin_brelu_lin_add_matches_oracle(cout, spatial)
+    test_lin_brelu_lin_backward_matches_oracle(cout, spatial)
+
+
 def test_lin_brelu_lin_backward_defaults_and_determinism():
     g = cpu_gen(41)
     c = 32

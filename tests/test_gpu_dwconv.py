@@ -65,6 +65,33 @@ def test_dwconv_wgrad_matches_oracle(shape):
                                       rtol_len=1e-3 * shape[0], atol_len=1e-3)
 
 
+def fixture_grid_sample(n, channels, max_voxels, seed):
+    """A deterministic sample of the grid the reference's tests sweep (tests/conftest.py:4-36): batch 1-4, three
+    extents from {2,3,7,13,16,32,37,53,111,128}, bounded so that the oracle stays fast."""
+    import random
+    rng = random.Random(seed)
+    extents = [2, 3, 7, 13, 16, 32, 37, 53, 111, 128]
+    out = []
+    while len(out) < n:
+        shape = (rng.choice([1, 2, 3, 4]), rng.choice(channels), rng.choice(extents), rng.choice(extents),
+                 rng.choice(extents))
+        if shape[0] * shape[2] * shape[3] * shape[4] * shape[1] <= max_voxels * 8 and shape not in out:
+            out.append(shape)
+    return out
+
+
+@pytest.mark.parametrize('shape', fixture_grid_sample(24, [8, 16, 32, 64, 128], 150_000, seed=322))
+def test_reference_fixture_grid_sample(shape):
+    g = cpu_gen(sum(shape))
+    x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    _, wk = rand_dw_weight(g, shape[1])
+    check_fwd(x, wk, DWConv(x.to(DEV), wk.to(DEV)))
+    ref = oracle.dwconv_wgrad(x, grad)
+    gw32 = DWConvWGRAD(x.to(DEV), grad.to(DEV), out_dtype=torch.float32).cpu()
+    rel = ((gw32.double() - ref).norm() / ref.norm()).item()
+    assert rel < 2e-6, rel
+
+
 from kerops_amd.ops.conv.variants import FWD_VARIANTS, WGRAD_VARIANTS as WG_VARIANTS  # noqa: E402
 
 

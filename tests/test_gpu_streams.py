@@ -88,6 +88,45 @@ def test_bnrelu_and_backward(shape):
     assert close64(dW.flatten(), rdW, 1e-5) and close64(dB.flatten(), rdB, 1e-5)
 
 
+def _grid_sample(n, seed):
+    """Deterministic sample of the reference's test grid (tests/conftest.py:4-36): channels {2,4,8,16,32}, batch
+    1-4, extents from {2,3,7,13,16,32,37,53,111,128}; bounded in size."""
+    import random
+    rng = random.Random(seed)
+    extents = [2, 3, 7, 13, 16, 32, 37, 53, 111, 128]
+    out = []
+    while len(out) < n:
+        shape = (rng.choice([1, 2, 3, 4]), rng.choice([2, 4, 8, 16, 32]), rng.choice(extents), rng.choice(extents),
+                 rng.choice(extents))
+        if shape[0] * shape[1] * shape[2] * shape[3] * shape[4] <= 4_000_000 and shape not in out:
+            out.append(shape)
+    return out
+
+
+@pytest.mark.parametrize('shape', _grid_sample(20, seed=322))
+def test_stream_ops_on_reference_fixture_grid_sample(shape):
+    g = cpu_gen(sum(shape))
+    c = shape[1]
+    x, y = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    xd, yd = x.to(DEV), y.to(DEV)
+    mean, sq = Stats(xd)
+    rm, rs = oracle.stats(x)
+    assert close64(mean, rm) and close64(sq, rs)
+    s_, m2, q2 = AddStats(xd, yd)
+    rsum, rm2, rq2 = oracle.add_stats(x, y)
+    assert bits_equal(s_, rsum) and close64(m2, rm2) and close64(q2, rq2)
+    w, b = torch.rand(c, generator=g) + 0.5, torch.randn(c, generator=g) * 0.3
+    assert bits_equal(ApplyBNReLU(xd, w.to(DEV), b.to(DEV)), oracle.bnrelu_fwd(x, w, b))
+    assert bits_equal(ApplyBNReLUBackward(xd, w.to(DEV), b.to(DEV), yd)[0], oracle.bnrelu_bwd(x, w, b, y)[0])
+    pooled, pm, pq = AvgPoolCeilStats(xd)
+    rp, rpm, rpq = oracle.avgpool_ceil_stats(x)
+    assert bits_equal(pooled, rp) and close64(pm, rpm) and close64(pq, rpq)
+    mg, sg = torch.randn(c, generator=g) / 3, torch.randn(c, generator=g) / 3
+    assert bits_equal(StatsBackward(xd, mg.to(DEV), sg.to(DEV)), oracle.stats_bwd(x, mg, sg))
+    q = QuantUint8Window(xd, 3.0)
+    assert torch.equal(q.cpu(), oracle.quant_u8_window(x, 3.0))
+
+
 def test_bn_block_end_to_end_vs_train_mode_batchnorm(golden):
     """Stats -> fold -> ApplyBNReLU as tests/ops/test_bn_relu.py:26-30 of the reference composes
     them, against the golden relu(BatchNorm3d(train)(x)) computed by torch on the CPU."""
