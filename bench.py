@@ -233,6 +233,18 @@ def main():
                                               clone_gbps)
         ops['QuantUint8Window'] = figures(time_op(torch, lambda: QuantUint8Window(x, 3.0), it, wm)[0], 3 * V * C,
                                           clone_gbps)
+        # the vendor path on the same GPU: torch's own depthwise conv3d (MIOpen) on the same tensor, forward only
+        # (its weight gradient takes 2.5 s per call after a 78 s kernel search, so it is not run here)
+        try:
+            import torch.nn.functional as F
+            wt_t = wk.permute(3, 0, 1, 2).unsqueeze(1).contiguous()
+            t_ms = time_op(torch, lambda: F.conv3d(x, wt_t, None, 1, 1, 1, C), 3, 1)[0]
+            ops['gpu_torch_conv3d_groups'] = {'fwd_ms': round(t_ms, 2), 'vs_DWConv': round(t_ms / fwd['ms'], 1),
+                                              'note': 'torch.nn.functional.conv3d(groups=C), fp16 channels_last_3d, '
+                                                      'same tensor, same GPU; median of 3 after 1 warm-up'}
+            del wt_t
+        except Exception as e:  # a reported side figure only
+            ops['gpu_torch_conv3d_groups'] = {'error': repr(e)[:200]}
         table = {}
         for c in (8, 16, 32, 64, 128):
             if c == C:
