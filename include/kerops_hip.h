@@ -60,6 +60,18 @@ int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int
                           int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk, int32_t lane_channels,
                           void* stream);
 
+/* Depthwise convolution as above plus the per-channel batch statistics of its output in the same pass
+ * (an addition, no single reference counterpart: it stands for kerops_dwconv_fwd_f16 followed by
+ * kerops_stats_f16 on y, i.e. kerops/ops/conv/dwconv.py:20-63 then kerops/ops/stats.py:11-38, and saves the
+ * second pass over y):
+ *   mean[c] = sum y / (N*H*W*D),  sqmean[c] = sum y*y / (N*H*W*D),  y as stored (fp16), fp32 sums per
+ *   workgroup in the workspace, added in a fixed order in fp64 by a second kernel (deterministic).
+ * Runs the matrix-core kernel at its built-in launch shape.  C in {8,16,32,64,128}. */
+int64_t kerops_dwconv_stats_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C);
+int kerops_dwconv_stats_f16(const void* x, const void* wt, void* y, float* mean, float* sqmean, void* workspace,
+                            int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
+                            void* stream);
+
 /* Depthwise weight gradient, fp32 end to end:
  *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]
  * gw is [3][3][3][C] fp32.  Deterministic: per-workgroup partials go to the

@@ -29,6 +29,8 @@ SIGNATURES = {
     'kerops_hip_version': (ctypes.c_int, []),
     'kerops_last_error_string': (ctypes.c_char_p, []),
     'kerops_dwconv_fwd_f16': (ctypes.c_int, [_p, _p, _p, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _p]),
+    'kerops_dwconv_stats_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32]),
+    'kerops_dwconv_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_dwconv_bwd_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_dwconv_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_dwconv_wgrad_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),

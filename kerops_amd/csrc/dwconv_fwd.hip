@@ -15,6 +15,8 @@
 // reads are consecutive words (conflict free).  The weights of the thread's channels stay
 // packed as fp16 pairs in registers; products are formed by the 2-way fp16 dot
 // instruction and mixed-precision FMA, both accumulating in fp32.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace kerops {
@@ -54,6 +56,7 @@ struct FwdArgs {
     const half_t* pw;   // [C][cout]
     half_t* y2;         // [N][H][W][D][cout]
     float* amax_ws;     // one max|y2| per workgroup
+    float* stats_ws;    // mode 3: per workgroup [2][slab channels] sums of y and y*y (y as stored, fp16)
     int H, W, D, C;
     int n_wt, n_dt, n_hc, n_slab, h_chunk;
     uint32_t nblocks;
@@ -450,7 +453,9 @@ struct FmCfg {
     static_assert(TW % RSPLIT == 0, "rows split evenly");
 };
 
-// MODE 0: y = conv; 1: y = max(conv * scale + shift, 0); 2: that result (fp16) goes through an LDS tile into the
+// MODE 0: y = conv; 3: the same plus per-channel sums of y and y*y over the workgroup's outputs (the statistics pass
+// of a following batch norm, taken from the registers that hold the rounded outputs); 1: y = max(conv * scale +
+// shift, 0); 2: that result (fp16) goes through an LDS tile into the
 // pointwise GEMM [TW*TD positions][C] x [C][COUT] on the 32x32x16 matrix instruction (the product is computed
 // transposed as in pointwise_kernel, a wavefront owns 32 positions x 32 output channels; pw^T sits in LDS), the
 // [positions][COUT] result is bounced through LDS and stored as 16-byte chunks with the running max|y| fused in.
@@ -459,7 +464,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, XSLOT = Cfg::XSLOT, NLDX = Cfg::NLDX;
-    constexpr bool EPI = MODE >= 1;
+    constexpr bool EPI = MODE == 1 || MODE == 2;
+    constexpr bool STATS = MODE == 3;
     // fused pointwise stage: t tile [NPOS][SC + 8] fp16 and y tile [NPOS][COUT + 4] fp16 behind the staging buffers
     constexpr int NPOS = Cfg::TW * TD, RT = SC + 8, RY = COUT + 4;
     constexpr int KS = SC / 16, MT = COUT / 32, NPT = NPOS / 32;  // k = 16 per matrix instruction
@@ -607,6 +613,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     for (int o = 0; o < RO; ++o)
 #pragma unroll
         for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float ssum[2] = {0.0f, 0.0f}, ssq[2] = {0.0f, 0.0f};  // mode 3: this lane's channel pair
 
     // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
     // They are unconditional (plane indices are clamped; planes that do not exist are never used):
@@ -667,6 +674,16 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
                     float f = T[o][e][2];
                     if (EPI) f = fmaxf(__builtin_fmaf(f, esc[e], esh[e]), 0.0f);
                     v[e] = (half_t)f;
+                }
+                if constexpr (STATS) {
+                    if (oval[o]) {  // positions of the patch outside the volume hold values but are not outputs
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            const float f = (float)v[e];
+                            ssum[e] += f;
+                            ssq[e] += f * f;
+                        }
+                    }
                 }
                 if constexpr (MODE == 2) {
                     *reinterpret_cast<half2_t*>(tt + ((ra + o) * TD + pgrp + rr) * RT + half * 32 + 2 * q) = v;
@@ -746,6 +763,35 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
         __syncthreads();
         flush_row(parity ^ 1);
     }
+    if constexpr (STATS) {
+        // lanes of a wavefront that share the channel pair differ in rr (lane bits 0-1) and sub (the bits above q)
+        float v4[4] = {ssum[0], ssum[1], ssq[0], ssq[1]};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v4[i] += __shfl_xor(v4[i], 1);
+            v4[i] += __shfl_xor(v4[i], 2);
+#pragma unroll
+            for (int m = 4 * NQ; m < kWave; m <<= 1) v4[i] += __shfl_xor(v4[i], m);
+        }
+        __syncthreads();  // the staging buffers are free now
+        float* sred = reinterpret_cast<float*>(smem);  // [wavefront][2 NQ channels][sum, sum of squares]
+        if (rr == 0 && sub == 0) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                sred[(wave * 2 * NQ + 2 * q + e) * 2 + 0] = v4[e];
+                sred[(wave * 2 * NQ + 2 * q + e) * 2 + 1] = v4[2 + e];
+            }
+        }
+        __syncthreads();
+        if (t < 2 * SC) {  // wavefronts that share a half of the slab, in a fixed order
+            const int st = t / SC, ch = t % SC;
+            const int hf = ch / (2 * NQ), cl = ch % (2 * NQ);
+            float acc = 0.0f;
+#pragma unroll
+            for (int pp = 0; pp < Cfg::NPART; ++pp) acc += sred[((pp * Cfg::NHALF + hf) * 2 * NQ + cl) * 2 + st];
+            a.stats_ws[(int64_t)wg_slot * 2 * SC + st * SC + ch] = acc;
+        }
+    }
     if constexpr (MODE == 2) {
         amax = wave_max(amax);
         if (lane == 0) amax_red[wave] = amax;
@@ -802,6 +848,44 @@ static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t 
                            a);
     }
     return check_launch("dwconv_fwd");
+}
+
+// Adds the per-workgroup sums of one channel in a fixed order (fp64) and divides by the number of voxels:
+// one workgroup per (statistic, channel); row r of the workspace belongs to slab r % n_slab.
+__global__ __launch_bounds__(256) void dwconv_stats_reduce_kernel(const float* __restrict__ ws, uint32_t nblocks,
+                                                                  int n_slab, int SC, double inv_count,
+                                                                  float* __restrict__ mean, float* __restrict__ sqmean)
+{
+    __shared__ double part[256];
+    const int C = n_slab * SC;
+    const int st = blockIdx.x / C, c = blockIdx.x % C;
+    const int slab = c / SC, ch = c % SC;
+    double s = 0.0;
+    for (uint32_t r = slab + (uint32_t)n_slab * threadIdx.x; r < nblocks; r += (uint32_t)n_slab * 256)
+        s += (double)ws[(int64_t)r * 2 * SC + st * SC + ch];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) part[threadIdx.x] += part[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) (st == 0 ? mean : sqmean)[c] = (float)(part[0] * inv_count);
+}
+
+// launch shape of the convolution + statistics kernel for a channel count (the default shapes of dwconv_fwd_run)
+template <class F>
+static int with_stats_shape(int C, F&& f)
+{
+    switch (C >= 64 ? 8 : C / 8) {
+        case 1: return f(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{},
+                         std::integral_constant<int, 32>{}, std::integral_constant<int, 256>{});
+        case 2: return f(std::integral_constant<int, 2>{}, std::integral_constant<int, 8>{},
+                         std::integral_constant<int, 32>{}, std::integral_constant<int, 512>{});
+        case 4: return f(std::integral_constant<int, 4>{}, std::integral_constant<int, 8>{},
+                         std::integral_constant<int, 16>{}, std::integral_constant<int, 512>{});
+        default: return f(std::integral_constant<int, 8>{}, std::integral_constant<int, 8>{},
+                          std::integral_constant<int, 8>{}, std::integral_constant<int, 512>{});
+    }
 }
 
 template <int CG, int TW, int TD, int CL, int WPE, int NT = 256>
@@ -969,6 +1053,78 @@ int dwsep_fused_run(const void* x, const void* wt, const float* scale, const flo
     return check_launch("dwsep_block");
 }
 }  // namespace kerops
+
+static int dwconv_stats_check(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C)
+{
+    if (N <= 0 || H <= 0 || W <= 0 || D <= 0) {
+        set_error("dwconv_stats: non-positive extent");
+        return KEROPS_E_BADARG;
+    }
+    if ((int64_t)W * D * C >= (1LL << 31)) {
+        set_error("dwconv_stats: one (W,D,C) plane must stay below 2^31 elements");
+        return KEROPS_E_BADARG;
+    }
+    if (!(C == 8 || C == 16 || C == 32 || C == 64 || C == 128)) {
+        set_error("dwconv_stats: unsupported channel count %d", C);
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    return KEROPS_OK;
+}
+
+extern "C" int64_t kerops_dwconv_stats_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C)
+{
+    int rc = dwconv_stats_check(N, H, W, D, C);
+    if (rc != KEROPS_OK) return rc;
+    FwdArgs a{};
+    a.H = H;
+    a.W = W;
+    a.D = D;
+    a.C = C;
+    rc = with_stats_shape(C, [&](auto cg, auto tw, auto td, auto nt) {
+        return plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0);
+    });
+    if (rc != KEROPS_OK) return rc;
+    return (int64_t)a.nblocks * 2 * std::min(C, 64) * (int64_t)sizeof(float);
+}
+
+extern "C" int kerops_dwconv_stats_f16(const void* x, const void* wt, void* y, float* mean, float* sqmean,
+                                       void* workspace, int64_t workspace_bytes, int32_t N, int32_t H, int32_t W,
+                                       int32_t D, int32_t C, void* stream)
+{
+    const int64_t need = kerops_dwconv_stats_workspace_bytes(N, H, W, D, C);
+    if (need < 0) return (int)need;
+    if (!x || !wt || !y || !mean || !sqmean || !aligned16(x) || !aligned16(wt) || !aligned16(y)) {
+        set_error("dwconv_stats: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
+        set_error("dwconv_stats: workspace of %lld bytes required, %lld given", (long long)need,
+                  (long long)workspace_bytes);
+        return KEROPS_E_WORKSPACE;
+    }
+    FwdArgs a{};
+    a.x = (const half_t*)x;
+    a.wt = (const half_t*)wt;
+    a.y = (half_t*)y;
+    a.stats_ws = (float*)workspace;
+    a.H = H;
+    a.W = W;
+    a.D = D;
+    a.C = C;
+    hipStream_t s = (hipStream_t)stream;
+    int rc = with_stats_shape(C, [&](auto cg, auto tw, auto td, auto nt) {
+        using Cfg = FmCfg<cg(), tw(), td(), nt()>;
+        int r = plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0);
+        if (r != KEROPS_OK) return r;
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+        return check_launch("dwconv_stats");
+    });
+    if (rc != KEROPS_OK) return rc;
+    const double inv_count = 1.0 / ((double)N * H * W * D);
+    hipLaunchKernelGGL(dwconv_stats_reduce_kernel, dim3(2 * C), dim3(256), 0, s, (const float*)workspace, a.nblocks,
+                       a.n_slab, std::min(C, 64), inv_count, mean, sqmean);
+    return check_launch("dwconv_stats_reduce");
+}
 
 extern "C" int kerops_dwconv_fwd_f16(const void* x, const void* wt, void* y, int32_t N, int32_t H, int32_t W,
                                      int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,

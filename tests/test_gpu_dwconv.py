@@ -10,7 +10,7 @@ import torch
 
 import oracle
 from conftest import cpu_gen, from_bits, rand_cl3d, rand_dw_weight
-from kerops_amd.ops.conv import DWConv, DWConvWGRAD
+from kerops_amd.ops.conv import DWConv, DWConvStats, DWConvWGRAD
 from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
 
 pytestmark = pytest.mark.gpu
@@ -63,6 +63,22 @@ def test_dwconv_wgrad_matches_oracle(shape):
     if ref.abs().max() < 6e4:
         assert weight_grad_similarity(ref.float(), gw16.float(), rtol_cos=1e-4, atol_cos=1e-4,
                                       rtol_len=1e-3 * shape[0], atol_len=1e-3)
+
+
+@pytest.mark.parametrize('shape', SHAPES + [(1, 64, 40, 70, 33), (2, 16, 30, 64, 64), (1, 8, 50, 40, 64)])
+def test_dwconv_stats_equals_dwconv_then_stats(shape):
+    g = cpu_gen(5)
+    x = rand_cl3d(g, *shape) * 1.5 + 0.25
+    _, wk = rand_dw_weight(g, shape[1])
+    xd, wd = x.to(DEV), wk.to(DEV)
+    y, mean, sq = DWConvStats(xd, wd)
+    assert torch.equal(y, DWConv(xd, wd))  # same kernel body, same rounding
+    assert mean.dtype == sq.dtype == torch.float32 and mean.shape == sq.shape == (shape[1],)
+    rm, rs = oracle.stats(y.cpu())  # the statistics of the tensor as stored
+    assert torch.allclose(mean.cpu().double(), rm, rtol=2e-6, atol=2e-6)
+    assert torch.allclose(sq.cpu().double(), rs, rtol=2e-6, atol=2e-6)
+    y2, mean2, sq2 = DWConvStats(xd, wd)
+    assert torch.equal(mean, mean2) and torch.equal(sq, sq2)  # fixed summation order
 
 
 def fixture_grid_sample(n, channels, max_voxels, seed):
