@@ -228,6 +228,9 @@ def main():
         ops['ApplyBNReLU+AvgPoolCeilStats_fused'] = figures(
             time_op(torch, lambda: ApplyBNReLUAvgPoolCeilStats(x, Wv, Bv), it, wm)[0], 2 * V * C * (1 + 1 / 8),
             clone_gbps)
+        from kerops_amd.ops.conv import DWConvStats
+        ops['DWConv+Stats_fused'] = figures(time_op(torch, lambda: DWConvStats(x, wk), it, wm)[0], 4 * V * C, clone_gbps)
+        ops['DWConv+Stats_fused']['note'] = 'replaces DWConv + Stats on its output (fwd.ms + ops.Stats.ms)'
         from kerops_amd.ops.conv import DWConvBackward
         ops['DWConvBackward_fused'] = figures(time_op(torch, lambda: DWConvBackward(x, g, wk), it, wm)[0], 6 * V * C,
                                               clone_gbps)

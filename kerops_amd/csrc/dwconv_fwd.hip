@@ -681,7 +681,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
                         for (int e = 0; e < 2; ++e) {
                             const float f = (float)v[e];
                             ssum[e] += f;
-                            ssq[e] += f * f;
+                            ssq[e] = __builtin_fmaf(f, f, ssq[e]);  // f * f is exact in fp32: same result as mul + add
                         }
                     }
                 }
