@@ -55,6 +55,19 @@ def test_argument_validation_needs_no_device():
     assert rc == _lib.KEROPS_E_BADARG and 'dtype' in _lib.last_error()
 
 
+def test_every_entry_point_rejects_null_pointers_before_touching_the_device():
+    # all pointers null, all sizes a plausible 16 / 1.0: every compute entry point must come back with an error
+    # code and a message (no launch, no dereference), so that a caller's mistake never reaches the GPU
+    lib = _lib.load()
+    for name, (res, argtypes) in _lib.SIGNATURES.items():
+        if res is not ctypes.c_int or not any(a is ctypes.c_void_p for a in argtypes):
+            continue
+        args = [None if a is ctypes.c_void_p else (1.0 if a is ctypes.c_float else 16) for a in argtypes]
+        rc = getattr(lib, name)(*args)
+        assert rc in (_lib.KEROPS_E_BADARG, _lib.KEROPS_E_UNSUPPORTED_C, _lib.KEROPS_E_WORKSPACE), (name, rc)
+        assert _lib.last_error(), name
+
+
 def test_workspace_queries():
     lib = _lib.load()
     assert lib.kerops_stats_workspace_bytes(1000, 64, 16) == 16 * 2 * 64 * 4
