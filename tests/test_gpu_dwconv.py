@@ -81,6 +81,24 @@ def test_dwconv_stats_equals_dwconv_then_stats(shape):
     assert torch.equal(mean, mean2) and torch.equal(sq, sq2)  # fixed summation order
 
 
+@pytest.mark.parametrize('shape', [(1, 8, 1, 1, 1), (1, 16, 1, 5, 1), (2, 64, 4, 1, 9), (1, 32, 1, 1, 70), (3, 128, 1, 2, 1),
+                                   (1, 8, 300, 1, 1)])
+def test_extents_of_one(shape):
+    # below the smallest extent of the reference's grid (2): whole taps fall outside the volume
+    g = cpu_gen(11)
+    x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    _, wk = rand_dw_weight(g, shape[1])
+    check_fwd(x, wk, DWConv(x.to(DEV), wk.to(DEV)))
+    ref = oracle.dwconv_wgrad(x, grad)
+    gw32 = DWConvWGRAD(x.to(DEV), grad.to(DEV), out_dtype=torch.float32).cpu()
+    assert ((gw32.double() - ref).norm() / max(ref.norm().item(), 1e-30)).item() < 2e-6
+    assert torch.equal(gw32 == 0, ref == 0)  # taps that never meet the volume stay exactly zero
+    y, mean, sq = DWConvStats(x.to(DEV), wk.to(DEV))
+    rm, rs = oracle.stats(y.cpu())
+    assert torch.allclose(mean.cpu().double(), rm, rtol=2e-6, atol=2e-6)
+    assert torch.allclose(sq.cpu().double(), rs, rtol=2e-6, atol=2e-6)
+
+
 def fixture_grid_sample(n, channels, max_voxels, seed):
     """A deterministic sample of the grid the reference's tests sweep (tests/conftest.py:4-36): batch 1-4, three
     extents from {2,3,7,13,16,32,37,53,111,128}, bounded so that the oracle stays fast."""
