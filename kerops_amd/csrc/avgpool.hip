@@ -166,14 +166,18 @@ static int pool_plan(const char* op, int N, int H, int W, int D, int C, int* blo
         set_error("%s: built for C <= %d (got %d)", op, kMaxReduceChannels, C);
         return KEROPS_E_UNSUPPORTED_C;
     }
+    if (volume_exceeds_i64(N, H, W, D, C)) {
+        set_error("%s: tensor too large", op);
+        return KEROPS_E_BADARG;
+    }
     const int V = C >= 8 ? 8 : C;
     p->N = N;
     p->H = H;
     p->W = W;
     p->D = D;
-    p->Ho = (H + 1) / 2;
-    p->Wo = (W + 1) / 2;
-    p->Do = (D + 1) / 2;
+    p->Ho = ceil_div(H, 2);
+    p->Wo = ceil_div(W, 2);
+    p->Do = ceil_div(D, 2);
     p->C = C;
     p->CG = C / V;
     *nchunks = (int64_t)N * p->Ho * p->Wo * p->Do * p->CG;

@@ -71,10 +71,28 @@ int pointwise_blocks(int64_t V);
 void launch_pw_absmax_final(const float* ws, int n, float* out, hipStream_t s);
 
 // ---- small host helpers -----------------------------------------------------
-static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
-static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+// for a >= 0, b > 0; no intermediate sum, so extents up to the type's maximum are safe
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return a / b + (a % b != 0); }
+static inline int ceil_div(int a, int b) { return a / b + (a % b != 0); }
 static inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// N*H*W*D*C elements (all positive) must be addressable with 64-bit byte offsets; checked before any product
+// of extents is formed in 64 bits
+static inline bool volume_exceeds_i64(int N, int H, int W, int D, int C)
+{
+    const __int128 lim = (__int128)1 << 60;
+    __int128 v = (__int128)N * H * W;  // < 2^93
+    if (v >= lim) return true;
+    v *= D;
+    if (v >= lim) return true;
+    return v * C >= lim;
+}
+// offsets inside one (W, D, C) plane are 32-bit in the convolution kernels (W, D, C positive)
+static inline bool plane_exceeds_i32(int W, int D, int C)
+{
+    const int64_t wd = (int64_t)W * D;  // < 2^62
+    return wd >= (1LL << 31) || wd * C >= (1LL << 31);
+}
 
 // The 8 XCDs of the chip receive workgroups round-robin (workgroup b runs on XCD
 // b % 8) and each XCD has a private L2.  remap_xcd turns the hardware workgroup

@@ -944,7 +944,7 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
         set_error("dwconv_fwd: non-positive extent");
         return KEROPS_E_BADARG;
     }
-    if ((int64_t)W * D * C >= (1LL << 31)) {
+    if (plane_exceeds_i32(W, D, C)) {
         set_error("dwconv_fwd: one (W,D,C) plane must stay below 2^31 elements");
         return KEROPS_E_BADARG;
     }
@@ -1060,7 +1060,7 @@ static int dwconv_stats_check(int32_t N, int32_t H, int32_t W, int32_t D, int32_
         set_error("dwconv_stats: non-positive extent");
         return KEROPS_E_BADARG;
     }
-    if ((int64_t)W * D * C >= (1LL << 31)) {
+    if (plane_exceeds_i32(W, D, C)) {
         set_error("dwconv_stats: one (W,D,C) plane must stay below 2^31 elements");
         return KEROPS_E_BADARG;
     }

@@ -926,7 +926,7 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
         set_error("dwconv_wgrad: unsupported channel count %d", C);
         return KEROPS_E_UNSUPPORTED_C;
     }
-    if ((int64_t)W * D * C >= (1LL << 31)) {
+    if (plane_exceeds_i32(W, D, C)) {
         set_error("dwconv_wgrad: one (W,D,C) plane must stay below 2^31 elements");
         return KEROPS_E_BADARG;
     }
@@ -1031,7 +1031,7 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
         set_error("dwconv_bwd: unsupported channel count %d", C);
         return KEROPS_E_UNSUPPORTED_C;
     }
-    if ((int64_t)W * D * C >= (1LL << 31)) {
+    if (plane_exceeds_i32(W, D, C)) {
         set_error("dwconv_bwd: one (W,D,C) plane must stay below 2^31 elements");
         return KEROPS_E_BADARG;
     }

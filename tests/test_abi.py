@@ -68,6 +68,22 @@ def test_every_entry_point_rejects_null_pointers_before_touching_the_device():
         assert _lib.last_error(), name
 
 
+def test_extreme_sizes_never_reach_a_launch():
+    # sizes up to INT32_MAX with null pointers, and every workspace query over a grid of extreme extents: the
+    # host arithmetic (grid planning, workspace sizes) must neither crash nor report success for a null pointer
+    import itertools
+    lib = _lib.load()
+    for name, (res, argtypes) in _lib.SIGNATURES.items():
+        if 'workspace_bytes' in name:
+            for vals in itertools.product([1, 8, 64, 350, 2 ** 31 - 1], repeat=min(len(argtypes), 5)):
+                n = getattr(lib, name)(*(list(vals) + [0] * (len(argtypes) - len(vals))))
+                assert n >= _lib.KEROPS_E_LAUNCH, (name, vals, n)  # a size or one of the error codes
+        elif res is ctypes.c_int and any(a is ctypes.c_void_p for a in argtypes):
+            for v in (0, 1, 7, 65535, 2 ** 31 - 1):
+                args = [None if a is ctypes.c_void_p else (1.0 if a is ctypes.c_float else v) for a in argtypes]
+                assert getattr(lib, name)(*args) < 0, (name, v)
+
+
 def test_workspace_queries():
     lib = _lib.load()
     assert lib.kerops_stats_workspace_bytes(1000, 64, 16) == 16 * 2 * 64 * 4
