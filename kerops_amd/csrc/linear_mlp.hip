@@ -88,7 +88,11 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_add_kernel(const ha
             if (v >= V) v = V - 1;  // ragged last tile: clamp the read, the write is masked
             half8_t xb[KS1];
 #pragma unroll
-            for (int s = 0; s < KS1; ++s) xb[s] = load_c8_nt(x + v * C + 16 * s + 8 * hl);
+            for (int s = 0; s < KS1; ++s) {
+                // rows of 128 bytes need the cache to hold the line until the row's other loads arrive
+                if constexpr (C <= 32) xb[s] = load_c8_nt(x + v * C + 16 * s + 8 * hl);
+                else xb[s] = load_c8(x + v * C + 16 * s + 8 * hl);
+            }
             // ---- first product, bias, ReLU: the B fragments of the second product ----
             half8_t hb[KS2];
 #pragma unroll

@@ -76,12 +76,16 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
             if (v >= V) v = V - 1;  // ragged last tile: clamp the read, the write is masked
             half8_t xb[KS];
 #pragma unroll
-            for (int q = 0; q < KS; ++q) xb[q] = load_c8(x + v * CIN + 8 * (2 * q + hl));
+            for (int q = 0; q < KS; ++q) {
+                // a load instruction touches 32 bytes of every voxel row: rows of 128 bytes and more need the
+                // cache to hold the line until the row's other loads arrive, so only narrow rows stream
+                if constexpr (CIN <= 32) xb[q] = load_c8_nt(x + v * CIN + 8 * (2 * q + hl));
+                else xb[q] = load_c8(x + v * CIN + 8 * (2 * q + hl));
+            }
             if (RELU_IN) {
+                const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int q = 0; q < KS; ++q)
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) xb[q][j] = xb[q][j] > (half_t)0 ? xb[q][j] : (half_t)0;
+                for (int q = 0; q < KS; ++q) xb[q] = __builtin_elementwise_max(xb[q], z8);  // packed maximum
             }
             float16_t acc[MT];
 #pragma unroll
@@ -108,7 +112,11 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                     }
                 }
         }
-        __syncthreads();
+        // the tile is private to the wavefront and its LDS operations complete in issue order: no workgroup
+        // barrier, the wavefronts of a workgroup run independently
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         if (live) {
 #pragma unroll
             for (int c0 = 0; c0 < Cfg::OUT_CHUNKS; c0 += kWave) {
@@ -120,7 +128,7 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                     half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     const int64_t off = (v0 + row) * COUT + cc * 8;
                     if (HAS_ADD) {
-                        const half8_t a8 = load_c8(add + off);
+                        const half8_t a8 = load_c8_nt(add + off);
 #pragma unroll
                         for (int j = 0; j < 8; ++j) o[j] = (half_t)((float)o[j] + (float)a8[j]);  // fp16 add, RNE
                     }
@@ -128,11 +136,13 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
 #pragma unroll
                         for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf((float)o[j]));
                     }
-                    store_c8(out + off, o);
+                    store_c8_nt(out + off, o);
                 }
             }
         }
-        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
     if (ABSMAX) {
         amax = wave_max(amax);
