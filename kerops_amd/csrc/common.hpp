@@ -87,6 +87,28 @@ static inline bool volume_exceeds_i64(int N, int H, int W, int D, int C)
     if (v >= lim) return true;
     return v * C >= lim;
 }
+// Rows per workgroup of the H-marching convolution kernels.  All workgroups of a launch do the same work, so
+// they run in ceil(workgroups / resident slots) rounds; a workgroup that marches over h rows pays h + 2 plane
+// steps (two halo planes) plus a fixed cost of about `setup` plane steps (prologue, pipeline fill, epilogue).
+// The number of chunks that minimises rounds * (h + 2 + setup) wins; ties go to fewer, longer chunks.
+static inline int pick_h_chunk(int H, int64_t per_plane, int slots, int setup)
+{
+    int best_h = H;
+    double best = 1e300;
+    const int max_chunks = H < 64 ? H : 64;
+    for (int c = 1; c <= max_chunks; ++c) {
+        const int h = ceil_div(H, c);
+        const int chunks = ceil_div(H, h);
+        if (chunks != c) continue;  // the same split as a smaller c
+        const int64_t rounds = ceil_div64(per_plane * chunks, slots);
+        const double cost = (double)rounds * (h + 2 + setup) * (1.0 + 0.004 * c);
+        if (cost < best) {
+            best = cost;
+            best_h = h;
+        }
+    }
+    return best_h;
+}
 // offsets inside one (W, D, C) plane are 32-bit in the convolution kernels (W, D, C positive)
 static inline bool plane_exceeds_i32(int W, int D, int C)
 {

@@ -813,13 +813,9 @@ static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk)
     a.n_wt = ceil_div(a.W, TW);
     a.n_dt = ceil_div(a.D, TD);
     if (h_chunk <= 0) {
-        // about 2.75 workgroups per resident slot (256 CUs x 2 workgroups of 512 threads, or x 4 of 256):
-        // measured best; fewer leave a long tail, more pay the two halo planes of a chunk more often
+        // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each
         const int64_t per_plane = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
-        const int64_t target = NT >= 512 ? 1408 : 2816;
-        const int want_chunks = (int)std::max<int64_t>(1, (target + per_plane / 2) / per_plane);
-        h_chunk = std::max(ceil_div(a.H, want_chunks), std::min(a.H, 24));
-        h_chunk = ceil_div(a.H, ceil_div(a.H, h_chunk));  // equal chunks, no short last one
+        h_chunk = pick_h_chunk(a.H, per_plane, NT >= 512 ? 512 : 1024, 6);
     }
     h_chunk = std::min(h_chunk, a.H);
     a.h_chunk = h_chunk;

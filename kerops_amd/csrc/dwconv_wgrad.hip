@@ -948,14 +948,10 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     p->n_wt = ceil_div(W, tile_w);
     p->n_dt = ceil_div(D, tile_d);
     if (h_chunk <= 0) {
-        // about 2.75 workgroups per resident slot (256 CUs x 2 workgroups of 512 threads, or x 4 of 256);
-        // every workgroup leaves one partial and pays two halo planes, so not more
+        // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each; every workgroup also leaves one partial
         const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
         const bool big_wg = p->cg == 8 && (tile_w * tile_d >= 64);
-        const int64_t target = big_wg ? 1408 : 2816;
-        const int want_chunks = (int)std::max<int64_t>(1, (target + per_plane / 2) / per_plane);
-        h_chunk = std::max(ceil_div(H, want_chunks), std::min(H, 24));
-        h_chunk = ceil_div(H, ceil_div(H, h_chunk));  // equal chunks, no short last one
+        h_chunk = pick_h_chunk(H, per_plane, big_wg ? 512 : 1024, 8);
     }
     p->h_chunk = std::min(h_chunk, H);
     p->n_hc = ceil_div(H, p->h_chunk);
