@@ -867,47 +867,38 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_bwd_mfma_kernel(const WgArg
     }
 }
 
-// Second pass, two small kernels, fixed summation order (deterministic).  The workspace holds one
-// row per (n, h-chunk, w-patch, d-patch) of width RW = slabs*27*SC floats.  Pass 1 sums the rows of
-// each of kRedSeg row segments (64 columns x 4 interleaved row slices per workgroup, coalesced
-// 256-byte reads); pass 2 sums the segments and scatters to the [27][C] layout.
-constexpr int kRedSeg = 32;
-
-__global__ __launch_bounds__(256) void wgrad_reduce1_kernel(const float* __restrict__ ws, float* __restrict__ ws2,
-                                                            int n_rows, int RW, int rows_per_seg)
+// Second pass, fixed summation order (deterministic).  The workspace holds one row per (n, h-chunk, w-patch,
+// d-patch) of width RW = slabs*27*SC floats.  A workgroup owns 16 columns, its 64 row slices sum interleaved rows
+// (four loads in flight), the slices are combined in LDS in a fixed order and the result is scattered to the
+// [27][C] layout.  One launch: at 128^3-class shapes a second small launch was 5 % of the whole op.
+__global__ __launch_bounds__(1024) void wgrad_reduce_kernel(const float* __restrict__ ws, float* __restrict__ gw,
+                                                            int n_rows, int RW, int SC, int C)
 {
-    __shared__ float part[4][64];
-    const int lane_col = threadIdx.x % 64, slice = threadIdx.x / 64;
-    const int col = blockIdx.x * 64 + lane_col;
-    const int seg = blockIdx.y;
-    const int r0 = seg * rows_per_seg, r1 = min(r0 + rows_per_seg, n_rows);
+    __shared__ float part[64][17];
+    const int cl = threadIdx.x % 16, slice = threadIdx.x / 16;
+    const int col = blockIdx.x * 16 + cl;
     float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
     if (col < RW) {
-        int r = r0 + slice;
-        for (; r + 12 < r1; r += 16) {
+        int r = slice;
+        for (; r + 192 < n_rows; r += 256) {
             s0 += ws[(int64_t)r * RW + col];
-            s1 += ws[(int64_t)(r + 4) * RW + col];
-            s2 += ws[(int64_t)(r + 8) * RW + col];
-            s3 += ws[(int64_t)(r + 12) * RW + col];
+            s1 += ws[(int64_t)(r + 64) * RW + col];
+            s2 += ws[(int64_t)(r + 128) * RW + col];
+            s3 += ws[(int64_t)(r + 192) * RW + col];
         }
-        for (; r < r1; r += 4) s0 += ws[(int64_t)r * RW + col];
+        for (; r < n_rows; r += 64) s0 += ws[(int64_t)r * RW + col];
     }
-    part[slice][lane_col] = (s0 + s1) + (s2 + s3);
+    part[slice][cl] = (s0 + s1) + (s2 + s3);
     __syncthreads();
-    if (slice == 0 && col < RW)
-        ws2[(int64_t)seg * RW + col] = (part[0][lane_col] + part[1][lane_col]) + (part[2][lane_col] + part[3][lane_col]);
-}
-
-__global__ __launch_bounds__(256) void wgrad_reduce2_kernel(const float* __restrict__ ws2, float* __restrict__ gw,
-                                                            int nseg, int RW, int SC, int C)
-{
-    const int col = blockIdx.x * 256 + threadIdx.x;
-    if (col >= RW) return;
-    float s = 0.0f;
-    for (int g = 0; g < nseg; ++g) s += ws2[(int64_t)g * RW + col];
-    const int slab = col / (27 * SC), rem = col % (27 * SC);
-    const int tap = rem / SC, cs = rem % SC;
-    gw[tap * C + slab * SC + cs] = s;
+    for (int w = 32; w > 0; w >>= 1) {
+        if (slice < w) part[slice][cl] += part[slice + w][cl];
+        __syncthreads();
+    }
+    if (slice == 0 && col < RW) {
+        const int slab = col / (27 * SC), rem = col % (27 * SC);
+        const int tap = rem / SC, cs = rem % SC;
+        gw[tap * C + slab * SC + cs] = part[0][cl];
+    }
 }
 
 struct WgPlan {
@@ -963,11 +954,11 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     return KEROPS_OK;
 }
 
-// per-workgroup partials followed by the kRedSeg x RW buffer of the second pass
+// per-workgroup partials
 static int64_t wgrad_ws_bytes(const WgPlan& p)
 {
     const int64_t sc = p.cg * 8;
-    return (p.nblocks * 27 * sc + (int64_t)kRedSeg * p.n_slab * 27 * sc) * (int64_t)sizeof(float);
+    return p.nblocks * 27 * sc * (int64_t)sizeof(float);
 }
 
 // the two reduction kernels over the per-workgroup partials [nblocks][27][SC] at the start of ws
@@ -975,15 +966,8 @@ static int reduce_partials(float* ws, const WgPlan& p, int SC, int C, float* gw,
 {
     const int n_rows = (int)(p.nblocks / p.n_slab);
     const int RW = p.n_slab * 27 * SC;
-    const int nseg = std::min(kRedSeg, n_rows);
-    const int rows_per_seg = ceil_div(n_rows, nseg);
-    float* ws2 = ws + p.nblocks * 27 * SC;
-    hipLaunchKernelGGL(wgrad_reduce1_kernel, dim3(ceil_div(RW, 64), nseg), dim3(256), 0, stream, ws, ws2, n_rows, RW,
-                       rows_per_seg);
-    int rc = check_launch("dwconv_wgrad_reduce1");
-    if (rc != KEROPS_OK) return rc;
-    hipLaunchKernelGGL(wgrad_reduce2_kernel, dim3(ceil_div(RW, 256)), dim3(256), 0, stream, ws2, gw, nseg, RW, SC, C);
-    return check_launch("dwconv_wgrad_reduce2");
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, stream, ws, gw, n_rows, RW, SC, C);
+    return check_launch("dwconv_wgrad_reduce");
 }
 
 template <class Cfg, class KernelT>

@@ -89,7 +89,7 @@ def test_workspace_queries():
     assert lib.kerops_stats_workspace_bytes(1000, 64, 16) == 16 * 2 * 64 * 4
     assert lib.kerops_stats_workspace_bytes(1000, 24, 16) == _lib.KEROPS_E_BADARG
     n = lib.kerops_dwconv_wgrad_workspace_bytes(1, 350, 350, 128, 64, 0, 0, 0, 0)
-    assert n > 0 and n % (27 * 64 * 4) == 0  # per-workgroup partials + second-pass buffer
+    assert n > 0 and n % (27 * 64 * 4) == 0  # one [27][64] fp32 partial per workgroup
     assert lib.kerops_dwconv_wgrad_workspace_bytes(1, 8, 8, 8, 24, 0, 0, 0, 0) == _lib.KEROPS_E_UNSUPPORTED_C
     assert lib.kerops_avgpool_ceil_stats_workspace_bytes(1, 7, 7, 7, 8, 4) == 4 * 2 * 8 * 4
     assert lib.kerops_absmax_workspace_bytes(10) == 40
