@@ -34,25 +34,39 @@ extern "C" const char* kerops_last_error_string(void) { return kerops::g_err; }
 
 namespace kerops {
 
-__global__ __launch_bounds__(256) void reduce_rows_kernel(const float* __restrict__ ws, int nrows, int ncols,
-                                                          float* __restrict__ out0, float* __restrict__ out1,
-                                                          int split, double scale)
+// Sums the rows of a partial buffer column by column in a fixed order (fp64) and writes scale * sum to out0
+// (columns below split) or out1.  A workgroup owns 16 columns; its 64 row slices take interleaved rows with four
+// loads in flight each (a single dependent chain over hundreds of rows took longer than the pass it finishes),
+// then the slices are combined by a fixed tree in LDS.
+__global__ __launch_bounds__(1024) void reduce_rows_kernel(const float* __restrict__ ws, int nrows, int ncols,
+                                                           float* __restrict__ out0, float* __restrict__ out1,
+                                                           int split, double scale)
 {
-    __shared__ double part[16][17];
+    __shared__ double part[64][17];
     const int lo = threadIdx.x % 16;
     const int sl = threadIdx.x / 16;
     const int j = blockIdx.x * 16 + lo;
-    double s = 0.0;
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
     if (j < ncols) {
-        for (int r = sl; r < nrows; r += 16) s += (double)ws[(int64_t)r * ncols + j];
+        int r = sl;
+        for (; r + 192 < nrows; r += 256) {
+            const float a = ws[(int64_t)r * ncols + j], b = ws[(int64_t)(r + 64) * ncols + j];
+            const float c = ws[(int64_t)(r + 128) * ncols + j], d = ws[(int64_t)(r + 192) * ncols + j];
+            s0 += (double)a;
+            s1 += (double)b;
+            s2 += (double)c;
+            s3 += (double)d;
+        }
+        for (; r < nrows; r += 64) s0 += (double)ws[(int64_t)r * ncols + j];
     }
-    part[sl][lo] = s;
+    part[sl][lo] = (s0 + s1) + (s2 + s3);
     __syncthreads();
+    for (int w = 32; w > 0; w >>= 1) {
+        if (sl < w) part[sl][lo] += part[sl + w][lo];
+        __syncthreads();
+    }
     if (sl == 0 && j < ncols) {
-        double v = 0.0;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) v += part[i][lo];
-        v *= scale;
+        const double v = part[0][lo] * scale;
         if (j < split) {
             out0[j] = (float)v;
         } else {
@@ -64,7 +78,7 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const float* __restric
 void launch_reduce_rows(const float* ws, int nrows, int ncols, float* out0, float* out1, int split, double scale,
                         hipStream_t stream)
 {
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3(ceil_div(ncols, 16)), dim3(256), 0, stream, ws, nrows, ncols, out0,
+    hipLaunchKernelGGL(reduce_rows_kernel, dim3(ceil_div(ncols, 16)), dim3(1024), 0, stream, ws, nrows, ncols, out0,
                        out1, split, scale);
 }
 

@@ -787,24 +787,36 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
     for (int i = t; i < Cfg::RW; i += kMlpThreads) out[i] = red[i];
 }
 
-// sums the rows of the partial buffer in a fixed order and scatters the three results
-__global__ __launch_bounds__(256) void mlp_reduce_kernel(const float* __restrict__ ws, int nrows, int RW, int n_up,
-                                                         int n_down, float* __restrict__ d_up,
-                                                         float* __restrict__ d_down, float* __restrict__ d_bias)
+// sums the rows of the partial buffer in a fixed order (16 columns per workgroup, 64 interleaved row slices with four
+// loads in flight, fixed tree in LDS; fp64) and scatters the three results
+__global__ __launch_bounds__(1024) void mlp_reduce_kernel(const float* __restrict__ ws, int nrows, int RW, int n_up,
+                                                          int n_down, float* __restrict__ d_up,
+                                                          float* __restrict__ d_down, float* __restrict__ d_bias)
 {
-    __shared__ double part[16][17];
+    __shared__ double part[64][17];
     const int lo = threadIdx.x % 16, sl = threadIdx.x / 16;
     const int j = blockIdx.x * 16 + lo;
-    double s = 0.0;
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
     if (j < RW) {
-        for (int r = sl; r < nrows; r += 16) s += (double)ws[(int64_t)r * RW + j];
+        int r = sl;
+        for (; r + 192 < nrows; r += 256) {
+            const float a = ws[(int64_t)r * RW + j], b = ws[(int64_t)(r + 64) * RW + j];
+            const float c = ws[(int64_t)(r + 128) * RW + j], d = ws[(int64_t)(r + 192) * RW + j];
+            s0 += (double)a;
+            s1 += (double)b;
+            s2 += (double)c;
+            s3 += (double)d;
+        }
+        for (; r < nrows; r += 64) s0 += (double)ws[(int64_t)r * RW + j];
     }
-    part[sl][lo] = s;
+    part[sl][lo] = (s0 + s1) + (s2 + s3);
     __syncthreads();
+    for (int w = 32; w > 0; w >>= 1) {
+        if (sl < w) part[sl][lo] += part[sl + w][lo];
+        __syncthreads();
+    }
     if (sl == 0 && j < RW) {
-        double v = 0.0;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) v += part[i][lo];
+        const double v = part[0][lo];
         if (j < n_up) d_up[j] = (float)v;
         else if (j < n_up + n_down) d_down[j - n_up] = (float)v;
         else d_bias[j - n_up - n_down] = (float)v;
@@ -872,7 +884,7 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
         int rc = check_launch("lin_brelu_lin_bwd");                                                               \
         if (rc != KEROPS_OK) return rc;                                                                           \
         const int RW = MtCfg<CV>::RW;                                                                             \
-        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(256), 0, s, ws, blocks, RW,           \
+        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws, blocks, RW,           \
                            2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);                                        \
         return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
     }
@@ -887,7 +899,7 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
         int rc = check_launch("lin_brelu_lin_bwd");                                                               \
         if (rc != KEROPS_OK) return rc;                                                                           \
         const int RW = MbCfg<CV>::RW;                                                                             \
-        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(256), 0, s, ws,                       \
+        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws,                      \
                            blocks * MbCfg<CV>::KSPL, RW, 2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);          \
         return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
     }
