@@ -1024,10 +1024,8 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
     p->n_dt = ceil_div(D, p->tile_d);
     if (h_chunk <= 0) {
         const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-        const int64_t target = p->cg == 8 ? 2816 : 704;  // measured at (1, C, 350, 350, 128)
-        const int want_chunks = (int)std::max<int64_t>(1, (target + per_plane / 2) / per_plane);
-        h_chunk = std::max(ceil_div(H, want_chunks), std::min(H, 24));
-        h_chunk = ceil_div(H, ceil_div(H, h_chunk));
+        // two workgroups of 256 threads per CU for 64-channel slabs, one of 512 threads otherwise (registers)
+        h_chunk = pick_h_chunk(H, per_plane, p->cg == 8 ? 512 : 256, 8);
     }
     p->h_chunk = std::min(h_chunk, H);
     p->n_hc = ceil_div(H, p->h_chunk);
