@@ -116,8 +116,14 @@ def ptr(t):
     return t.data_ptr() if t is not None else None
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def stream_of(t):
     """Raw hipStream_t of torch's current stream on the tensor's device."""
+    if _raw_stream is not None:  # one C call instead of building a torch.cuda.Stream object (4 us)
+        index = t.device.index
+        return _raw_stream(index if index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
 
 

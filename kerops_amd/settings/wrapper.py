@@ -40,6 +40,10 @@ class ConfiguredFunction:
 
     def _refresh(self):
         self._conf_params = {k: _param_names(c) for k, c in self.configurators.items() if callable(c)}
+        # positions of those parameters among the wrapped function's positional arguments
+        self._conf_index = {k: [self.usual_args.index(p) for p in names if p in self.usual_args]
+                            for k, names in self._conf_params.items()}
+        self._config_set = frozenset(self.configurable_args)
 
     def __repr__(self):
         lines = [f'{self.origin_function.__name__}{self.signature}']
@@ -62,6 +66,23 @@ class ConfiguredFunction:
         return conf(*[positional[self.usual_args.index(p)] for p in self._conf_params[name]])
 
     def __call__(self, *args, **kwargs):
+        # common case: every ordinary argument positional, keywords only for configurable ones; the general
+        # path below (Signature.bind) costs as much host time as a small kernel takes to run
+        if len(args) == len(self.usual_args) and self._config_set.issuperset(kwargs):
+            final = {}
+            for name in self.configurable_args:
+                if name in kwargs:
+                    final[name] = kwargs[name]
+                else:
+                    conf = self.configurators[name]
+                    if callable(conf):
+                        index = self._conf_index[name]
+                        if len(index) != len(self._conf_params[name]):
+                            break  # a configurator parameter that is not a positional argument: general path
+                        conf = conf(*[args[i] for i in index])
+                    final[name] = conf
+            else:
+                return self.origin_function(*args, **final)
         filled = dict.fromkeys(self.configurable_args, EmptyKwarg)
         filled.update(kwargs)
         bound = self.signature.bind(*args, **filled)
