@@ -5,7 +5,7 @@
 
 One "step" is one pass of the hot path over one synthetic batch that is already resident in
 HBM: DWConv forward followed by DWConvWGRAD at the README shape (1, C, 350, 350, 128), fp16,
-channels_last_3d (BASELINE.json configs 2 and 3).  The script prints ONE JSON line:
+channels_last_3d (the README-shape forward and weight-gradient target configurations).  The script prints ONE JSON line:
 
   metric / value / unit   DWConv fwd + wgrad milliseconds per step (lower is better)
   fwd / wgrad             per-op ms, algorithmic GB/s (4*V*C bytes), % of the 8 TB/s HBM peak and
@@ -268,7 +268,7 @@ def main():
                              'dwconv_frac_hbm_peak': round(4 * V * c / fm / 1e6 / HBM_PEAK_GBPS, 4),
                              'wgrad_frac_hbm_peak': round(4 * V * c / wgm / 1e6 / HBM_PEAK_GBPS, 4)}
         ops['readme_table'] = table
-        # BASELINE config 5: fused depthwise-separable block with int8 output at (1,64,128,128,128)
+        # target configuration 5: fused depthwise-separable block with int8 output at (1,64,128,128,128)
         del x, g
         torch.cuda.empty_cache()
         from kerops_amd.ops.fused import DWSepBlock, PointwiseLinear
@@ -324,7 +324,7 @@ def main():
         'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'f16 in/out, f32 accumulate', 'data': 'synthetic',
         'config': {'workload': f'DWConv fwd + DWConvWGRAD, x/grad fp16 channels_last_3d (1,{C},350,350,128), '
-                               'weight [3,3,3,C], pad 1, stride 1 (BASELINE configs[1] and configs[2])',
+                               'weight [3,3,3,C], pad 1, stride 1 (target configurations 2 and 3)',
                    'channels': C, 'voxels': V, 'inputs_resident_in_hbm': True},
         'fwd': fwd, 'wgrad': wg,
         'clone': {'ms': round(clone_ms, 4), 'ms_min': round(clone_min, 4), 'GBps': round(clone_gbps, 1),

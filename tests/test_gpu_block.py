@@ -1,5 +1,5 @@
 """GPU parity tests of the pointwise MFMA kernel, the ReLULinearAdd drop-in and the fused
-depthwise-separable block with its int8 output (BASELINE config 5)."""
+depthwise-separable block with its int8 output (the fused-block target configuration: x (1,64,128,128,128), 64 -> 128 channels)."""
 import math
 
 import pytest

@@ -307,7 +307,7 @@ def test_quant_i8_sym_bit_exact():
 
 
 def test_config4_pipeline_full_shape():
-    """BASELINE config 4 at (1,64,350,350,128): Stats -> fold -> ApplyBNReLU -> AvgPoolCeilStats.
+    """The BN block target configuration at (1,64,350,350,128): Stats -> fold -> ApplyBNReLU -> AvgPoolCeilStats.
     Checked through properties that do not need a full-size CPU run: the statistics against an
     fp64 reduction on the GPU, BN-ReLU against the formula evaluated by torch on a slab, the
     pooled tensor against torch's AvgPool3d on a slab, and the pooled statistics against the
