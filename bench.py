@@ -303,6 +303,13 @@ def main():
         cl_gbps = 4 * V * cl / cl_ms / 1e6
         ops['ReLULinearAdd_32_32'] = figures(time_op(torch, lambda: ReLULinearAdd(xl, Wl, gl), it, wm)[0],
                                              6 * V * cl, cl_gbps)
+        from kerops_amd.ops.linear import ApplyBNReLULinearAdd
+        bwl = torch.rand(cl, device=dev, generator=gen) + 0.5
+        bbl = torch.randn(cl, device=dev, generator=gen) * 0.3
+        ops['ApplyBNReLU+ReLULinearAdd_fused_32_32'] = figures(
+            time_op(torch, lambda: ApplyBNReLULinearAdd(xl, bwl, bbl, Wl, gl), it, wm)[0], 6 * V * cl, cl_gbps)
+        ops['ApplyBNReLU+ReLULinearAdd_fused_32_32']['note'] = (
+            'replaces ApplyBNReLU (4*V*C bytes more) + ReLULinearAdd, bit-identical')
         ops['ReLULinearBackward_32_32'] = figures(time_op(torch, lambda: ReLULinearBackward(xl, gl, Wl), it, wm)[0],
                                                   6 * V * cl, cl_gbps)
         ops['LinBReLULinAdd_32'] = figures(time_op(torch, lambda: LinBReLULinAdd(xl, Wu, Wd, bl, gl), it, wm)[0],

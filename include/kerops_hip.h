@@ -209,6 +209,15 @@ int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t
 int kerops_pointwise_f16(const void* x, const void* Wm, const void* add, void* out, int64_t V, int32_t Cin,
                          int32_t Cout, int32_t relu_in, void* stream);
 
+/* Batch-norm affine map + ReLU + pointwise product + residual in one pass (an addition, no single reference
+ * counterpart: it stands for kerops_bnrelu_fwd_f16 followed by kerops_pointwise_f16 with relu_in, i.e.
+ * kerops/ops/bnrelu.py:11-42 then kerops/ops/linear/relu_linear_add.py:20-52, bit-identical to that composition,
+ * without writing and re-reading the normalised activation):
+ *   out[v, co] = fp16( sum_ci fp16(max(fma(x[v, ci], scale[ci], shift[ci]), 0)) * Wm[ci, co] ) + add[v, co]
+ * scale, shift: [Cin] fp32.  add may be null.  Cin, Cout in {16,32,64,128}. */
+int kerops_bnrelu_pointwise_f16(const void* x, const float* scale, const float* shift, const void* Wm,
+                                const void* add, void* out, int64_t V, int32_t Cin, int32_t Cout, void* stream);
+
 /* Backward of the ReLU-linear op, one pass over x and grad on MFMA:
  *   dx[v, ci] = x[v, ci] > 0 ? fp16(sum_co g[v, co] * Wm[ci, co]) : 0
  *   dW[ci, co] = sum_v relu(x[v, ci]) * g[v, co]         (fp32, deterministic)

@@ -55,6 +55,7 @@ SIGNATURES = {
     'kerops_absmax_f16': (ctypes.c_int, [_p, _p, _i64, _p, _i64, _i32, _p]),
     'kerops_quant_i8_sym_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p]),
     'kerops_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p]),
+    'kerops_bnrelu_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
     'kerops_lin_brelu_lin_add_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _p]),
     'kerops_lin_brelu_lin_bwd_workspace_bytes': (_i64, [_i64, _i32]),
     'kerops_lin_brelu_lin_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _p]),

@@ -66,7 +66,8 @@ int dwsep_fused_blocks(int32_t N, int32_t H, int32_t W, int32_t D);
 int dwsep_fused_run(const void* x, const void* wt, const float* scale, const float* shift, const void* pw, void* y2,
                     float* amax_ws, int32_t N, int32_t H, int32_t W, int32_t D, int32_t Cout, void* stream);
 int pointwise_dispatch(const _Float16* x, const _Float16* Wm, const _Float16* add, _Float16* out, float* amax_ws,
-                       int64_t V, int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s);
+                       int64_t V, int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s,
+                       const float* scale = nullptr, const float* shift = nullptr);
 int pointwise_blocks(int64_t V);
 void launch_pw_absmax_final(const float* ws, int n, float* out, hipStream_t s);
 

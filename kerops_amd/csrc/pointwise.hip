@@ -35,18 +35,22 @@ struct PwCfg {
     static_assert(COUT % 8 == 0 && COUT <= 128, "COUT in {16,32,64,128}");
 };
 
-template <int CIN, int COUT, bool RELU_IN, bool HAS_ADD, bool ABSMAX>
+// AFFINE: x is first mapped to fp16(max(fma(x, scale[c], shift[c]), 0)), the arithmetic of the batch-norm + ReLU
+// stream op, so that op and the product run as one pass and its result never reaches memory.
+template <int CIN, int COUT, bool RELU_IN, bool HAS_ADD, bool ABSMAX, bool AFFINE = false>
 __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __restrict__ x,
                                                                const half_t* __restrict__ Wm,
                                                                const half_t* __restrict__ add,
                                                                half_t* __restrict__ out, float* __restrict__ amax_ws,
-                                                               int64_t V)
+                                                               int64_t V, const float* __restrict__ scale = nullptr,
+                                                               const float* __restrict__ shift = nullptr)
 {
     using Cfg = PwCfg<CIN, COUT>;
     constexpr int MT = Cfg::MT, KS = Cfg::KS, RH = Cfg::ROW_HALVES;
     __shared__ __attribute__((aligned(16))) half_t tile[kPwWaves][Cfg::TILE_HALVES];
     __shared__ __attribute__((aligned(16))) half_t wfrag[MT * KS * 64 * 8];
     __shared__ float red[kPwWaves];
+    __shared__ __attribute__((aligned(16))) float aff[AFFINE ? 2 * CIN : 4];  // [scale | shift]
 
     const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
     const int vl = lane % 32, hl = lane / 32;
@@ -56,6 +60,12 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
         const int j = i % 8, l = (i / 8) % 64, s = (i / 512) % KS, mt = i / (512 * KS);
         const int co = 32 * mt + l % 32;
         wfrag[i] = (co < COUT) ? Wm[(16 * s + 8 * (l / 32) + j) * COUT + co] : (half_t)0;
+    }
+    if constexpr (AFFINE) {
+        for (int i = t; i < CIN; i += kPwThreads) {
+            aff[i] = scale[i];
+            aff[CIN + i] = shift[i];
+        }
     }
     __syncthreads();
     const half8_t* wa = reinterpret_cast<const half8_t*>(wfrag) + lane;
@@ -81,6 +91,21 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                 // cache to hold the line until the row's other loads arrive, so only narrow rows stream
                 if constexpr (CIN <= 32) xb[q] = load_c8_nt(x + v * CIN + 8 * (2 * q + hl));
                 else xb[q] = load_c8(x + v * CIN + 8 * (2 * q + hl));
+            }
+            if constexpr (AFFINE) {
+#pragma unroll
+                for (int q = 0; q < KS; ++q) {
+                    const int c0 = 8 * (2 * q + hl);  // the chunk's first channel: two addresses per wavefront
+                    const float4_t s0 = *reinterpret_cast<const float4_t*>(aff + c0);
+                    const float4_t s1 = *reinterpret_cast<const float4_t*>(aff + c0 + 4);
+                    const float4_t b0 = *reinterpret_cast<const float4_t*>(aff + CIN + c0);
+                    const float4_t b1 = *reinterpret_cast<const float4_t*>(aff + CIN + c0 + 4);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        xb[q][j] = (half_t)fmaxf(__builtin_fmaf((float)xb[q][j], s0[j], b0[j]), 0.0f);
+                        xb[q][4 + j] = (half_t)fmaxf(__builtin_fmaf((float)xb[q][4 + j], s1[j], b1[j]), 0.0f);
+                    }
+                }
             }
             if (RELU_IN) {
                 const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -179,11 +204,22 @@ static int pw_blocks(int64_t V)
 
 template <int CIN, int COUT>
 static int launch_pw(const half_t* x, const half_t* Wm, const half_t* add, half_t* out, float* amax_ws, int64_t V,
-                     bool relu_in, bool absmax, int blocks, hipStream_t s)
+                     bool relu_in, bool absmax, int blocks, hipStream_t s, const float* scale = nullptr,
+                     const float* shift = nullptr)
 {
+    if (scale) {  // the affine map ends in a ReLU of its own
+        if (add) {
+            hipLaunchKernelGGL((pointwise_kernel<CIN, COUT, false, true, false, true>), dim3(blocks), dim3(kPwThreads), 0,
+                               s, x, Wm, add, out, amax_ws, V, scale, shift);
+        } else {
+            hipLaunchKernelGGL((pointwise_kernel<CIN, COUT, false, false, false, true>), dim3(blocks), dim3(kPwThreads),
+                               0, s, x, Wm, add, out, amax_ws, V, scale, shift);
+        }
+        return check_launch("bnrelu_pointwise");
+    }
 #define KEROPS_PW_GO(R, A, M)                                                                                    \
     hipLaunchKernelGGL((pointwise_kernel<CIN, COUT, R, A, M>), dim3(blocks), dim3(kPwThreads), 0, s, x, Wm, add, \
-                       out, amax_ws, V)
+                       out, amax_ws, V, nullptr, nullptr)
     if (absmax) {
         if (relu_in) KEROPS_PW_GO(true, false, true);
         else KEROPS_PW_GO(false, false, true);
@@ -199,10 +235,12 @@ static int launch_pw(const half_t* x, const half_t* Wm, const half_t* add, half_
 }
 
 int pointwise_dispatch(const half_t* x, const half_t* Wm, const half_t* add, half_t* out, float* amax_ws, int64_t V,
-                       int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s)
+                       int Cin, int Cout, bool relu_in, bool absmax, int blocks, hipStream_t s, const float* scale,
+                       const float* shift)
 {
-#define KEROPS_PW_CASE(CI, CO) \
-    if (Cin == CI && Cout == CO) return launch_pw<CI, CO>(x, Wm, add, out, amax_ws, V, relu_in, absmax, blocks, s);
+#define KEROPS_PW_CASE(CI, CO)      \
+    if (Cin == CI && Cout == CO)    \
+        return launch_pw<CI, CO>(x, Wm, add, out, amax_ws, V, relu_in, absmax, blocks, s, scale, shift);
     KEROPS_PW_CASE(16, 16)
     KEROPS_PW_CASE(16, 32)
     KEROPS_PW_CASE(32, 16)
@@ -248,4 +286,21 @@ extern "C" int kerops_pointwise_f16(const void* x, const void* Wm, const void* a
     }
     return pointwise_dispatch((const half_t*)x, (const half_t*)Wm, (const half_t*)add, (half_t*)out, nullptr, V, Cin,
                               Cout, relu_in != 0, false, pw_blocks(V), (hipStream_t)stream);
+}
+
+extern "C" int kerops_bnrelu_pointwise_f16(const void* x, const float* scale, const float* shift, const void* Wm,
+                                           const void* add, void* out, int64_t V, int32_t Cin, int32_t Cout,
+                                           void* stream)
+{
+    if (!x || !scale || !shift || !Wm || !out || !aligned16(x) || !aligned16(Wm) || !aligned16(out) ||
+        (add && !aligned16(add))) {
+        set_error("bnrelu_pointwise: null or misaligned pointer");
+        return KEROPS_E_BADARG;
+    }
+    if (V <= 0) {
+        set_error("bnrelu_pointwise: V must be positive");
+        return KEROPS_E_BADARG;
+    }
+    return pointwise_dispatch((const half_t*)x, (const half_t*)Wm, (const half_t*)add, (half_t*)out, nullptr, V, Cin,
+                              Cout, false, false, pw_blocks(V), (hipStream_t)stream, scale, shift);
 }

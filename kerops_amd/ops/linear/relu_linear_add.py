@@ -43,3 +43,32 @@ def ReLULinearAdd(x, weight, add_other, *, num_warps: ConfigurableArg, D_block: 
     _lib.call('kerops_pointwise_f16', x.data_ptr(), weight.data_ptr(), add_other.data_ptr(), output.data_ptr(),
               x.numel() // in_channels, in_channels, out_channels, 1, _lib.stream_of(x))
     return output
+
+
+def ApplyBNReLULinearAdd(x, bn_weight, bn_bias, weight, add_other):
+    """ReLULinearAdd(ApplyBNReLU(x, bn_weight, bn_bias), weight, add_other) in one pass, bit-identical to that
+    composition (kerops/ops/bnrelu.py:11-42 then kerops/ops/linear/relu_linear_add.py:20-52): the normalised
+    activation is formed in registers from the loaded x fragments and never written.  An addition to the
+    reference's op set; host side of kerops_bnrelu_pointwise_f16."""
+    in_channels = x.shape[1]
+    out_channels = add_other.shape[1]
+
+    assert x.ndim == add_other.ndim == 5
+    assert list(x.shape[2:]) == list(add_other.shape[2:])
+    assert x.shape[0] == add_other.shape[0]
+    assert list(weight.shape) == [in_channels, out_channels]
+    assert x.dtype == weight.dtype == add_other.dtype == torch.float16
+    assert bn_weight.numel() == bn_bias.numel() == in_channels
+    assert x.is_contiguous(memory_format=torch.channels_last_3d)
+    assert add_other.is_contiguous(memory_format=torch.channels_last_3d)
+    assert in_channels in _BUILT and out_channels in _BUILT, 'built for 16, 32, 64 or 128 channels on either side'
+    require_cuda(x, bn_weight, bn_bias, weight, add_other)
+
+    weight = weight.contiguous()
+    scale = bn_weight.to(torch.float32).contiguous()
+    shift = bn_bias.to(torch.float32).contiguous()
+    output = torch.empty_like(add_other)
+    _lib.call('kerops_bnrelu_pointwise_f16', x.data_ptr(), scale.data_ptr(), shift.data_ptr(), weight.data_ptr(),
+              add_other.data_ptr(), output.data_ptr(), x.numel() // in_channels, in_channels, out_channels,
+              _lib.stream_of(x))
+    return output

@@ -9,7 +9,9 @@ from torch.nn import functional as F
 import oracle
 from conftest import cpu_gen, rand_cl3d, rand_dw_weight
 from kerops_amd.ops.fused import DWSepBlock, DWSepBlockInt8, PointwiseLinear
-from kerops_amd.ops.linear import LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd, ReLULinearBackward
+from kerops_amd.ops.bnrelu import ApplyBNReLU
+from kerops_amd.ops.linear import (ApplyBNReLULinearAdd, LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd,
+                               ReLULinearBackward)
 from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
 
 pytestmark = pytest.mark.gpu
@@ -41,6 +43,26 @@ def test_relu_linear_add_matches_oracle(cin, cout, spatial):
     # the reference's own ground truth: 1x1x1 conv3d of relu(x) plus the residual
     conv = F.conv3d(F.relu(x.float()), Wm.float().t().reshape(cout, cin, 1, 1, 1)).half() + add
     assert torch.allclose(out.float(), conv.float(), rtol=1e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize('cin,cout', [(16, 16), (32, 32), (32, 16), (64, 128), (128, 64), (16, 128)])
+@pytest.mark.parametrize('spatial', [(1, 3, 5, 7), (2, 4, 4, 4), (1, 1, 1, 1), (3, 5, 13, 37)])
+def test_bnrelu_linear_add_equals_composition(cin, cout, spatial):
+    g = cpu_gen(cin * 7 + cout)
+    n, h, w, d = spatial
+    x = rand_cl3d(g, n, cin, h, w, d) * 2 + 0.3
+    add = rand_cl3d(g, n, cout, h, w, d)
+    Wm = rand_pw(g, cin, cout)
+    bw = torch.rand(cin, generator=g) + 0.5
+    bb = torch.randn(cin, generator=g) * 0.5
+    dev = [t_.to(DEV) for t_ in (x, bw, bb, Wm, add)]
+    fused = ApplyBNReLULinearAdd(*dev)
+    composed = ReLULinearAdd(ApplyBNReLU(dev[0], dev[1], dev[2]), dev[3], dev[4])
+    assert fused.shape == add.shape and fused.stride() == add.stride()
+    assert torch.equal(fused.view(torch.int16), composed.view(torch.int16))  # bit for bit
+    ref = oracle.pointwise(oracle.bnrelu_fwd(x, bw, bb), Wm, add=add, relu_in=True)
+    # fp32 MFMA sums against the oracle's fp64: one fp16 rounding of the product apart before the residual add
+    assert (fused.cpu().float() - ref.float()).abs().max() <= 2.0 ** -9 * max(1.0, ref.abs().max().item())
 
 
 @pytest.mark.parametrize('cin,cout', [(16, 16), (16, 32), (32, 16), (32, 32), (32, 64), (64, 64), (64, 128),
