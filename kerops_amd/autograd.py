@@ -13,8 +13,9 @@ import torch
 from .ops.addition import AddStats, AddStatsBackward
 from .ops.avgpool import AvgPoolCeilStats, AvgPoolCeilStatsBackward
 from .ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
-from .ops.conv import DWConv, DWConvWGRAD
-from .ops.linear import LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd, ReLULinearBackward
+from .ops.conv import DWConv, DWConvStats, DWConvWGRAD
+from .ops.linear import (ApplyBNReLULinearAdd, LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd,
+                         ReLULinearBackward)
 from .ops.stats import Stats, StatsBackward
 
 
@@ -136,3 +137,49 @@ class LinBReLULinAddFn(torch.autograd.Function):
         grad_x, grad_up, grad_down, grad_bias = LinBReLULinBackward(x, grad_out, weight_up, weight_down, bias,
                                                                     out_dtype=weight_up.dtype)
         return grad_x, grad_up, grad_down, grad_bias, grad_out
+
+
+class DWConvStatsFn(torch.autograd.Function):
+    """(y, mean, sqmean) = DWConvStats(x, weight): DWConvFn followed by StatsFn on y in one forward pass.
+
+    Backward: the gradient that reaches y is the upstream gradient of y plus the statistics' contribution
+    (AddStatsBackward on y does exactly that sum), then the two convolution gradients as in DWConvFn."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        y, mean, sqmean = DWConvStats(x, weight)
+        ctx.save_for_backward(x, weight, y)
+        return y, mean, sqmean
+
+    @staticmethod
+    def backward(ctx, grad_y, grad_mean, grad_sqmean):
+        x, weight, y = ctx.saved_tensors
+        g = AddStatsBackward(_cl3d(grad_y), grad_mean.float().contiguous(), grad_sqmean.float().contiguous(), y)
+        grad_x = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_x = DWConv(g, torch.flip(weight, dims=(0, 1, 2)).contiguous())
+        if ctx.needs_input_grad[1]:
+            grad_w = DWConvWGRAD(x, g, out_dtype=weight.dtype)
+        return grad_x, grad_w
+
+
+class ApplyBNReLULinearAddFn(torch.autograd.Function):
+    """out = ReLULinearAdd(ApplyBNReLU(x, bn_weight, bn_bias), weight, add_other) in one forward pass.
+
+    The normalised activation is not kept: backward recomputes it (one ApplyBNReLU pass, the time the forward
+    saved) and then runs the two backward ops of the composition."""
+
+    @staticmethod
+    def forward(ctx, x, bn_weight, bn_bias, weight, add_other):
+        ctx.save_for_backward(x, bn_weight, bn_bias, weight)
+        return ApplyBNReLULinearAdd(x, bn_weight, bn_bias, weight, add_other)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, bn_weight, bn_bias, weight = ctx.saved_tensors
+        grad_out = _cl3d(grad_out)
+        z = ApplyBNReLU(x, bn_weight, bn_bias)
+        grad_z, grad_w = ReLULinearBackward(z, grad_out, weight, out_dtype=weight.dtype)
+        dx, dbw, dbb = ApplyBNReLUBackward(x, bn_weight.float(), bn_bias.float(), grad_z)
+        return (dx, dbw.reshape(bn_weight.shape).to(bn_weight.dtype), dbb.reshape(bn_bias.shape).to(bn_bias.dtype),
+                grad_w, grad_out)

@@ -8,7 +8,8 @@ from torch.nn import functional as F
 
 import oracle
 from conftest import cpu_gen, rand_cl3d, rand_dw_weight
-from kerops_amd.autograd import AddStatsFn, ApplyBNReLUFn, AvgPoolCeilStatsFn, DWConvFn, StatsFn
+from kerops_amd.autograd import (AddStatsFn, ApplyBNReLUFn, ApplyBNReLULinearAddFn, AvgPoolCeilStatsFn, DWConvFn,
+                                 DWConvStatsFn, ReLULinearAddFn, StatsFn)
 from kerops_amd.utils import allclose_two_stage, weight_grad_similarity
 
 pytestmark = pytest.mark.gpu
@@ -135,3 +136,45 @@ def test_linear_family_gradients_against_torch_autograd():
         # (the same flips reach the weight gradients; the strict comparison is the one against the oracle)
         assert ((got.grad.float().cpu() - want.grad).norm() / want.grad.norm()).item() < 3e-2
     assert torch.equal(dev[4].grad.cpu(), up2)
+
+
+def test_fused_forward_functions_have_the_gradients_of_their_compositions():
+    # the one-pass forward ops are bit-identical to the compositions they stand for; their backward runs the same
+    # backward ops
+    g = cpu_gen(47)
+    n, c, h, w, d = 2, 32, 6, 7, 9
+    x = rand_cl3d(g, n, c, h, w, d)
+    res = rand_cl3d(g, n, c, h, w, d)
+    _, wk = rand_dw_weight(g, c)
+    pw = (torch.randn(c, c, generator=g) / math.sqrt(c)).half()
+    gamma = torch.rand(c, generator=g) + 0.5
+    beta = torch.randn(c, generator=g) * 0.3
+    go = rand_cl3d(g, n, c, h, w, d)
+
+    def run(fused):
+        leaves = [t.to(DEV).requires_grad_(True) for t in (x, wk, gamma, beta, pw, res)]
+        xd, wd, gd, bd, pd, rd = leaves
+        if fused:
+            y, mean, sq = DWConvStatsFn.apply(xd, wd)
+        else:
+            y = DWConvFn.apply(xd, wd)
+            mean, sq = StatsFn.apply(y)
+        # batch-norm fold in torch autograd (fp32), as a user of the ops would write it
+        inv = torch.rsqrt(sq - mean * mean + 1e-5)
+        scale, shift = gd * inv, bd - mean * gd * inv
+        if fused:
+            out = ApplyBNReLULinearAddFn.apply(y, scale, shift, pd, rd)
+        else:
+            out = ReLULinearAddFn.apply(ApplyBNReLUFn.apply(y, scale, shift), pd, rd)
+        out.backward(go.to(DEV))
+        return [out.detach()] + [t.grad for t in leaves]
+
+    a, b = run(True), run(False)
+    assert torch.equal(a[0], b[0])  # forward: bit for bit
+    # backward: the same backward ops on the same tensors, except that the composition lets torch add the two fp16
+    # gradients that reach y (one more rounding) where the fused Function adds them in fp32 inside AddStatsBackward
+    for i, (u, v) in enumerate(zip(a[1:], b[1:])):
+        assert u.dtype == v.dtype and u.shape == v.shape, i
+        err = (u.float() - v.float()).abs().max().item()
+        assert err <= 2.0 ** -8 * max(1.0, v.float().abs().max().item()), (i, err)
+    assert torch.equal(a[6], b[6])  # the residual's gradient is the upstream gradient in both
