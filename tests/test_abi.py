@@ -95,6 +95,25 @@ def test_workspace_queries():
     assert lib.kerops_absmax_workspace_bytes(10) == 40
 
 
+def test_h_chunk_choice_fills_whole_rounds():
+    # workgroup counts of the built-in launch shapes, read back from the workspace sizes (one partial per
+    # workgroup): 1408 = 2.75 per resident slot at the README shape (the measured optimum), exactly one round of
+    # 512 (or 1024 narrower) workgroups at 128^3-class volumes instead of several short chunks
+    lib = _lib.load()
+
+    def wgrad_blocks(n, h, w, d, c):
+        return lib.kerops_dwconv_wgrad_workspace_bytes(n, h, w, d, c, 0, 0, 0, 0) // (27 * min(c, 64) * 4)
+
+    def fwd_blocks(n, h, w, d, c):
+        return lib.kerops_dwconv_stats_workspace_bytes(n, h, w, d, c) // (2 * min(c, 64) * 4)
+
+    assert wgrad_blocks(1, 350, 350, 128, 64) == 1408 and fwd_blocks(1, 350, 350, 128, 64) == 1408
+    assert wgrad_blocks(1, 128, 128, 128, 64) == 512 and fwd_blocks(1, 128, 128, 128, 64) == 512
+    assert wgrad_blocks(2, 128, 128, 128, 32) == 1024 and fwd_blocks(2, 128, 128, 128, 32) == 512
+    assert fwd_blocks(1, 350, 350, 128, 128) == 4 * 1408  # four chunks of 88 rows: 11 whole rounds
+    assert fwd_blocks(1, 1, 8, 8, 64) == 1 and wgrad_blocks(1, 1, 8, 8, 8) == 1
+
+
 def cl3d(*shape, dtype=torch.float16):
     return torch.zeros(*shape, dtype=dtype).to(memory_format=torch.channels_last_3d)
 
