@@ -5,15 +5,16 @@ The reference exposes forward and backward as separate plain functions (`Stats` 
 wiring once.  Each `apply` takes and returns exactly what the forward op does.  `DWConvFn` also
 provides the input gradient, which the reference lacks (a TODO at kerops/kernels/dw_conv.py:145):
 it is the same depthwise kernel run on the upstream gradient with the weight flipped along the
-three spatial axes.  (`ops.conv.DWConvBackward` computes both gradients in one pass over x and the
-upstream gradient; it moves 27 % fewer bytes but is not faster on MI355X, so the wrapper uses the two kernels.)
+three spatial axes.  With 64 channels and more, and both gradients wanted, the wrapper calls
+`ops.conv.DWConvBackward`, which computes them in one pass over x and the upstream gradient (3-8 % faster
+there, the same input gradient bit for bit); narrower tensors use the two kernels, which are as fast.
 """
 import torch
 
 from .ops.addition import AddStats, AddStatsBackward
 from .ops.avgpool import AvgPoolCeilStats, AvgPoolCeilStatsBackward
 from .ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
-from .ops.conv import DWConv, DWConvStats, DWConvWGRAD
+from .ops.conv import DWConv, DWConvBackward, DWConvStats, DWConvWGRAD
 from .ops.linear import (ApplyBNReLULinearAdd, LinBReLULinAdd, LinBReLULinBackward, ReLULinearAdd,
                          ReLULinearBackward)
 from .ops.stats import Stats, StatsBackward
@@ -21,6 +22,15 @@ from .ops.stats import Stats, StatsBackward
 
 def _cl3d(t):
     return t.contiguous(memory_format=torch.channels_last_3d)
+
+
+def _dwconv_grads(x, weight, grad_out, want_x, want_w):
+    """Input and weight gradient of DWConv for the upstream gradient grad_out."""
+    if want_x and want_w and x.shape[1] >= 64:
+        return DWConvBackward(x, grad_out, weight, out_dtype=weight.dtype)
+    grad_x = DWConv(grad_out, torch.flip(weight, dims=(0, 1, 2)).contiguous()) if want_x else None
+    grad_w = DWConvWGRAD(x, grad_out, out_dtype=weight.dtype) if want_w else None
+    return grad_x, grad_w
 
 
 class DWConvFn(torch.autograd.Function):
@@ -34,13 +44,7 @@ class DWConvFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         x, weight = ctx.saved_tensors
-        grad_out = _cl3d(grad_out)
-        grad_x = grad_w = None
-        if ctx.needs_input_grad[0]:
-            grad_x = DWConv(grad_out, torch.flip(weight, dims=(0, 1, 2)).contiguous())
-        if ctx.needs_input_grad[1]:
-            grad_w = DWConvWGRAD(x, grad_out, out_dtype=weight.dtype)
-        return grad_x, grad_w
+        return _dwconv_grads(x, weight, _cl3d(grad_out), ctx.needs_input_grad[0], ctx.needs_input_grad[1])
 
 
 class StatsFn(torch.autograd.Function):
@@ -155,12 +159,7 @@ class DWConvStatsFn(torch.autograd.Function):
     def backward(ctx, grad_y, grad_mean, grad_sqmean):
         x, weight, y = ctx.saved_tensors
         g = AddStatsBackward(_cl3d(grad_y), grad_mean.float().contiguous(), grad_sqmean.float().contiguous(), y)
-        grad_x = grad_w = None
-        if ctx.needs_input_grad[0]:
-            grad_x = DWConv(g, torch.flip(weight, dims=(0, 1, 2)).contiguous())
-        if ctx.needs_input_grad[1]:
-            grad_w = DWConvWGRAD(x, g, out_dtype=weight.dtype)
-        return grad_x, grad_w
+        return _dwconv_grads(x, weight, g, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
 
 
 class ApplyBNReLULinearAddFn(torch.autograd.Function):

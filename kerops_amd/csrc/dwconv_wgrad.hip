@@ -552,10 +552,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
 // p+1, p, p-1 of g plane p) and, through the interior of the slots of the planes p, p-1, p-2, as the
 // lane-indexed operand of the weight-gradient scheme against x plane p-1.  The g planes next to the chunk
 // are real data for dx but belong to other chunks for gw: the lanes that read them there are masked.
-// The ring with halo, the x buffers and the output tiles take 64 KB (4x8 patch, 256 threads, two workgroups
-// per CU) to 93 KB of LDS and the kernel needs ~190 registers, so few wavefronts are resident: measured at
-// (1,64,350,350,128) it moves 27 % fewer bytes than the two separate kernels but takes the same time
-// (1.49 ms against 1.50 ms); loads run two planes ahead.
+// The ring with halo, the x buffers and the output tiles take up to 93 KB of LDS and the kernel needs ~190
+// registers, so one workgroup of 8 wavefronts is resident per CU; it serves slabs of 8 to 32 channels
+// (64-channel slabs run dwconv_bwd_split_kernel below).  Loads run two planes ahead.
 template <int CG_, int TW_, int TD_, int NT_>
 struct BwCfg {
     static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, NWAVE = NT_ / 64;
@@ -867,6 +866,297 @@ __global__ __launch_bounds__(Cfg::NT, 2) void dwconv_bwd_mfma_kernel(const WgArg
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fused backward for 64-channel slabs with the two products on different wavefronts: a workgroup of 16
+// wavefronts owns an 8x8 patch; all of them stage the planes of x and g (with halo) into LDS, then wavefronts
+// 0-7 run the input-gradient scheme (and store dx through the output tile) while wavefronts 8-15 run the
+// weight-gradient scheme on the same LDS data.  Each role keeps only its own accumulators, so the kernel fits
+// 128 registers and 16 wavefronts stay resident per CU (the one-role-after-the-other kernel above needs ~190
+// and holds 8); the patch is the 8x8 of the separate kernels, so the halo re-reads are theirs too.
+// The roles execute the same sequence of workgroup barriers from two different loops.
+struct BsCfg {
+    static constexpr int CG = 8, TW = 8, TD = 8, NT = 1024, RWAVES = 8;
+    static constexpr int SC = 64, PB = 128, NQ = 16, NHALF = 2;
+    static constexpr int NPART = RWAVES / NHALF, GD = TD / 4, RSPLIT = NPART / GD, RO = TW / RSPLIT;
+    static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, SLOT = R * PDP * PB, GSLOT = SLOT + 32;
+    static constexpr int XOFF = 4 * GSLOT;
+    static constexpr int NPOS = TW * TD, OT_BYTES = NPOS * PB, OT_OFF = XOFF + 2 * SLOT;
+    static constexpr int DUMP = OT_OFF + 2 * OT_BYTES, STAGE_BYTES = DUMP + 16;
+    static constexpr int NCH = R * (TD + 2) * CG;  // 16-byte chunks of a staged plane: one per thread, t < NCH
+    static constexpr int RED_BYTES = NPART * 27 * SC * 4;
+    static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
+    static_assert(NCH <= NT && NPOS * CG == RWAVES * 64 && RO == 4, "one chunk per thread; dx role flushes the tile");
+};
+
+__global__ __launch_bounds__(BsCfg::NT) void dwconv_bwd_split_kernel(const WgArgs a)
+{
+    using Cfg = BsCfg;
+    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
+    constexpr int NQ = Cfg::NQ, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+
+    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
+    if (L >= a.nblocks) return;
+    const uint32_t ws_slot = L;
+    const int slab = L % a.n_slab;
+    L /= a.n_slab;
+    const int dt = L % a.n_dt;
+    L /= a.n_dt;
+    const int wt_i = L % a.n_wt;
+    L /= a.n_wt;
+    const int hc = L % a.n_hc;
+    const int n = L / a.n_hc;
+
+    const int t = threadIdx.x;
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
+    const int hs = hc * a.h_chunk;
+    const int he = min(hs + a.h_chunk, H);
+    const int cslab = slab * SC;
+    const int64_t plane_stride = (int64_t)W * D * C;
+    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
+    const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
+    half_t* dxn = a.dx + (int64_t)n * H * plane_stride;
+
+    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int o = t * 16; o < Cfg::STAGE_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
+
+    // staging: thread t owns chunk t of the patch with halo (x and g alike); threads without a chunk inside the
+    // volume load the plane's first chunk and write it to the dump slot
+    uint32_t go;
+    int ls;
+    {
+        const int wq = t / ((TD + 2) * CG);
+        const int rem = t - wq * ((TD + 2) * CG);
+        const int dq = rem / CG, cq = rem - dq * CG;
+        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
+        const bool ok = (t < Cfg::NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+        go = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        ls = ok ? lds_swizzle<PB>(wq * PDP + dq, cq * 16) : -1;
+    }
+
+    const int lane = t % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
+    const int role = wave / Cfg::RWAVES, rwave = wave % Cfg::RWAVES;  // 0: input gradient, 1: weight gradient
+    const int half = rwave % Cfg::NHALF, part = rwave / Cfg::NHALF;
+    const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RO;
+    const int b = lane / 4, rr = lane % 4;
+    const int q = b;  // 16 channel pairs per instruction, one group of four positions
+    const int r2 = min(rr, 2);
+    const int cb = half * 64 + q * 4;
+    const int c0 = cslab + half * 32 + 2 * q;
+    const int pgrp = gd * 4;
+
+    // loads run two steps ahead in two register sets; unconditional (clamped plane indices)
+    half8_t xpre0, xpre1, gpre0, gpre1;
+    auto prefetch = [&](int p, half8_t& xpre, half8_t& gpre) {  // x plane p-1, g plane p
+        const char* xplane = reinterpret_cast<const char*>(xn + min(max(p - 1, 0), H - 1) * plane_stride);
+        const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(p, 0), H - 1) * plane_stride);
+        xpre = *reinterpret_cast<const half8_t*>(xplane + go);
+        gpre = *reinterpret_cast<const half8_t*>(gplane + go);
+    };
+    int parity = 0;
+    auto stage = [&](int p, const half8_t& xpre, const half8_t& gpre) {
+        const bool gin = (p >= 0) && (p < H) && (p <= he);  // g plane p exists and is needed (dx)
+        unsigned char* xbuf = smem + Cfg::XOFF + parity * SLOT;
+        unsigned char* gslot = smem + (p & 3) * GSLOT;
+        unsigned char* xd = ls >= 0 ? xbuf + ls : smem + Cfg::DUMP;
+        unsigned char* gdst = ls >= 0 ? gslot + ls : smem + Cfg::DUMP;
+        *reinterpret_cast<half8_t*>(xd) = xpre;
+        *reinterpret_cast<half8_t*>(gdst) = gin ? gpre : z8;
+    };
+
+    prefetch(hs - 1, xpre0, gpre0);
+    prefetch(hs, xpre1, gpre1);
+    __syncthreads();  // the one-off zero fill is complete before staging writes anything
+
+    if (role == 0) {
+        // ---- input gradient: flipped weight operands, lane rr = kh' holds (kd' = 0, 1, 2, -) ----
+        half4_t wA[3][2];
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+                if (rr < 3) {
+#pragma unroll
+                    for (int kd = 0; kd < 3; ++kd)
+                        v[kd] = a.wt[(((2 - rr) * 3 + (2 - kw)) * 3 + (2 - kd)) * C + c0 + e];
+                }
+                wA[kw][e] = v;
+            }
+        int dboff[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) dboff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
+        auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
+        int owr[RO];
+#pragma unroll
+        for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
+        // the 512 threads of this role store the tile: one 16-byte chunk each
+        const int opos = t / CG, ocq = t % CG;
+        const int ord = ot_swz(opos, ocq * 16);
+        const int ow = w0 + opos / TD, odd = d0 + opos % TD;
+        const bool ovalid = (ow < W) && (odd < D);
+        const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
+        int pending_row = -1;
+        auto flush_row = [&](int par) {
+            if (pending_row >= 0) {  // workgroup-uniform
+                const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + Cfg::OT_OFF + par * Cfg::OT_BYTES + ord);
+                if (ovalid)
+                    __builtin_nontemporal_store(
+                        o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(dxn + pending_row * plane_stride) + ogo));
+            }
+        };
+        float4_t T[RO][2];  // dx tiles: registers 0, 1, 2 = planes p+1, p, p-1
+#pragma unroll
+        for (int o = 0; o < RO; ++o)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+        auto step = [&](int p, half8_t& xpre, half8_t& gpre) {
+            const bool gin = (p >= 0) && (p < H) && (p <= he);
+            unsigned char* gslot = smem + (p & 3) * GSLOT;
+            stage(p, xpre, gpre);
+            __syncthreads();
+            flush_row(parity ^ 1);
+            prefetch(p + 2, xpre, gpre);
+            __builtin_amdgcn_sched_barrier(0);
+            if (gin) {
+#pragma unroll
+                for (int xr = 0; xr < RO + 2; ++xr) {
+                    uint32_t r[3];
+#pragma unroll
+                    for (int k = 0; k < 3; ++k)
+                        r[k] = *reinterpret_cast<const uint32_t*>(gslot + dboff[k] + xr * PDP * PB);
+                    half4_t B[2];
+                    split_operands3(r, B[0], B[1]);
+#pragma unroll
+                    for (int kw = 0; kw < 3; ++kw) {
+                        if (xr - kw >= 0 && xr - kw < RO) {
+#pragma unroll
+                            for (int e = 0; e < 2; ++e)
+                                T[xr - kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(wA[kw][e], B[e], T[xr - kw][e], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            const int ho = p - 1;  // dx plane p-1 is complete
+            const bool store = (ho >= hs) && (ho < he);
+            pending_row = store ? ho : -1;
+            if (store) {
+                unsigned char* otile = smem + Cfg::OT_OFF + parity * Cfg::OT_BYTES;
+#pragma unroll
+                for (int o = 0; o < RO; ++o) {
+                    half2_t v;
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
+                    *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
+                }
+            }
+#pragma unroll
+            for (int o = 0; o < RO; ++o)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    T[o][e][2] = T[o][e][1];
+                    T[o][e][1] = T[o][e][0];
+                    T[o][e][0] = 0.0f;
+                }
+            parity ^= 1;
+        };
+        for (int p = hs - 1;;) {
+            step(p, xpre0, gpre0);
+            if (++p > he + 1) break;
+            step(p, xpre1, gpre1);
+            if (++p > he + 1) break;
+        }
+        __syncthreads();  // the last tile is written
+        flush_row(parity ^ 1);
+        __syncthreads();  // (the other role: staging buffers are dead)
+        __syncthreads();  // (the other role: partial sums are in LDS)
+    } else {
+        // ---- weight gradient: x windows (patch row ra + xr, positions pgrp + r2 + k) against the interior of
+        // the g slots (patch row ra + 1 + gr, positions pgrp + 1 + k), lane j reads the slot of plane p - j ----
+        int aoff[4], boff[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            aoff[k] = lds_swizzle<PB>(ra * PDP + pgrp + r2 + k, cb);
+            boff[k] = lds_swizzle<PB>((ra + 1) * PDP + pgrp + 1 + k, cb);
+        }
+        float4_t acc[3][2];  // one tile per kw: D[i = kd][j = kh]
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+        auto step = [&](int p, half8_t& xpre, half8_t& gpre) {
+            const int xq = p - 1;
+            const bool xin = (xq >= 0) && (xq < H) && (xq >= hs - 1) && (xq <= he);
+            const unsigned char* xbuf = smem + Cfg::XOFF + parity * SLOT;
+            stage(p, xpre, gpre);
+            __syncthreads();
+            prefetch(p + 2, xpre, gpre);
+            __builtin_amdgcn_sched_barrier(0);
+            if (xin) {
+                const int gp = p - r2;  // the lane's g plane; planes of other chunks are masked
+                const uint32_t gmask = (gp >= hs && gp < he) ? 0xffffffffu : 0u;
+                const int gso = (gp & 3) * GSLOT;
+                half4_t G[RO][2];
+#pragma unroll
+                for (int xr = 0; xr < RO + 2; ++xr) {
+                    if (xr < RO) {
+                        uint32_t r[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            r[k] = *reinterpret_cast<const uint32_t*>(smem + gso + boff[k] + xr * PDP * PB) & gmask;
+                        split_operands(r, G[xr][0], G[xr][1]);
+                    }
+                    uint32_t r[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) r[k] = *reinterpret_cast<const uint32_t*>(xbuf + aoff[k] + xr * PDP * PB);
+                    half4_t A[2];
+                    split_operands(r, A[0], A[1]);
+#pragma unroll
+                    for (int kw = 0; kw < 3; ++kw) {
+                        if (xr - kw >= 0 && xr - kw < RO) {
+#pragma unroll
+                            for (int e = 0; e < 2; ++e)
+                                acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], G[xr - kw][e], acc[kw][e], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            parity ^= 1;
+        };
+        for (int p = hs - 1;;) {
+            step(p, xpre0, gpre0);
+            if (++p > he + 1) break;
+            step(p, xpre1, gpre1);
+            if (++p > he + 1) break;
+        }
+        __syncthreads();  // (the other role: the last tile is written)
+        __syncthreads();  // staging buffers are dead from here on
+        float* red = reinterpret_cast<float*>(smem);  // [NPART][27][SC]
+        if (rr < 3) {
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+#pragma unroll
+                    for (int i = 0; i < 3; ++i)
+                        red[(part * 27 + (rr * 3 + kw) * 3 + i) * SC + half * 32 + 2 * q + e] = acc[kw][e][i];
+        }
+        __syncthreads();
+    }
+    const float* red = reinterpret_cast<const float*>(smem);
+    float* out = a.ws + (int64_t)ws_slot * 27 * SC;
+    for (int o = t; o < 27 * SC; o += NT) {
+        float sacc = 0.0f;
+#pragma unroll
+        for (int pt = 0; pt < Cfg::NPART; ++pt) sacc += red[pt * 27 * SC + o];
+        out[o] = sacc;
+    }
+}
+
 // Second pass, fixed summation order (deterministic).  The workspace holds one row per (n, h-chunk, w-patch,
 // d-patch) of width RW = slabs*27*SC floats.  A workgroup owns 16 columns, its 64 row slices sum interleaved rows
 // (four loads in flight), the slices are combined in LDS in a fixed order and the result is scattered to the
@@ -1000,7 +1290,7 @@ static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, float* gw, hip
     return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg>, base, p, gw, stream);
 }
 
-// fused backward: one patch shape per channel count, one workgroup of 512 threads per CU
+// fused backward: one patch shape per channel count, one workgroup per CU
 static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
 {
     if (N <= 0 || H <= 0 || W <= 0 || D <= 0) {
@@ -1017,15 +1307,15 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
     }
     p->cg = C >= 64 ? 8 : C / 8;
     p->cl = 16;
-    p->tile_w = p->cg == 8 ? 4 : 8;
+    p->tile_w = 8;
     p->tile_d = p->cg == 8 ? 8 : p->cg == 4 ? 16 : p->cg == 2 ? 32 : 64;
     p->n_slab = C / (p->cg * 8);
     p->n_wt = ceil_div(W, p->tile_w);
     p->n_dt = ceil_div(D, p->tile_d);
     if (h_chunk <= 0) {
         const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-        // two workgroups of 256 threads per CU for 64-channel slabs, one of 512 threads otherwise (registers)
-        h_chunk = pick_h_chunk(H, per_plane, p->cg == 8 ? 512 : 256, 8);
+        // one workgroup per CU: 1024 threads for 64-channel slabs (LDS), 512 threads otherwise (registers)
+        h_chunk = pick_h_chunk(H, per_plane, 256, 8);
     }
     p->h_chunk = std::min(h_chunk, H);
     p->n_hc = ceil_div(H, p->h_chunk);
@@ -1100,7 +1390,19 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
         case 1: return launch_bwd<1, 8, 64>(a, p, gw, s);
         case 2: return launch_bwd<2, 8, 32>(a, p, gw, s);
         case 4: return launch_bwd<4, 8, 16>(a, p, gw, s);
-        default: return launch_bwd<8, 4, 8, 256>(a, p, gw, s);
+        default: {
+            WgArgs b = a;
+            b.n_wt = p.n_wt;
+            b.n_dt = p.n_dt;
+            b.n_hc = p.n_hc;
+            b.n_slab = p.n_slab;
+            b.h_chunk = p.h_chunk;
+            b.nblocks = (uint32_t)p.nblocks;
+            hipLaunchKernelGGL(dwconv_bwd_split_kernel, dim3(xcd_padded_grid(b.nblocks)), dim3(BsCfg::NT), 0, s, b);
+            rc = check_launch("dwconv_bwd");
+            if (rc != KEROPS_OK) return rc;
+            return reduce_partials(b.ws, p, BsCfg::SC, b.C, gw, s);
+        }
     }
 }
 
