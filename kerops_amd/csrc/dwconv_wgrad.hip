@@ -547,354 +547,46 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
 //   gw[kh,kw,kd,c] = sum g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]
 //
 // Run separately the two products read g twice (8.8 GB at C=64 with the halos); here a workgroup stages
-// every g plane of its patch once, with halo, into the ring of four LDS slots and uses it twice: as the
+// every g plane of its patch once, with halo, into a ring of four LDS slots and uses it twice: as the
 // scattered operand of the forward scheme (weights flipped, accumulator registers = the dx planes
 // p+1, p, p-1 of g plane p) and, through the interior of the slots of the planes p, p-1, p-2, as the
 // lane-indexed operand of the weight-gradient scheme against x plane p-1.  The g planes next to the chunk
 // are real data for dx but belong to other chunks for gw: the lanes that read them there are masked.
-// The ring with halo, the x buffers and the output tiles take up to 93 KB of LDS and the kernel needs ~190
-// registers, so one workgroup of 8 wavefronts is resident per CU; it serves slabs of 8 to 32 channels
-// (64-channel slabs run dwconv_bwd_split_kernel below).  Loads run two planes ahead.
+//
+// The two products run on different wavefronts: all 8 wavefronts of a workgroup stage the planes of x and g
+// (with halo) into LDS, then wavefronts 0-3 run the input-gradient scheme (and store dx) while wavefronts 4-7
+// run the weight-gradient scheme on the same LDS data, each role in its own loop with the same sequence of
+// workgroup barriers.  A role keeps only its own accumulators: 112-122 registers and 35-62 KB of LDS, so two
+// workgroups (16 wavefronts) are resident per CU, where running both schemes in every wavefront needs ~190
+// registers and holds 8 wavefronts (that version took 1.55 ms at (1,64,350,350,128), this one 1.42 ms; the
+// two separate kernels 1.54-1.58 ms).  An 8x8 patch with 16 wavefronts re-reads less halo but leaves one
+// workgroup per CU, whose per-plane barriers are then fully exposed: 1.50 ms.
 template <int CG_, int TW_, int TD_, int NT_>
-struct BwCfg {
-    static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, NWAVE = NT_ / 64;
+struct BsCfg {
+    static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, RWAVES = NT_ / 128;  // wavefronts per role
     static constexpr int SC = CG * 8, PB = SC * 2;
     static constexpr int NQ = SC >= 32 ? 16 : SC / 2, NSUB = 16 / NQ, NHALF = SC / (2 * NQ);
-    static constexpr int NPART = NWAVE / NHALF, GD = TD / (4 * NSUB), RSPLIT = NPART / GD;
-    static constexpr int RO = TW / RSPLIT;            // rows of the patch per wavefront (dx rows = g rows)
-    static constexpr int R = TW + 2;                  // rows incl. halo
-    static constexpr int PDP = (TD + 3 + 3) / 4 * 4;  // positions per row: halo + one over-read, padded to 4
-    static constexpr int SLOT = R * PDP * PB;
+    static constexpr int NPART = RWAVES / NHALF, GD = TD / (4 * NSUB), RSPLIT = NPART / GD, RO = TW / RSPLIT;
+    static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, SLOT = R * PDP * PB;
     static constexpr int GSLOT = SLOT + (SC == 8 ? 16 : 32);  // lanes j read different slots: shift their banks apart
-    static constexpr int XOFF = 4 * GSLOT;            // [4 g slots][2 x slots][2 output tiles][dump]
-    static constexpr int NPOS = TW * TD, OT_BYTES = NPOS * PB;
-    static constexpr int OT_OFF = XOFF + 2 * SLOT;
-    static constexpr int DUMP = OT_OFF + 2 * OT_BYTES;
-    static constexpr int STAGE_BYTES = DUMP + 16;
-    static constexpr int NCH = R * (TD + 2) * CG;
-    static constexpr int NLD = (NCH + NT - 1) / NT;
-    static constexpr int RED_BYTES = NPART * 27 * SC * 4;
-    static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
-    static constexpr bool BOUNCE = SC == 64;          // dx leaves through the output tile as whole 128-byte lines
-    static_assert(TD % (4 * NSUB) == 0 && NPART % GD == 0 && NPART >= GD && TW % RSPLIT == 0, "even split");
-    static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
-    static_assert(STAGE_BYTES % 16 == 0, "16-byte chunks");
-};
-
-template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, 2) void dwconv_bwd_mfma_kernel(const WgArgs a)
-{
-    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
-    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT, NLD = Cfg::NLD;
-    constexpr bool BOUNCE = Cfg::BOUNCE;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
-
-    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
-    if (L >= a.nblocks) return;
-    const uint32_t ws_slot = L;
-    const int slab = L % a.n_slab;
-    L /= a.n_slab;
-    const int dt = L % a.n_dt;
-    L /= a.n_dt;
-    const int wt_i = L % a.n_wt;
-    L /= a.n_wt;
-    const int hc = L % a.n_hc;
-    const int n = L / a.n_hc;
-
-    const int t = threadIdx.x;
-    const int H = a.H, W = a.W, D = a.D, C = a.C;
-    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
-    const int hs = hc * a.h_chunk;
-    const int he = min(hs + a.h_chunk, H);
-    const int cslab = slab * SC;
-    const int64_t plane_stride = (int64_t)W * D * C;
-    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
-    const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
-    half_t* dxn = a.dx + (int64_t)n * H * plane_stride;
-
-    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int o = t * 16; o < Cfg::STAGE_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
-
-    // staging assignment, shared by x and g (same patch with halo): 16-byte chunks; lanes without a chunk
-    // inside the volume load the plane's first chunk and write it to the dump slot
-    uint32_t go[NLD];
-    int ls[NLD];
-#pragma unroll
-    for (int j = 0; j < NLD; ++j) {
-        const int ch = t + j * NT;
-        const int wq = ch / ((TD + 2) * CG);
-        const int rem = ch - wq * ((TD + 2) * CG);
-        const int dq = rem / CG, cq = rem - dq * CG;
-        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
-        const bool ok = (ch < Cfg::NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
-        go[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
-        ls[j] = ok ? lds_swizzle<PB>(wq * PDP + dq, cq * 16) : -1;
-    }
-
-    const int lane = t % kWave, wave = t / kWave;
-    const int half = wave % Cfg::NHALF, part = wave / Cfg::NHALF;
-    const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RO;
-    const int b = lane / 4, rr = lane % 4;
-    const int q = b % NQ, sub = b / NQ;
-    const int r2 = min(rr, 2);
-    const int cb = half * 64 + q * 4;
-    const int c0 = cslab + half * 32 + 2 * q;
-    const int pgrp = (gd * NSUB + sub) * 4;
-
-    // dx: flipped weight operands, lane rr = kh' holds (kd' = 0, 1, 2, -) with wt index (2-kh', 2-kw', 2-kd')
-    half4_t wA[3][2];
-#pragma unroll
-    for (int kw = 0; kw < 3; ++kw)
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
-            if (rr < 3) {
-#pragma unroll
-                for (int kd = 0; kd < 3; ++kd) v[kd] = a.wt[(((2 - rr) * 3 + (2 - kw)) * 3 + (2 - kd)) * C + c0 + e];
-            }
-            wA[kw][e] = v;
-        }
-    // dx operand from the g slot (patch coordinates incl. halo): positions pgrp + rr + k of patch row ra + xr
-    int dboff[3];
-#pragma unroll
-    for (int k = 0; k < 3; ++k) dboff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
-    // gw operands: x windows (patch row ra + xr, positions pgrp + r2 + k) and the interior of the g slots
-    // (patch row ra + 1 + gr, positions pgrp + 1 + k)
-    int aoff[4], boff[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        aoff[k] = Cfg::XOFF + lds_swizzle<PB>(ra * PDP + pgrp + r2 + k, cb);
-        boff[k] = lds_swizzle<PB>((ra + 1) * PDP + pgrp + 1 + k, cb);
-    }
-
-    // dx output (see the forward kernel): tile + one 16-byte chunk per thread, or direct dwords
-    auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
-    int owr[RO];
-#pragma unroll
-    for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
-    const int opos = t / CG, ocq = t % CG;
-    const int ord = ot_swz(opos, ocq * 16);
-    const int ow = w0 + opos / TD, odd = d0 + opos % TD;
-    const bool ovalid = (ow < W) && (odd < D);
-    const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
-    const int od = d0 + pgrp + rr;
-    uint32_t ooff[RO];
-    bool oval[RO];
-#pragma unroll
-    for (int o = 0; o < RO; ++o) {
-        const int w = w0 + ra + o;
-        oval[o] = (od < D) && (w < W);
-        ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
-    }
-    int pending_row = -1;
-    auto flush_row = [&](int par) {
-        if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
-            const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + Cfg::OT_OFF + par * Cfg::OT_BYTES + ord);
-            if (ovalid)
-                __builtin_nontemporal_store(
-                    o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(dxn + pending_row * plane_stride) + ogo));
-        }
-    };
-
-    float4_t T[RO][2];   // dx tiles: registers 0, 1, 2 = planes p+1, p, p-1
-    float4_t acc[3][2];  // gw tiles, one per kw: D[i = kd][j = kh]
-#pragma unroll
-    for (int o = 0; o < RO; ++o)
-#pragma unroll
-        for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int kw = 0; kw < 3; ++kw)
-#pragma unroll
-        for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-
-    // step p: g plane p and x plane p-1 arrive.  Loads are unconditional (clamped plane indices; what is not
-    // needed is dropped or overwritten by zeros at staging) and run two steps ahead in two register sets.
-    half8_t xpre0[NLD], xpre1[NLD], gpre0[NLD], gpre1[NLD];
-    auto prefetch = [&](int p, half8_t(&xpre)[NLD], half8_t(&gpre)[NLD]) {
-        const char* xplane = reinterpret_cast<const char*>(xn + min(max(p - 1, 0), H - 1) * plane_stride);
-        const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(p, 0), H - 1) * plane_stride);
-#pragma unroll
-        for (int j = 0; j < NLD; ++j) xpre[j] = *reinterpret_cast<const half8_t*>(xplane + go[j]);
-#pragma unroll
-        for (int j = 0; j < NLD; ++j) gpre[j] = *reinterpret_cast<const half8_t*>(gplane + go[j]);
-    };
-
-    int parity = 0;
-    auto step = [&](int p, half8_t(&xpre)[NLD], half8_t(&gpre)[NLD]) {
-        const int xq = p - 1;
-        const bool gin = (p >= 0) && (p < H) && (p <= he);            // g plane p exists and is needed (dx)
-        const bool xin = (xq >= 0) && (xq < H) && (xq >= hs - 1) && (xq <= he);  // x plane p-1 exists and is needed
-        unsigned char* xbuf = smem + Cfg::XOFF + parity * SLOT;
-        unsigned char* gslot = smem + (p & 3) * GSLOT;
-#pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            unsigned char* xd = ls[j] >= 0 ? xbuf + ls[j] : smem + Cfg::DUMP;
-            unsigned char* gdst = ls[j] >= 0 ? gslot + ls[j] : smem + Cfg::DUMP;
-            *reinterpret_cast<half8_t*>(xd) = xpre[j];
-            *reinterpret_cast<half8_t*>(gdst) = gin ? gpre[j] : z8;
-        }
-        __syncthreads();
-        flush_row(parity ^ 1);
-        prefetch(p + 2, xpre, gpre);
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- dx: scatter g plane p into the planes p+1, p, p-1 ----
-        if (gin) {
-#pragma unroll
-            for (int xr = 0; xr < RO + 2; ++xr) {
-                uint32_t r[3];
-#pragma unroll
-                for (int k = 0; k < 3; ++k) r[k] = *reinterpret_cast<const uint32_t*>(gslot + dboff[k] + xr * PDP * PB);
-                half4_t B[2];
-                split_operands3(r, B[0], B[1]);
-#pragma unroll
-                for (int kw = 0; kw < 3; ++kw) {
-                    if (xr - kw >= 0 && xr - kw < RO) {
-#pragma unroll
-                        for (int e = 0; e < 2; ++e)
-                            T[xr - kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(wA[kw][e], B[e], T[xr - kw][e], 0, 0, 0);
-                    }
-                }
-            }
-        }
-        // ---- gw: x plane p-1 against the g planes p, p-1, p-2 (lane j), masked to the chunk ----
-        if (xin) {
-            const int gp = p - r2;                                    // the lane's g plane
-            const uint32_t gmask = (gp >= hs && gp < he) ? 0xffffffffu : 0u;
-            const int gso = (gp & 3) * GSLOT;
-            half4_t G[RO][2];
-#pragma unroll
-            for (int xr = 0; xr < RO + 2; ++xr) {
-                if (xr < RO) {
-                    uint32_t r[4];
-#pragma unroll
-                    for (int k = 0; k < 4; ++k)
-                        r[k] = *reinterpret_cast<const uint32_t*>(smem + gso + boff[k] + xr * PDP * PB) & gmask;
-                    split_operands(r, G[xr][0], G[xr][1]);
-                }
-                uint32_t r[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) r[k] = *reinterpret_cast<const uint32_t*>(xbuf - Cfg::XOFF + aoff[k] + xr * PDP * PB);
-                half4_t A[2];
-                split_operands(r, A[0], A[1]);
-#pragma unroll
-                for (int kw = 0; kw < 3; ++kw) {
-                    if (xr - kw >= 0 && xr - kw < RO) {
-#pragma unroll
-                        for (int e = 0; e < 2; ++e)
-                            acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], G[xr - kw][e], acc[kw][e], 0, 0, 0);
-                    }
-                }
-            }
-        }
-        // ---- dx plane p-1 is complete ----
-        const int ho = p - 1;
-        const bool store = (ho >= hs) && (ho < he);  // workgroup-uniform
-        pending_row = store ? ho : -1;
-        if (store) {
-            unsigned char* otile = smem + Cfg::OT_OFF + parity * Cfg::OT_BYTES;
-#pragma unroll
-            for (int o = 0; o < RO; ++o) {
-                half2_t v;
-#pragma unroll
-                for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
-                if constexpr (BOUNCE) {
-                    *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
-                } else {
-                    if (oval[o])
-                        __builtin_nontemporal_store(
-                            v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(dxn + ho * plane_stride) + ooff[o]));
-                }
-            }
-        }
-#pragma unroll
-        for (int o = 0; o < RO; ++o)
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                T[o][e][2] = T[o][e][1];
-                T[o][e][1] = T[o][e][0];
-                T[o][e][0] = 0.0f;
-            }
-        parity ^= 1;
-    };
-
-    prefetch(hs - 1, xpre0, gpre0);
-    prefetch(hs, xpre1, gpre1);
-    __syncthreads();  // the one-off zero fill is complete before staging writes anything
-    for (int p = hs - 1;;) {
-        step(p, xpre0, gpre0);
-        if (++p > he + 1) break;
-        step(p, xpre1, gpre1);
-        if (++p > he + 1) break;
-    }
-    if constexpr (BOUNCE) {
-        __syncthreads();
-        flush_row(parity ^ 1);
-    }
-
-    // ---- gw partial of the workgroup (as in the weight-gradient kernel) ----
-    if (NSUB > 1) {
-#pragma unroll
-        for (int kw = 0; kw < 3; ++kw)
-#pragma unroll
-            for (int e = 0; e < 2; ++e)
-#pragma unroll
-                for (int i = 0; i < 3; ++i) {
-                    float v = acc[kw][e][i];
-#pragma unroll
-                    for (int off = 4 * NQ; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
-                    acc[kw][e][i] = v;
-                }
-    }
-    __syncthreads();
-    float* red = reinterpret_cast<float*>(smem);  // [NPART][27][SC]
-    if (sub == 0 && rr < 3) {
-#pragma unroll
-        for (int kw = 0; kw < 3; ++kw)
-#pragma unroll
-            for (int e = 0; e < 2; ++e)
-#pragma unroll
-                for (int i = 0; i < 3; ++i)
-                    red[(part * 27 + (rr * 3 + kw) * 3 + i) * SC + half * 32 + 2 * q + e] = acc[kw][e][i];
-    }
-    __syncthreads();
-    float* out = a.ws + (int64_t)ws_slot * 27 * SC;
-    for (int o = t; o < 27 * SC; o += NT) {
-        float sacc = 0.0f;
-#pragma unroll
-        for (int pt = 0; pt < Cfg::NPART; ++pt) sacc += red[pt * 27 * SC + o];
-        out[o] = sacc;
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Fused backward for 64-channel slabs with the two products on different wavefronts: a workgroup of 8
-// wavefronts owns a 4x8 patch; all of them stage the planes of x and g (with halo) into LDS, then wavefronts
-// 0-3 run the input-gradient scheme (and store dx through the output tile) while wavefronts 4-7 run the
-// weight-gradient scheme on the same LDS data, each role in its own loop with the same sequence of workgroup
-// barriers.  A role keeps only its own accumulators: 112 registers and 62 KB of LDS, so two workgroups (16
-// wavefronts) are resident per CU, where a kernel that runs both schemes in every wavefront needs ~190 registers
-// and holds 8.  (An 8x8 patch with 16 wavefronts re-reads less halo but leaves one workgroup per CU, whose
-// per-plane barriers are then fully exposed: 1.50 ms against 1.42 ms at (1,64,350,350,128).)
-template <int TW_, int NT_>
-struct BsCfg {
-    static constexpr int CG = 8, TW = TW_, TD = 8, NT = NT_, RWAVES = NT_ / 128;  // wavefronts per role
-    static constexpr int SC = 64, PB = 128, NQ = 16, NHALF = 2;
-    static constexpr int NPART = RWAVES / NHALF, GD = TD / 4, RSPLIT = NPART / GD, RO = TW / RSPLIT;
-    static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, SLOT = R * PDP * PB, GSLOT = SLOT + 32;
     static constexpr int XOFF = 4 * GSLOT;
-    static constexpr int NPOS = TW * TD, OT_BYTES = NPOS * PB, OT_OFF = XOFF + 2 * SLOT;
+    static constexpr bool BOUNCE = SC == 64;  // dx leaves through the output tile as whole 128-byte lines
+    static constexpr int NPOS = TW * TD, OT_BYTES = BOUNCE ? NPOS * PB : 0, OT_OFF = XOFF + 2 * SLOT;
     static constexpr int DUMP = OT_OFF + 2 * OT_BYTES, STAGE_BYTES = DUMP + 16;
     static constexpr int NCH = R * (TD + 2) * CG;  // 16-byte chunks of a staged plane: one per thread, t < NCH
     static constexpr int RED_BYTES = NPART * 27 * SC * 4;
     static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
-    static_assert(NCH <= NT && NPOS * CG == RWAVES * 64 && RO == 4, "one chunk per thread; dx role flushes the tile");
+    static_assert(NCH <= NT && RO == 4 && TD % (4 * NSUB) == 0 && NPART % GD == 0 && TW % RSPLIT == 0, "even split");
+    static_assert(!BOUNCE || NPOS * CG == RWAVES * 64, "the dx role stores the tile: one 16-byte chunk per thread");
+    static_assert(STAGE_BYTES % 16 == 0, "16-byte chunks");
 };
 
 template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
-    constexpr int NQ = Cfg::NQ, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
+    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
+    constexpr bool BOUNCE = Cfg::BOUNCE;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
     uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
@@ -943,11 +635,11 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
     const int half = rwave % Cfg::NHALF, part = rwave / Cfg::NHALF;
     const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RO;
     const int b = lane / 4, rr = lane % 4;
-    const int q = b;  // 16 channel pairs per instruction, one group of four positions
+    const int q = b % NQ, sub = b / NQ;  // block = (channel pair, group of four positions)
     const int r2 = min(rr, 2);
     const int cb = half * 64 + q * 4;
     const int c0 = cslab + half * 32 + 2 * q;
-    const int pgrp = gd * 4;
+    const int pgrp = (gd * NSUB + sub) * 4;
 
     // loads run two steps ahead in two register sets; unconditional (clamped plane indices)
     half8_t xpre0, xpre1, gpre0, gpre1;
@@ -994,15 +686,25 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
         int owr[RO];
 #pragma unroll
         for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
-        // the 512 threads of this role store the tile: one 16-byte chunk each
+        // 64-channel slabs: the threads of this role store the tile, one 16-byte chunk each; narrower slabs
+        // store their dwords directly (runs of 256 contiguous bytes per instruction)
         const int opos = t / CG, ocq = t % CG;
         const int ord = ot_swz(opos, ocq * 16);
         const int ow = w0 + opos / TD, odd = d0 + opos % TD;
         const bool ovalid = (ow < W) && (odd < D);
         const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
+        const int od = d0 + pgrp + rr;
+        uint32_t ooff[RO];
+        bool oval[RO];
+#pragma unroll
+        for (int o = 0; o < RO; ++o) {
+            const int w = w0 + ra + o;
+            oval[o] = (od < D) && (w < W);
+            ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
+        }
         int pending_row = -1;
         auto flush_row = [&](int par) {
-            if (pending_row >= 0) {  // workgroup-uniform
+            if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
                 const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + Cfg::OT_OFF + par * Cfg::OT_BYTES + ord);
                 if (ovalid)
                     __builtin_nontemporal_store(
@@ -1052,7 +754,13 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
                     half2_t v;
 #pragma unroll
                     for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
-                    *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
+                    if constexpr (BOUNCE) {
+                        *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
+                    } else {
+                        if (oval[o])
+                            __builtin_nontemporal_store(
+                                v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(dxn + ho * plane_stride) + ooff[o]));
+                    }
                 }
             }
 #pragma unroll
@@ -1135,10 +843,23 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
             step(p, xpre1, gpre1);
             if (++p > he + 1) break;
         }
+        if (NSUB > 1) {  // position groups inside the wavefront
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+#pragma unroll
+                    for (int i = 0; i < 3; ++i) {
+                        float v = acc[kw][e][i];
+#pragma unroll
+                        for (int off = 4 * NQ; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
+                        acc[kw][e][i] = v;
+                    }
+        }
         __syncthreads();  // (the other role: the last tile is written)
         __syncthreads();  // staging buffers are dead from here on
         float* red = reinterpret_cast<float*>(smem);  // [NPART][27][SC]
-        if (rr < 3) {
+        if (sub == 0 && rr < 3) {
 #pragma unroll
             for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
@@ -1310,14 +1031,14 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
     p->cg = C >= 64 ? 8 : C / 8;
     p->cl = 16;
     p->tile_w = p->cg == 8 ? 4 : 8;
-    p->tile_d = p->cg == 8 ? 8 : p->cg == 4 ? 16 : p->cg == 2 ? 32 : 64;
+    p->tile_d = p->cg >= 4 ? 8 : p->cg == 2 ? 16 : 32;
     p->n_slab = C / (p->cg * 8);
     p->n_wt = ceil_div(W, p->tile_w);
     p->n_dt = ceil_div(D, p->tile_d);
     if (h_chunk <= 0) {
         const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-        // 64-channel slabs: two workgroups of 512 threads per CU (LDS); narrower: one (registers)
-        h_chunk = pick_h_chunk(H, per_plane, p->cg == 8 ? 512 : 256, 8);
+        // two workgroups of 512 threads per CU
+        h_chunk = pick_h_chunk(H, per_plane, 512, 8);
     }
     p->h_chunk = std::min(h_chunk, H);
     p->n_hc = ceil_div(H, p->h_chunk);
@@ -1327,23 +1048,6 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
         return KEROPS_E_BADARG;
     }
     return KEROPS_OK;
-}
-
-template <int CG, int TW, int TD, int NT = 512>
-static int launch_bwd(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
-{
-    using Cfg = BwCfg<CG, TW, TD, NT>;
-    WgArgs a = base;
-    a.n_wt = p.n_wt;
-    a.n_dt = p.n_dt;
-    a.n_hc = p.n_hc;
-    a.n_slab = p.n_slab;
-    a.h_chunk = p.h_chunk;
-    a.nblocks = (uint32_t)p.nblocks;
-    hipLaunchKernelGGL(dwconv_bwd_mfma_kernel<Cfg>, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
-    int rc = check_launch("dwconv_bwd");
-    if (rc != KEROPS_OK) return rc;
-    return reduce_partials(a.ws, p, Cfg::SC, a.C, gw, stream);
 }
 
 }  // namespace kerops
@@ -1388,25 +1092,28 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
     a.D = D;
     a.C = C;
     hipStream_t s = (hipStream_t)stream;
-    switch (p.cg) {
-        case 1: return launch_bwd<1, 8, 64>(a, p, gw, s);
-        case 2: return launch_bwd<2, 8, 32>(a, p, gw, s);
-        case 4: return launch_bwd<4, 8, 16>(a, p, gw, s);
-        default: {
-            WgArgs b = a;
-            b.n_wt = p.n_wt;
-            b.n_dt = p.n_dt;
-            b.n_hc = p.n_hc;
-            b.n_slab = p.n_slab;
-            b.h_chunk = p.h_chunk;
-            b.nblocks = (uint32_t)p.nblocks;
-            using Cfg = BsCfg<4, 512>;
-            hipLaunchKernelGGL(dwconv_bwd_split_kernel<Cfg>, dim3(xcd_padded_grid(b.nblocks)), dim3(Cfg::NT), 0, s, b);
-            rc = check_launch("dwconv_bwd");
-            if (rc != KEROPS_OK) return rc;
-            return reduce_partials(b.ws, p, 64, b.C, gw, s);
-        }
+    WgArgs b = a;
+    b.n_wt = p.n_wt;
+    b.n_dt = p.n_dt;
+    b.n_hc = p.n_hc;
+    b.n_slab = p.n_slab;
+    b.h_chunk = p.h_chunk;
+    b.nblocks = (uint32_t)p.nblocks;
+#define KEROPS_BS_GO(CGv, TWv, TDv)                                                                                  \
+    {                                                                                                                \
+        using Cfg = BsCfg<CGv, TWv, TDv, 512>;                                                                       \
+        hipLaunchKernelGGL(dwconv_bwd_split_kernel<Cfg>, dim3(xcd_padded_grid(b.nblocks)), dim3(Cfg::NT), 0, s, b); \
     }
+    switch (p.cg) {
+        case 1: KEROPS_BS_GO(1, 8, 32) break;
+        case 2: KEROPS_BS_GO(2, 8, 16) break;
+        case 4: KEROPS_BS_GO(4, 8, 8) break;
+        default: KEROPS_BS_GO(8, 4, 8) break;
+    }
+#undef KEROPS_BS_GO
+    rc = check_launch("dwconv_bwd");
+    if (rc != KEROPS_OK) return rc;
+    return reduce_partials(b.ws, p, p.cg * 8, b.C, gw, s);
 }
 
 extern "C" int64_t kerops_dwconv_wgrad_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
