@@ -245,6 +245,29 @@ def main():
                                               clone_gbps)
         ops['QuantUint8Window'] = figures(time_op(torch, lambda: QuantUint8Window(x, 3.0), it, wm)[0], 3 * V * C,
                                           clone_gbps)
+        # the remaining stream ops (backward passes, residual add, dequantiser) on the same tensor
+        from kerops_amd.ops.addition import AddStats, AddStatsBackward
+        from kerops_amd.ops.avgpool import AvgPoolCeilStatsBackward
+        from kerops_amd.ops.bnrelu import ApplyBNReLUBackward
+        from kerops_amd.ops.quantization import DequantUint8Window
+        from kerops_amd.ops.stats import StatsBackward
+        mg = torch.randn(C, device=dev, generator=gen)
+        sg = torch.randn(C, device=dev, generator=gen)
+        ops['StatsBackward'] = figures(time_op(torch, lambda: StatsBackward(x, mg, sg), it, wm)[0], 4 * V * C, clone_gbps)
+        ops['AddStats'] = figures(time_op(torch, lambda: AddStats(x, g), it, wm)[0], 6 * V * C, clone_gbps)
+        ops['AddStatsBackward'] = figures(time_op(torch, lambda: AddStatsBackward(g, mg, sg, x), it, wm)[0], 6 * V * C,
+                                          clone_gbps)
+        ops['ApplyBNReLUBackward'] = figures(time_op(torch, lambda: ApplyBNReLUBackward(x, Wv, Bv, g), it, wm)[0],
+                                             6 * V * C, clone_gbps)
+        pooled = AvgPoolCeilStats(x)[0]
+        gp = torch.randn_like(pooled)
+        ops['AvgPoolCeilStatsBackward'] = figures(
+            time_op(torch, lambda: AvgPoolCeilStatsBackward(gp, mg, sg, pooled, tuple(x.shape)), it, wm)[0],
+            2 * V * C + 4 * pooled.numel(), clone_gbps)
+        q8 = QuantUint8Window(x, 3.0)
+        ops['DequantUint8Window'] = figures(time_op(torch, lambda: DequantUint8Window(q8, torch.float16, 3.0), it, wm)[0],
+                                            3 * V * C, clone_gbps)
+        del pooled, gp, q8
         # the vendor path on the same GPU: torch's own depthwise conv3d (MIOpen) on the same tensor, forward only
         # (its weight gradient takes 2.5 s per call after a 78 s kernel search, so it is not run here)
         try:
