@@ -113,6 +113,56 @@ static inline int pick_h_chunk(int H, int64_t per_plane, int slots, int setup)
     }
     return best_h;
 }
+// Balanced split of the H-marching kernels.  The tiles of the tensor, in their linear order (slab fastest, then
+// the tiles along D, along W, the batch), are cut into bundles of `group` neighbours; the launch has `ngroups`
+// groups of `group` workgroups, and a group owns a contiguous share of the sequence (bundle, row): its workgroups
+// march in step over the tiles of a bundle (they share halo voxels through the L2 of their XCD) and cross into
+// the next bundle together.  Every group then carries the same number of plane steps whatever the tile count,
+// where uniform chunks leave the last round of workgroups partly filled (2-10 % slower at the shapes measured).
+// `row_len` = tiles (times slabs) in one row along D.  The group size is chosen by a cost model fitted to
+// sweeps at (1, C, 350, 350, 128), C = 8..128: time ~ plane steps of a group, 10 % / (tile rows in a bundle) for
+// the halo rows that neighbouring bundles no longer share in L2, a fixed cost per workgroup and per crossing.
+struct BalancedSplit {
+    uint32_t group, ngroups;
+    int64_t units;  // bundles * H
+};
+static inline BalancedSplit make_balanced(int H, int64_t tiles, int slots, int group)
+{
+    BalancedSplit b;
+    b.group = (uint32_t)group;
+    b.units = ((tiles + group - 1) / group) * H;
+    // a share of fewer than 2 rows is all halo planes: use fewer groups then
+    b.ngroups = (uint32_t)std::min<int64_t>(std::max(1, slots / group), std::max<int64_t>(1, b.units / 2));
+    return b;
+}
+static inline double balanced_cost(const BalancedSplit& b, int H, int row_len, int setup)
+{
+    const double share = (double)((b.units + b.ngroups - 1) / b.ngroups);
+    const double crossings = share / H;  // expected bundle boundaries inside a share
+    const double rows = (double)b.group / row_len;
+    return (share + 2 + setup + crossings * 5.0) * (1.0 + 0.1 / rows) * (1.0 + 0.004 * H / share);
+}
+// slab_mult: the group size must be a multiple of it (kernels that keep per-slab state across bundles)
+static inline BalancedSplit pick_balanced(int H, int64_t tiles, int row_len, int slots, int setup, int slab_mult)
+{
+    BalancedSplit best = make_balanced(H, tiles, slots, slab_mult);
+    double best_cost = 1e300;
+    auto consider = [&](int64_t g) {
+        if (g < 1 || g > slots || g % slab_mult != 0) return;
+        if (g >= tiles + row_len && g > slab_mult) return;  // more than a row of idle members
+        const BalancedSplit b = make_balanced(H, tiles, slots, (int)g);
+        const double c = balanced_cost(b, H, row_len, setup);
+        if (c < best_cost) {
+            best_cost = c;
+            best = b;
+        }
+    };
+    for (int r = 1; r <= 16; ++r) consider((int64_t)r * row_len);             // whole tile rows
+    for (int f = 2; f <= 8; f *= 2)                                           // parts of a long row
+        if (row_len % f == 0) consider(row_len / f);
+    consider(slab_mult);
+    return best;
+}
 // offsets inside one (W, D, C) plane are 32-bit in the convolution kernels (W, D, C positive)
 static inline bool plane_exceeds_i32(int W, int D, int C)
 {

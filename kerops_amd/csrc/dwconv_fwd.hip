@@ -60,6 +60,9 @@ struct FwdArgs {
     int H, W, D, C;
     int n_wt, n_dt, n_hc, n_slab, h_chunk;
     uint32_t nblocks;
+    // balanced split (matrix-core kernel, modes 0 and 1): bal_group > 0 switches it on
+    uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
+    uint32_t n_tiles;                  // tiles in the tensor
 };
 
 // Packed weights of one thread: for every weight row kh and every channel j of the lane,
@@ -482,23 +485,58 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
     __shared__ float amax_red[Cfg::NWAVE];
 
-    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
-    if (L >= a.nblocks) return;
-    const uint32_t wg_slot = L;
+    const uint32_t wg_slot = remap_xcd(blockIdx.x, a.nblocks);
+    if (wg_slot >= a.nblocks) return;
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    // Work of this workgroup: one (tile, row range) segment with uniform chunks, or, in the balanced split, its
+    // group's contiguous share [u, u_end) of the (bundle of bal_group tiles, row) sequence: the workgroups of a
+    // group march in step over neighbouring tiles (member = tile inside the bundle) and cross into the next
+    // bundle together, so that every group carries the same number of plane steps.
+    constexpr bool SEGMENTS = MODE == 0 || MODE == 1;  // the other modes always run one segment (uniform chunks)
+    const bool balanced = SEGMENTS && a.bal_group > 0;
+    uint32_t u = 0, u_end = 0, member = 0;  // wavefront-uniform, kept in scalar registers
+    if (balanced) {
+        const uint32_t group = wg_slot / a.bal_group;
+        member = wg_slot - group * a.bal_group;
+        // shares of bal_q or bal_q + 1 units: the first bal_r groups take the longer ones
+        u = __builtin_amdgcn_readfirstlane(group * a.bal_q + min(group, a.bal_r));
+        u_end = __builtin_amdgcn_readfirstlane(u + a.bal_q + (group < a.bal_r ? 1u : 0u));
+    }
+    for (bool first = true;; first = false) {
+    // The thread index is made opaque per segment: everything derived from it is then computed inside the segment
+    // and dies with the prologue, instead of being hoisted out of this loop and held in registers across the march.
+    int t = threadIdx.x;
+    if constexpr (SEGMENTS) asm volatile("" : "+v"(t));
+    uint32_t L;
+    int hs, he;
+    if (balanced) {
+        if (u >= u_end) break;
+        const uint32_t bundle = u / (uint32_t)H;
+        hs = (int)(u - bundle * (uint32_t)H);
+        he = (int)min((uint32_t)H, hs + (u_end - u));
+        u += he - hs;
+        L = bundle * a.bal_group + member;
+        if (L >= a.n_tiles) continue;  // a partly filled last bundle
+    } else {
+        if (!first) break;
+        L = wg_slot;
+    }
     const int slab = L % a.n_slab;
     L /= a.n_slab;
     const int dt = L % a.n_dt;
     L /= a.n_dt;
     const int wt_i = L % a.n_wt;
     L /= a.n_wt;
-    const int hc = L % a.n_hc;
-    const int n = L / a.n_hc;
-
-    const int t = threadIdx.x;
-    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    int n;
+    if (balanced) {
+        n = L;
+    } else {
+        const int hc = L % a.n_hc;
+        n = L / a.n_hc;
+        hs = hc * a.h_chunk;
+        he = min(hs + a.h_chunk, H);
+    }
     const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
-    const int hs = hc * a.h_chunk;
-    const int he = min(hs + a.h_chunk, H);
     const int cslab = slab * SC;
     const int64_t plane_stride = (int64_t)W * D * C;
     const half_t* xn = a.x + (int64_t)n * H * plane_stride;
@@ -762,7 +800,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     if constexpr (BOUNCE) {
         __syncthreads();
         flush_row(parity ^ 1);
+    } else {
+        if (balanced) __syncthreads();  // the staging buffers are free before the next segment refills them
     }
+    if constexpr (SEGMENTS) continue;  // the other modes run one segment and finish below
     if constexpr (STATS) {
         // lanes of a wavefront that share the channel pair differ in rr (lane bits 0-1) and sub (the bits above q)
         float v4[4] = {ssum[0], ssum[1], ssq[0], ssq[1]};
@@ -803,19 +844,44 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
             a.amax_ws[wg_slot] = m;
         }
     }
+    break;
+    }  // segments
 }
 
 // grid of the matrix-core kernels: fills the n_* fields and nblocks of `a`
 template <int CG, int TW, int TD, int NT>
-static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk)
+static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk, bool balanced_ok = false)
 {
     a.n_slab = a.C / (CG * 8);
     a.n_wt = ceil_div(a.W, TW);
     a.n_dt = ceil_div(a.D, TD);
+    a.bal_group = 0;
+    const int slots = NT >= 512 ? 512 : 1024;  // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each
+    // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups) for the kernels
+    // that support it; > 0: uniform chunks of that many rows
+    if (h_chunk < 0 || (h_chunk == 0 && balanced_ok)) {
+        const int64_t tiles = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
+        const BalancedSplit b = h_chunk < 0 ? make_balanced(a.H, tiles, slots, -h_chunk)
+                                            : pick_balanced(a.H, tiles, a.n_dt * a.n_slab, slots, 6, 1);
+        const bool fits = b.units < (1LL << 31) && tiles + b.group < (1LL << 31);  // 32-bit counters in the kernel
+        if (!fits && h_chunk < 0) {
+            set_error("dwconv_fwd: too many plane steps for the balanced split");
+            return KEROPS_E_BADARG;
+        }
+        if (fits) {
+            a.bal_group = b.group;
+            a.bal_q = (uint32_t)(b.units / b.ngroups);
+            a.bal_r = (uint32_t)(b.units % b.ngroups);
+            a.n_tiles = (uint32_t)tiles;
+            a.h_chunk = a.H;
+            a.n_hc = 1;
+            a.nblocks = b.group * b.ngroups;
+            return KEROPS_OK;
+        }
+    }
     if (h_chunk <= 0) {
-        // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each
         const int64_t per_plane = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
-        h_chunk = pick_h_chunk(a.H, per_plane, NT >= 512 ? 512 : 1024, 6);
+        h_chunk = pick_h_chunk(a.H, per_plane, slots, 6);
     }
     h_chunk = std::min(h_chunk, a.H);
     a.h_chunk = h_chunk;
@@ -834,7 +900,7 @@ static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t 
 {
     using Cfg = FmCfg<CG, TW, TD, NT>;
     FwdArgs a = base;
-    int rc = plan_fwd_mfma<CG, TW, TD, NT>(a, N, h_chunk);
+    int rc = plan_fwd_mfma<CG, TW, TD, NT>(a, N, h_chunk, true);
     if (rc != KEROPS_OK) return rc;
     if (a.scale) {
         hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 1>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,

@@ -50,6 +50,9 @@ struct WgArgs {
     int H, W, D, C;
     int n_wt, n_dt, n_hc, n_slab, h_chunk;
     uint32_t nblocks;
+    // balanced split (matrix-core weight-gradient kernel): bal_group > 0 switches it on, see pick_balanced
+    uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
+    uint32_t n_tiles;                  // tiles in the tensor
 };
 
 __device__ __forceinline__ half2_t pack_lo(uint32_t a, uint32_t b)
@@ -349,23 +352,79 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
     constexpr int NLDX = Cfg::NLDX, NLDG = Cfg::NLDG;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
-    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
-    if (L >= a.nblocks) return;
-    const uint32_t ws_slot = L;
+    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
+    if (ws_slot >= a.nblocks) return;
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
+
+    // operand gathering: lane = (block b, index rr); block = (channel pair q, position group sub)
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int half = wave % Cfg::NHALF, part = wave / Cfg::NHALF;
+    const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RG;  // this wavefront: position group, first g row
+    const int b = lane / 4, rr = lane % 4;
+    const int q = b % NQ, sub = b / NQ;
+    const int r2 = min(rr, 2);  // index 3 repeats index 2: its results are never used
+    const int cb = half * 64 + q * 4;
+    const int pgrp = (gd * NSUB + sub) * 4;  // first position of the lane's group inside a row
+    int aoff[4], boff[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        aoff[k] = Cfg::XOFF + Cfg::swz(ra * PDP + pgrp + r2 + k, cb);  // x row ra (patch row ra-1), window r2
+        boff[k] = Cfg::swz(ra * TD + pgrp + k, cb);                     // g row ra; the slot is added per step
+    }
+
+    // the sums run over every segment of the workgroup: all its tiles belong to the same slab
+    float4_t acc[3][2];
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Work of this workgroup: one (tile, row range) segment with uniform chunks, or, in the balanced split, its
+    // group's contiguous share [u, u_end) of the (bundle of bal_group tiles, row) sequence (see pick_balanced).
+    const bool balanced = a.bal_group > 0;
+    uint32_t u = 0, u_end = 0, member = 0;  // wavefront-uniform, kept in scalar registers
+    if (balanced) {
+        const uint32_t group = ws_slot / a.bal_group;
+        member = ws_slot - group * a.bal_group;
+        u = __builtin_amdgcn_readfirstlane(group * a.bal_q + min(group, a.bal_r));
+        u_end = __builtin_amdgcn_readfirstlane(u + a.bal_q + (group < a.bal_r ? 1u : 0u));
+    }
+    for (bool first = true;; first = false) {
+    // the thread index is made opaque per segment: the staging assignment derived from it is then computed inside
+    // the segment instead of being hoisted out of this loop and held in registers across the march
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    uint32_t L;
+    int hs, he;
+    if (balanced) {
+        if (u >= u_end) break;
+        const uint32_t bundle = u / (uint32_t)H;
+        hs = (int)(u - bundle * (uint32_t)H);
+        he = (int)min((uint32_t)H, hs + (u_end - u));
+        u += he - hs;
+        L = bundle * a.bal_group + member;
+        if (L >= a.n_tiles) continue;  // a partly filled last bundle
+        if (!first) __syncthreads();   // the previous segment's last plane has been read by every wavefront
+    } else {
+        if (!first) break;
+        L = ws_slot;
+    }
     const int slab = L % a.n_slab;
     L /= a.n_slab;
     const int dt = L % a.n_dt;
     L /= a.n_dt;
     const int wt_i = L % a.n_wt;
     L /= a.n_wt;
-    const int hc = L % a.n_hc;
-    const int n = L / a.n_hc;
-
-    const int t = threadIdx.x;
-    const int H = a.H, W = a.W, D = a.D, C = a.C;
+    int n;
+    if (balanced) {
+        n = L;
+    } else {
+        const int hc = L % a.n_hc;
+        n = L / a.n_hc;
+        hs = hc * a.h_chunk;
+        he = min(hs + a.h_chunk, H);
+    }
     const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
-    const int hs = hc * a.h_chunk;
-    const int he = min(hs + a.h_chunk, H);
     const int cslab = slab * SC;
     const int64_t plane_stride = (int64_t)W * D * C;
     const half_t* xn = a.x + (int64_t)n * H * plane_stride;
@@ -402,28 +461,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
         ggo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
         gls[j] = ok ? Cfg::swz(wq * TD + dq, cq * 16) : -1;
     }
-
-    // operand gathering: lane = (block b, index rr); block = (channel pair q, position group sub)
-    const int lane = t % kWave, wave = t / kWave;
-    const int half = wave % Cfg::NHALF, part = wave / Cfg::NHALF;
-    const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RG;  // this wavefront: position group, first g row
-    const int b = lane / 4, rr = lane % 4;
-    const int q = b % NQ, sub = b / NQ;
-    const int r2 = min(rr, 2);  // index 3 repeats index 2: its results are never used
-    const int cb = half * 64 + q * 4;
-    const int pgrp = (gd * NSUB + sub) * 4;  // first position of the lane's group inside a row
-    int aoff[4], boff[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        aoff[k] = Cfg::XOFF + Cfg::swz(ra * PDP + pgrp + r2 + k, cb);  // x row ra (patch row ra-1), window r2
-        boff[k] = Cfg::swz(ra * TD + pgrp + k, cb);                     // g row ra; the slot is added per step
-    }
-
-    float4_t acc[3][2];
-#pragma unroll
-    for (int kw = 0; kw < 3; ++kw)
-#pragma unroll
-        for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
     // They are unconditional (plane indices are clamped, values of planes that do not exist or lie
@@ -504,7 +541,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
         step(hp, xpre1, gpre1);
         if (++hp > he) break;
     }
+    }  // segments
 
+    const int t = threadIdx.x;
     // ---- combine: position groups inside a wavefront, then the wavefronts of a half via LDS ----
     if (NSUB > 1) {
 #pragma unroll
@@ -917,6 +956,7 @@ __global__ __launch_bounds__(1024) void wgrad_reduce_kernel(const float* __restr
 struct WgPlan {
     int cg, tile_w, tile_d, cl, h_chunk, n_wt, n_dt, n_hc, n_slab;
     int64_t nblocks;
+    uint32_t bal_group = 0, bal_q = 0, bal_r = 0, n_tiles = 0;  // balanced split (bal_group > 0), see pick_balanced
 };
 
 static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d, int h_chunk, int lane_channels,
@@ -951,12 +991,38 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     p->n_slab = C / (p->cg * 8);
     p->n_wt = ceil_div(W, tile_w);
     p->n_dt = ceil_div(D, tile_d);
-    if (h_chunk <= 0) {
-        // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each; every workgroup also leaves one partial
-        const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-        const bool big_wg = p->cg == 8 && (tile_w * tile_d >= 64);
-        h_chunk = pick_h_chunk(H, per_plane, big_wg ? 512 : 1024, 8);
+    // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each; every workgroup also leaves one partial
+    const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
+    const bool big_wg = p->cg == 8 && (tile_w * tile_d >= 64);
+    const int slots = big_wg ? 512 : 1024;
+    p->bal_group = 0;
+    // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups; matrix-core
+    // kernels only); > 0: uniform chunks of that many rows
+    if (lane_channels == 16 && h_chunk <= 0) {
+        if (h_chunk < 0 && (-h_chunk) % p->n_slab != 0) {
+            set_error("dwconv_wgrad: the group size of the balanced split must be a multiple of the slab count %d",
+                      p->n_slab);
+            return KEROPS_E_BADARG;
+        }
+        const BalancedSplit b = h_chunk < 0 ? make_balanced(H, per_plane, slots, -h_chunk)
+                                            : pick_balanced(H, per_plane, p->n_dt * p->n_slab, slots, 8, p->n_slab);
+        const bool fits = b.units < (1LL << 31) && per_plane + b.group < (1LL << 31);  // 32-bit counters in the kernel
+        if (!fits && h_chunk < 0) {
+            set_error("dwconv_wgrad: too many plane steps for the balanced split");
+            return KEROPS_E_BADARG;
+        }
+        if (fits) {
+            p->bal_group = b.group;
+            p->bal_q = (uint32_t)(b.units / b.ngroups);
+            p->bal_r = (uint32_t)(b.units % b.ngroups);
+            p->n_tiles = (uint32_t)per_plane;
+            p->h_chunk = H;
+            p->n_hc = 1;
+            p->nblocks = (int64_t)b.group * b.ngroups;
+            return KEROPS_OK;
+        }
     }
+    if (h_chunk <= 0) h_chunk = pick_h_chunk(H, per_plane, slots, 8);
     p->h_chunk = std::min(h_chunk, H);
     p->n_hc = ceil_div(H, p->h_chunk);
     p->nblocks = (int64_t)N * p->n_hc * p->n_wt * p->n_dt * p->n_slab;
@@ -993,6 +1059,10 @@ static int launch_wgrad_cfg(KernelT kernel, const WgArgs& base, const WgPlan& p,
     a.n_slab = p.n_slab;
     a.h_chunk = p.h_chunk;
     a.nblocks = (uint32_t)p.nblocks;
+    a.bal_group = p.bal_group;
+    a.bal_q = p.bal_q;
+    a.bal_r = p.bal_r;
+    a.n_tiles = p.n_tiles;
     hipLaunchKernelGGL(kernel, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
     int rc = check_launch("dwconv_wgrad");
     if (rc != KEROPS_OK) return rc;
