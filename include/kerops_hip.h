@@ -25,6 +25,13 @@
  *    launch-shape knobs (patch extents along W and D, rows of H one workgroup
  *    marches over, channels one lane owns, workgroup count); 0 selects the built-in
  *    choice for gfx950, an unbuilt combination returns KEROPS_E_BADARG.
+ *    For kerops_dwconv_fwd_f16 and kerops_dwconv_wgrad_f16 with the matrix-core
+ *    kernels, h_chunk > 0 cuts H into uniform chunks of that many rows, one per
+ *    workgroup; h_chunk = 0 is the balanced split: as many workgroups as the GPU
+ *    holds at once, in groups that each own an equal, contiguous share of the
+ *    (bundle of neighbouring patches, row) sequence and march over it in step;
+ *    h_chunk = -g selects that split with groups of g workgroups (for the weight
+ *    gradient g must be a multiple of C / 64 when C > 64).
  */
 #ifndef KEROPS_HIP_H
 #define KEROPS_HIP_H

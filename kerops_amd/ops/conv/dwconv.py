@@ -64,9 +64,11 @@ def DWConv(
     fp32 ('float16' is accepted and computed in fp32), num_warps is the number of
     64-wide wavefronts per workgroup (fixed per patch shape in the library: 4, or 8 for the
     8x8 patch) and D_block the tile
-    extent along D.  W_block (tile extent along W) and H_chunk (rows one workgroup
-    marches over, 0 = automatic) and lane_channels (16 = matrix-core kernels, the default;
-    2 or 4 = vector kernels with that many channels per lane) are additional gfx950 knobs.
+    extent along D.  W_block (tile extent along W), H_chunk (> 0: rows one workgroup marches
+    over; 0: the balanced split, in which groups of workgroups share out the rows of all
+    patches evenly; -g: that split with groups of g workgroups) and lane_channels (16 =
+    matrix-core kernels, the default; 2 or 4 = vector kernels with that many channels per
+    lane) are additional gfx950 knobs.
     """
     channels = x.shape[1]
 

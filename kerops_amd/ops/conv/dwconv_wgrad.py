@@ -61,7 +61,12 @@ def DWConvWGRAD(
     lane_channels: ConfigurableArg,
     out_dtype: ConfigurableArg,
 ):
-    """grad_w[kh,kw,kd,c] = sum_{n,h,w,d} grad[n,c,h,w,d] * x[n,c,h+kh-1,w+kw-1,d+kd-1]."""
+    """grad_w[kh,kw,kd,c] = sum_{n,h,w,d} grad[n,c,h,w,d] * x[n,c,h+kh-1,w+kw-1,d+kd-1].
+
+    H_chunk > 0: rows one workgroup marches over; 0: the balanced split (groups of workgroups share out the
+    rows of all patches evenly); -g: that split with groups of g workgroups.  The split fixes the order of the
+    fp32 additions: the same call always returns the same bits, different splits differ in the last bits.
+    """
     channels = x.shape[1]
 
     assert x.ndim == grad.ndim == 5

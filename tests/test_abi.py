@@ -97,21 +97,34 @@ def test_workspace_queries():
 
 def test_h_chunk_choice_fills_whole_rounds():
     # workgroup counts of the built-in launch shapes, read back from the workspace sizes (one partial per
-    # workgroup): 1408 = 2.75 per resident slot at the README shape (the measured optimum), exactly one round of
-    # 512 (or 1024 narrower) workgroups at 128^3-class volumes instead of several short chunks
+    # workgroup).  Uniform chunks (the convolution + statistics kernel): 1408 = 2.75 per resident slot at the README
+    # shape (the measured optimum), exactly one round of 512 workgroups at 128^3-class volumes instead of several
+    # short chunks.  The weight gradient uses the balanced split: never more workgroups than the GPU holds at once
+    # (512 of 512 threads, 1024 of 256), all of them busy at the large shapes.
     lib = _lib.load()
 
-    def wgrad_blocks(n, h, w, d, c):
-        return lib.kerops_dwconv_wgrad_workspace_bytes(n, h, w, d, c, 0, 0, 0, 0) // (27 * min(c, 64) * 4)
+    def wgrad_blocks(n, h, w, d, c, h_chunk=0):
+        return lib.kerops_dwconv_wgrad_workspace_bytes(n, h, w, d, c, 0, 0, h_chunk, 0) // (27 * min(c, 64) * 4)
 
     def fwd_blocks(n, h, w, d, c):
         return lib.kerops_dwconv_stats_workspace_bytes(n, h, w, d, c) // (2 * min(c, 64) * 4)
 
-    assert wgrad_blocks(1, 350, 350, 128, 64) == 1408 and fwd_blocks(1, 350, 350, 128, 64) == 1408
-    assert wgrad_blocks(1, 128, 128, 128, 64) == 512 and fwd_blocks(1, 128, 128, 128, 64) == 512
-    assert wgrad_blocks(2, 128, 128, 128, 32) == 1024 and fwd_blocks(2, 128, 128, 128, 32) == 512
+    assert fwd_blocks(1, 350, 350, 128, 64) == 1408
+    assert fwd_blocks(1, 128, 128, 128, 64) == 512
+    assert fwd_blocks(2, 128, 128, 128, 32) == 512
     assert fwd_blocks(1, 350, 350, 128, 128) == 4 * 1408  # four chunks of 88 rows: 11 whole rounds
-    assert fwd_blocks(1, 1, 8, 8, 64) == 1 and wgrad_blocks(1, 1, 8, 8, 8) == 1
+    assert fwd_blocks(1, 1, 8, 8, 64) == 1
+
+    assert wgrad_blocks(1, 350, 350, 128, 64) == 512      # 8 groups of 64 = 4 rows of 16 patches
+    assert wgrad_blocks(1, 350, 350, 128, 128) == 512     # 4 groups of 128 = 4 rows of 16 patches x 2 slabs
+    assert wgrad_blocks(1, 350, 350, 128, 8) in range(960, 1025)
+    assert wgrad_blocks(1, 128, 128, 128, 64) == 512
+    assert wgrad_blocks(1, 1, 8, 8, 8) == 1
+    # uniform chunks on request: patches x chunks; explicit groups: group x groups
+    assert wgrad_blocks(1, 350, 350, 128, 64, 175) == 1408
+    assert wgrad_blocks(1, 350, 350, 128, 64, -32) == 512
+    # a group that is not a multiple of the two slabs of 128 channels is refused
+    assert lib.kerops_dwconv_wgrad_workspace_bytes(1, 350, 350, 128, 128, 0, 0, -3, 0) == _lib.KEROPS_E_BADARG
 
 
 def cl3d(*shape, dtype=torch.float16):

@@ -147,6 +147,49 @@ def test_every_built_launch_shape(c):
         assert rel < 2e-6, (tw, td, cl, hc, rel)
 
 
+@pytest.mark.parametrize('c', [8, 16, 32, 64, 128])
+def test_balanced_split_small(c):
+    """The balanced split of the H march (H_chunk = 0, and explicit group sizes -g): shares that end inside a
+    bundle of patches, a partly filled last bundle, groups larger than the tensor, group sizes that do not divide
+    the resident workgroup count, several samples.  The forward result does not depend on the split (bit-identical
+    to one uniform chunk, itself checked against the oracle); the weight gradient is checked against the oracle."""
+    g = cpu_gen(11)
+    shape = (3, c, 13, 21, 37)
+    x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    _, wk = rand_dw_weight(g, c)
+    xd, gd, wd = x.to(DEV), grad.to(DEV), wk.to(DEV)
+    one_chunk = DWConv(xd, wd, H_chunk=100)
+    check_fwd(x, wk, one_chunk)
+    for hc in (0, -1, -2, -3, -4, -7, -16, -64, -600):
+        assert torch.equal(DWConv(xd, wd, H_chunk=hc), one_chunk), hc
+    ref_gw = oracle.dwconv_wgrad(x, grad)
+    for hc in (0, -2, -4, -6, -16, -64, -600):
+        gw = DWConvWGRAD(xd, gd, H_chunk=hc, out_dtype=torch.float32)
+        rel = ((gw.cpu().double() - ref_gw).norm() / ref_gw.norm()).item()
+        assert rel < 2e-6, (hc, rel)
+        assert torch.equal(gw, DWConvWGRAD(xd, gd, H_chunk=hc, out_dtype=torch.float32)), hc  # deterministic
+
+
+@pytest.mark.parametrize('shape', [(1, 8, 9, 300, 1000), (1, 16, 9, 300, 600), (1, 32, 9, 200, 400),
+                                   (1, 64, 9, 260, 260), (1, 128, 9, 130, 260), (2, 64, 5, 260, 130)])
+def test_balanced_split_many_patches(shape):
+    """More patches than resident workgroups: every group owns several bundles and crosses from one into the next
+    in the middle of its share (for 128 channels with both slabs in a bundle); the last bundle holds a single
+    patch.  Compared on the GPU with uniform chunks of the whole height, which the tests above pin to the oracle."""
+    g = torch.Generator(DEV).manual_seed(sum(shape))
+    n, c, h, w, d = shape
+    xd = torch.randn(n, h, w, d, c, device=DEV, dtype=torch.float16, generator=g).permute(0, 4, 1, 2, 3)
+    gd = torch.randn(n, h, w, d, c, device=DEV, dtype=torch.float16, generator=g).permute(0, 4, 1, 2, 3)
+    wd = (torch.randn(3, 3, 3, c, device=DEV, generator=g) / 5).half()
+    y_uniform = DWConv(xd, wd, H_chunk=h)
+    gw_uniform = DWConvWGRAD(xd, gd, H_chunk=h, out_dtype=torch.float32)
+    for hc in (0, -64, -128, -34):
+        assert torch.equal(DWConv(xd, wd, H_chunk=hc), y_uniform), hc
+        gw = DWConvWGRAD(xd, gd, H_chunk=hc, out_dtype=torch.float32)
+        rel = ((gw.double() - gw_uniform.double()).norm() / gw_uniform.double().norm()).item()
+        assert rel < 2e-6, (hc, rel)
+
+
 def test_golden_vectors(golden):
     x = from_bits(golden['x']).to(memory_format=torch.channels_last_3d)
     grad = from_bits(golden['grad']).to(memory_format=torch.channels_last_3d)
