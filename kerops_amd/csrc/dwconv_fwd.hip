@@ -492,8 +492,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     // group's contiguous share [u, u_end) of the (bundle of bal_group tiles, row) sequence: the workgroups of a
     // group march in step over neighbouring tiles (member = tile inside the bundle) and cross into the next
     // bundle together, so that every group carries the same number of plane steps.
-    constexpr bool SEGMENTS = MODE == 0 || MODE == 1;  // the other modes always run one segment (uniform chunks)
+    constexpr bool SEGMENTS = MODE != 2;  // the fused pointwise mode always runs one segment (uniform chunks)
     const bool balanced = SEGMENTS && a.bal_group > 0;
+    // mode 3: sums over the lane's channel pair, carried over every segment (all tiles of a workgroup belong to
+    // the same slab: the group size is a multiple of the slab count)
+    float ssum[2] = {0.0f, 0.0f}, ssq[2] = {0.0f, 0.0f};
     uint32_t u = 0, u_end = 0, member = 0;  // wavefront-uniform, kept in scalar registers
     if (balanced) {
         const uint32_t group = wg_slot / a.bal_group;
@@ -651,7 +654,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     for (int o = 0; o < RO; ++o)
 #pragma unroll
         for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float ssum[2] = {0.0f, 0.0f}, ssq[2] = {0.0f, 0.0f};  // mode 3: this lane's channel pair
 
     // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
     // They are unconditional (plane indices are clamped; planes that do not exist are never used):
@@ -803,8 +805,25 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     } else {
         if (balanced) __syncthreads();  // the staging buffers are free before the next segment refills them
     }
-    if constexpr (SEGMENTS) continue;  // the other modes run one segment and finish below
+    if constexpr (SEGMENTS) continue;  // the fused pointwise mode runs one segment and finishes here
+    if constexpr (MODE == 2) {
+        amax = wave_max(amax);
+        if (lane == 0) amax_red[wave] = amax;
+        __syncthreads();
+        if (t == 0) {
+            float m = amax_red[0];
+#pragma unroll
+            for (int wv = 1; wv < Cfg::NWAVE; ++wv) m = fmaxf(m, amax_red[wv]);
+            a.amax_ws[wg_slot] = m;
+        }
+    }
+    break;
+    }  // segments
     if constexpr (STATS) {
+        const int t = threadIdx.x;
+        const int lane = t % kWave, wave = t / kWave;
+        const int b = lane / 4, rr = lane % 4;
+        const int q = b % NQ, sub = b / NQ;
         // lanes of a wavefront that share the channel pair differ in rr (lane bits 0-1) and sub (the bits above q)
         float v4[4] = {ssum[0], ssum[1], ssq[0], ssq[1]};
 #pragma unroll
@@ -833,24 +852,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
             a.stats_ws[(int64_t)wg_slot * 2 * SC + st * SC + ch] = acc;
         }
     }
-    if constexpr (MODE == 2) {
-        amax = wave_max(amax);
-        if (lane == 0) amax_red[wave] = amax;
-        __syncthreads();
-        if (t == 0) {
-            float m = amax_red[0];
-#pragma unroll
-            for (int wv = 1; wv < Cfg::NWAVE; ++wv) m = fmaxf(m, amax_red[wv]);
-            a.amax_ws[wg_slot] = m;
-        }
-    }
-    break;
-    }  // segments
 }
 
 // grid of the matrix-core kernels: fills the n_* fields and nblocks of `a`
 template <int CG, int TW, int TD, int NT>
-static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk, bool balanced_ok = false)
+static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk, bool balanced_ok = false, bool per_slab_state = false)
 {
     a.n_slab = a.C / (CG * 8);
     a.n_wt = ceil_div(a.W, TW);
@@ -862,7 +868,8 @@ static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk, bool balanced_ok = fals
     if (h_chunk < 0 || (h_chunk == 0 && balanced_ok)) {
         const int64_t tiles = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
         const BalancedSplit b = h_chunk < 0 ? make_balanced(a.H, tiles, slots, -h_chunk)
-                                            : pick_balanced(a.H, tiles, a.n_dt * a.n_slab, slots, 6, 1);
+                                            : pick_balanced(a.H, tiles, a.n_dt * a.n_slab, slots, 6,
+                                                            per_slab_state ? a.n_slab : 1);
         const bool fits = b.units < (1LL << 31) && tiles + b.group < (1LL << 31);  // 32-bit counters in the kernel
         if (!fits && h_chunk < 0) {
             set_error("dwconv_fwd: too many plane steps for the balanced split");
@@ -1143,7 +1150,7 @@ extern "C" int64_t kerops_dwconv_stats_workspace_bytes(int32_t N, int32_t H, int
     a.D = D;
     a.C = C;
     rc = with_stats_shape(C, [&](auto cg, auto tw, auto td, auto nt) {
-        return plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0);
+        return plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0, true, true);
     });
     if (rc != KEROPS_OK) return rc;
     return (int64_t)a.nblocks * 2 * std::min(C, 64) * (int64_t)sizeof(float);
@@ -1176,7 +1183,7 @@ extern "C" int kerops_dwconv_stats_f16(const void* x, const void* wt, void* y, f
     hipStream_t s = (hipStream_t)stream;
     int rc = with_stats_shape(C, [&](auto cg, auto tw, auto td, auto nt) {
         using Cfg = FmCfg<cg(), tw(), td(), nt()>;
-        int r = plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0);
+        int r = plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0, true, true);
         if (r != KEROPS_OK) return r;
         hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
         return check_launch("dwconv_stats");

@@ -621,64 +621,105 @@ struct BsCfg {
 };
 
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs a)
+__global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_split_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
     constexpr bool BOUNCE = Cfg::BOUNCE;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
-    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
-    if (L >= a.nblocks) return;
-    const uint32_t ws_slot = L;
-    const int slab = L % a.n_slab;
-    L /= a.n_slab;
-    const int dt = L % a.n_dt;
-    L /= a.n_dt;
-    const int wt_i = L % a.n_wt;
-    L /= a.n_wt;
-    const int hc = L % a.n_hc;
-    const int n = L / a.n_hc;
-
+    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
+    if (ws_slot >= a.nblocks) return;
     const int t = threadIdx.x;
     const int H = a.H, W = a.W, D = a.D, C = a.C;
-    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
-    const int hs = hc * a.h_chunk;
-    const int he = min(hs + a.h_chunk, H);
-    const int cslab = slab * SC;
     const int64_t plane_stride = (int64_t)W * D * C;
-    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
-    const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
-    half_t* dxn = a.dx + (int64_t)n * H * plane_stride;
-
     const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int o = t * 16; o < Cfg::STAGE_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
-
-    // staging: thread t owns chunk t of the patch with halo (x and g alike); threads without a chunk inside the
-    // volume load the plane's first chunk and write it to the dump slot
-    uint32_t go;
-    int ls;
-    {
-        const int wq = t / ((TD + 2) * CG);
-        const int rem = t - wq * ((TD + 2) * CG);
-        const int dq = rem / CG, cq = rem - dq * CG;
-        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
-        const bool ok = (t < Cfg::NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
-        go = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
-        ls = ok ? lds_swizzle<PB>(wq * PDP + dq, cq * 16) : -1;
-    }
 
     const int lane = t % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
     const int role = wave / Cfg::RWAVES, rwave = wave % Cfg::RWAVES;  // 0: input gradient, 1: weight gradient
     const int half = rwave % Cfg::NHALF, part = rwave / Cfg::NHALF;
     const int gd = part % Cfg::GD, ra = (part / Cfg::GD) * RO;
-    const int b = lane / 4, rr = lane % 4;
-    const int q = b % NQ, sub = b / NQ;  // block = (channel pair, group of four positions)
-    const int r2 = min(rr, 2);
-    const int cb = half * 64 + q * 4;
-    const int c0 = cslab + half * 32 + 2 * q;
-    const int pgrp = (gd * NSUB + sub) * 4;
+    // every tile of a workgroup belongs to the same slab (uniform chunks: one tile; balanced split: the group
+    // size is a multiple of the slab count)
+    const int cslab = (int)(ws_slot % (uint32_t)a.n_slab) * SC;
+
+    // Work of this workgroup: one (tile, row range) segment with uniform chunks, or, in the balanced split, its
+    // group's contiguous share [u, u_end) of the (bundle of bal_group tiles, row) sequence (see pick_balanced).
+    // Both roles walk the same segments with the same sequence of workgroup barriers.
+    const bool balanced = a.bal_group > 0;
+    uint32_t u = 0, u_end = 0, member = 0;  // wavefront-uniform, kept in scalar registers
+    if (balanced) {
+        const uint32_t group = ws_slot / a.bal_group;
+        member = ws_slot - group * a.bal_group;
+        u = __builtin_amdgcn_readfirstlane(group * a.bal_q + min(group, a.bal_r));
+        u_end = __builtin_amdgcn_readfirstlane(u + a.bal_q + (group < a.bal_r ? 1u : 0u));
+    }
+    bool first = true;
+    // the segment in hand
+    int hs = 0, he = 0, w0 = 0, d0 = 0;
+    const half_t* xn = a.x;
+    const half_t* gn_ptr = a.g;
+    half_t* dxn = a.dx;
+    uint32_t go = 0;  // staging: thread t owns chunk t of the patch with halo (x and g alike); threads without a
+    int ls = -1;      // chunk inside the volume load the plane's first chunk and write it to the dump slot
+    auto next_segment = [&]() -> bool {  // workgroup-uniform
+        uint32_t L;
+        for (;;) {
+            if (balanced) {
+                if (u >= u_end) return false;
+                const uint32_t bundle = u / (uint32_t)H;
+                hs = (int)(u - bundle * (uint32_t)H);
+                he = (int)min((uint32_t)H, hs + (u_end - u));
+                u += he - hs;
+                L = bundle * a.bal_group + member;
+                if (L >= a.n_tiles) continue;  // a partly filled last bundle
+            } else {
+                if (!first) return false;
+                L = ws_slot;
+            }
+            break;
+        }
+        first = false;
+        L /= a.n_slab;
+        const int dt = L % a.n_dt;
+        L /= a.n_dt;
+        const int wt_i = L % a.n_wt;
+        L /= a.n_wt;
+        int n;
+        if (balanced) {
+            n = L;
+        } else {
+            const int hc = L % a.n_hc;
+            n = L / a.n_hc;
+            hs = hc * a.h_chunk;
+            he = min(hs + a.h_chunk, H);
+        }
+        // the decoded values are wavefront-uniform but come out of vector divisions: back to scalar registers
+        n = __builtin_amdgcn_readfirstlane(n);
+        hs = __builtin_amdgcn_readfirstlane(hs);
+        he = __builtin_amdgcn_readfirstlane(he);
+        w0 = __builtin_amdgcn_readfirstlane(wt_i * Cfg::TW);
+        d0 = __builtin_amdgcn_readfirstlane(dt * TD);
+        xn = a.x + (int64_t)n * H * plane_stride;
+        gn_ptr = a.g + (int64_t)n * H * plane_stride;
+        dxn = a.dx + (int64_t)n * H * plane_stride;
+        // what staging never writes must read as zero (positions outside the volume, g planes before the chunk); the
+        // previous segment's barrier after its last plane makes the buffers free.  The output tiles behind the
+        // staging buffers are left alone: the other role may still be storing the last one.
+        for (int o = t * 16; o < Cfg::OT_OFF; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
+        // an opaque copy of the thread index keeps this assignment from being hoisted out of the segment loop
+        int ts = t;
+        asm volatile("" : "+v"(ts));
+        const int wq = ts / ((TD + 2) * CG);
+        const int rem = ts - wq * ((TD + 2) * CG);
+        const int dq = rem / CG, cq = rem - dq * CG;
+        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
+        const bool ok = (ts < Cfg::NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+        go = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+        ls = ok ? lds_swizzle<PB>(wq * PDP + dq, cq * 16) : -1;
+        return true;
+    };
 
     // loads run two steps ahead in two register sets; unconditional (clamped plane indices)
     half8_t xpre0, xpre1, gpre0, gpre1;
@@ -699,35 +740,45 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
         *reinterpret_cast<half8_t*>(gdst) = gin ? gpre : z8;
     };
 
-    prefetch(hs - 1, xpre0, gpre0);
-    prefetch(hs, xpre1, gpre1);
-    __syncthreads();  // the one-off zero fill is complete before staging writes anything
-
     if (role == 0) {
         // ---- input gradient: flipped weight operands, lane rr = kh' holds (kd' = 0, 1, 2, -) ----
         half4_t wA[3][2];
+        {
+            const int rr = lane % 4, c0 = cslab + half * 32 + 2 * ((lane / 4) % NQ);
 #pragma unroll
-        for (int kw = 0; kw < 3; ++kw)
+            for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
-                if (rr < 3) {
+                for (int e = 0; e < 2; ++e) {
+                    half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+                    if (rr < 3) {
 #pragma unroll
-                    for (int kd = 0; kd < 3; ++kd)
-                        v[kd] = a.wt[(((2 - rr) * 3 + (2 - kw)) * 3 + (2 - kd)) * C + c0 + e];
+                        for (int kd = 0; kd < 3; ++kd)
+                            v[kd] = a.wt[(((2 - rr) * 3 + (2 - kw)) * 3 + (2 - kd)) * C + c0 + e];
+                    }
+                    wA[kw][e] = v;
                 }
-                wA[kw][e] = v;
-            }
+        }
+        auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
+        while (next_segment()) {
+        // lane constants from an opaque copy of the thread index: computed per segment, so that what only the
+        // segment's set-up needs is not held in registers across the march
+        int tl = t;
+        asm volatile("" : "+v"(tl));
+        const int lane = tl % kWave;
+        const int b = lane / 4, rr = lane % 4;
+        const int q = b % NQ, sub = b / NQ;
+        const int cb = half * 64 + q * 4;
+        const int c0 = cslab + half * 32 + 2 * q;
+        const int pgrp = (gd * NSUB + sub) * 4;
         int dboff[3];
 #pragma unroll
         for (int k = 0; k < 3; ++k) dboff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
-        auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
         int owr[RO];
 #pragma unroll
         for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
         // 64-channel slabs: the threads of this role store the tile, one 16-byte chunk each; narrower slabs
         // store their dwords directly (runs of 256 contiguous bytes per instruction)
-        const int opos = t / CG, ocq = t % CG;
+        const int opos = tl / CG, ocq = tl % CG;
         const int ord = ot_swz(opos, ocq * 16);
         const int ow = w0 + opos / TD, odd = d0 + opos % TD;
         const bool ovalid = (ow < W) && (odd < D);
@@ -741,6 +792,10 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
             oval[o] = (od < D) && (w < W);
             ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
         }
+        parity = 0;
+        prefetch(hs - 1, xpre0, gpre0);
+        prefetch(hs, xpre1, gpre1);
+        __syncthreads();  // the zero fill is complete before staging writes anything
         int pending_row = -1;
         auto flush_row = [&](int par) {
             if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
@@ -818,19 +873,15 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
             step(p, xpre1, gpre1);
             if (++p > he + 1) break;
         }
-        __syncthreads();  // the last tile is written
+        __syncthreads();  // the last tile is written, every wavefront is done with the staging buffers
         flush_row(parity ^ 1);
+        }  // segments
         __syncthreads();  // (the other role: staging buffers are dead)
         __syncthreads();  // (the other role: partial sums are in LDS)
     } else {
         // ---- weight gradient: x windows (patch row ra + xr, positions pgrp + r2 + k) against the interior of
         // the g slots (patch row ra + 1 + gr, positions pgrp + 1 + k), lane j reads the slot of plane p - j ----
-        int aoff[4], boff[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            aoff[k] = lds_swizzle<PB>(ra * PDP + pgrp + r2 + k, cb);
-            boff[k] = lds_swizzle<PB>((ra + 1) * PDP + pgrp + 1 + k, cb);
-        }
+        int aoff[4], boff[4], r2s = 0;  // set per segment (see the other role)
         float4_t acc[3][2];  // one tile per kw: D[i = kd][j = kh]
 #pragma unroll
         for (int kw = 0; kw < 3; ++kw)
@@ -846,7 +897,7 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
             prefetch(p + 2, xpre, gpre);
             __builtin_amdgcn_sched_barrier(0);
             if (xin) {
-                const int gp = p - r2;  // the lane's g plane; planes of other chunks are masked
+                const int gp = p - r2s;  // the lane's g plane; planes of other chunks are masked
                 const uint32_t gmask = (gp >= hs && gp < he) ? 0xffffffffu : 0u;
                 const int gso = (gp & 3) * GSLOT;
                 half4_t G[RO][2];
@@ -876,11 +927,32 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
             }
             parity ^= 1;
         };
-        for (int p = hs - 1;;) {
-            step(p, xpre0, gpre0);
-            if (++p > he + 1) break;
-            step(p, xpre1, gpre1);
-            if (++p > he + 1) break;
+        while (next_segment()) {
+            {
+                int tl = t;
+                asm volatile("" : "+v"(tl));
+                const int ln = tl % kWave;
+                const int bb = ln / 4;
+                const int qq = bb % NQ, ss = bb / NQ;
+                const int cbs = half * 64 + qq * 4, pg = (gd * NSUB + ss) * 4;
+                r2s = min(ln % 4, 2);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    aoff[k] = lds_swizzle<PB>(ra * PDP + pg + r2s + k, cbs);
+                    boff[k] = lds_swizzle<PB>((ra + 1) * PDP + pg + 1 + k, cbs);
+                }
+            }
+            parity = 0;
+            prefetch(hs - 1, xpre0, gpre0);
+            prefetch(hs, xpre1, gpre1);
+            __syncthreads();  // the zero fill is complete before staging writes anything
+            for (int p = hs - 1;;) {
+                step(p, xpre0, gpre0);
+                if (++p > he + 1) break;
+                step(p, xpre1, gpre1);
+                if (++p > he + 1) break;
+            }
+            __syncthreads();  // (the other role: the last tile is written); the staging buffers are free
         }
         if (NSUB > 1) {  // position groups inside the wavefront
 #pragma unroll
@@ -895,9 +967,9 @@ __global__ __launch_bounds__(Cfg::NT) void dwconv_bwd_split_kernel(const WgArgs 
                         acc[kw][e][i] = v;
                     }
         }
-        __syncthreads();  // (the other role: the last tile is written)
         __syncthreads();  // staging buffers are dead from here on
         float* red = reinterpret_cast<float*>(smem);  // [NPART][27][SC]
+        const int rr = lane % 4, q = (lane / 4) % NQ, sub = (lane / 4) / NQ;
         if (sub == 0 && rr < 3) {
 #pragma unroll
             for (int kw = 0; kw < 3; ++kw)
@@ -1105,10 +1177,35 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
     p->n_slab = C / (p->cg * 8);
     p->n_wt = ceil_div(W, p->tile_w);
     p->n_dt = ceil_div(D, p->tile_d);
+    const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
+    const int slots = 512;  // two workgroups of 512 threads per CU
+    p->bal_group = 0;
+    // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups); > 0: uniform
+    // chunks of that many rows
     if (h_chunk <= 0) {
-        const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-        // two workgroups of 512 threads per CU
-        h_chunk = pick_h_chunk(H, per_plane, 512, 8);
+        if (h_chunk < 0 && (-h_chunk) % p->n_slab != 0) {
+            set_error("dwconv_bwd: the group size of the balanced split must be a multiple of the slab count %d",
+                      p->n_slab);
+            return KEROPS_E_BADARG;
+        }
+        const BalancedSplit b = h_chunk < 0 ? make_balanced(H, per_plane, slots, -h_chunk)
+                                            : pick_balanced(H, per_plane, p->n_dt * p->n_slab, slots, 8, p->n_slab);
+        const bool fits = b.units < (1LL << 31) && per_plane + b.group < (1LL << 31);  // 32-bit counters in the kernel
+        if (!fits && h_chunk < 0) {
+            set_error("dwconv_bwd: too many plane steps for the balanced split");
+            return KEROPS_E_BADARG;
+        }
+        if (fits) {
+            p->bal_group = b.group;
+            p->bal_q = (uint32_t)(b.units / b.ngroups);
+            p->bal_r = (uint32_t)(b.units % b.ngroups);
+            p->n_tiles = (uint32_t)per_plane;
+            p->h_chunk = H;
+            p->n_hc = 1;
+            p->nblocks = (int64_t)b.group * b.ngroups;
+            return KEROPS_OK;
+        }
+        h_chunk = pick_h_chunk(H, per_plane, slots, 8);
     }
     p->h_chunk = std::min(h_chunk, H);
     p->n_hc = ceil_div(H, p->h_chunk);
@@ -1169,6 +1266,10 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
     b.n_slab = p.n_slab;
     b.h_chunk = p.h_chunk;
     b.nblocks = (uint32_t)p.nblocks;
+    b.bal_group = p.bal_group;
+    b.bal_q = p.bal_q;
+    b.bal_r = p.bal_r;
+    b.n_tiles = p.n_tiles;
 #define KEROPS_BS_GO(CGv, TWv, TDv)                                                                                  \
     {                                                                                                                \
         using Cfg = BsCfg<CGv, TWv, TDv, 512>;                                                                       \

@@ -95,36 +95,33 @@ def test_workspace_queries():
     assert lib.kerops_absmax_workspace_bytes(10) == 40
 
 
-def test_h_chunk_choice_fills_whole_rounds():
+def test_split_of_the_h_march():
     # workgroup counts of the built-in launch shapes, read back from the workspace sizes (one partial per
-    # workgroup).  Uniform chunks (the convolution + statistics kernel): 1408 = 2.75 per resident slot at the README
-    # shape (the measured optimum), exactly one round of 512 workgroups at 128^3-class volumes instead of several
-    # short chunks.  The weight gradient uses the balanced split: never more workgroups than the GPU holds at once
-    # (512 of 512 threads, 1024 of 256), all of them busy at the large shapes.
+    # workgroup).  The matrix-core convolution kernels use the balanced split by default: never more workgroups than
+    # the GPU holds at once (512 of 512 threads, 1024 of 256), all of them busy at the large shapes.  Uniform chunks
+    # on request: patches x chunks.
     lib = _lib.load()
 
     def wgrad_blocks(n, h, w, d, c, h_chunk=0):
         return lib.kerops_dwconv_wgrad_workspace_bytes(n, h, w, d, c, 0, 0, h_chunk, 0) // (27 * min(c, 64) * 4)
 
-    def fwd_blocks(n, h, w, d, c):
+    def bwd_blocks(n, h, w, d, c, h_chunk=0):
+        return lib.kerops_dwconv_bwd_workspace_bytes(n, h, w, d, c, h_chunk) // (27 * min(c, 64) * 4)
+
+    def stats_blocks(n, h, w, d, c):
         return lib.kerops_dwconv_stats_workspace_bytes(n, h, w, d, c) // (2 * min(c, 64) * 4)
 
-    assert fwd_blocks(1, 350, 350, 128, 64) == 1408
-    assert fwd_blocks(1, 128, 128, 128, 64) == 512
-    assert fwd_blocks(2, 128, 128, 128, 32) == 512
-    assert fwd_blocks(1, 350, 350, 128, 128) == 4 * 1408  # four chunks of 88 rows: 11 whole rounds
-    assert fwd_blocks(1, 1, 8, 8, 64) == 1
-
-    assert wgrad_blocks(1, 350, 350, 128, 64) == 512      # 8 groups of 64 = 4 rows of 16 patches
-    assert wgrad_blocks(1, 350, 350, 128, 128) == 512     # 4 groups of 128 = 4 rows of 16 patches x 2 slabs
+    for blocks in (wgrad_blocks, bwd_blocks, stats_blocks):
+        assert blocks(1, 350, 350, 128, 64) == 512   # 8 groups of 64 (weight gradient: 4 rows of 16 patches)
+        assert blocks(1, 350, 350, 128, 128) == 512  # the same patches in 2 slabs
+        assert blocks(1, 128, 128, 128, 64) == 512
     assert wgrad_blocks(1, 350, 350, 128, 8) in range(960, 1025)
-    assert wgrad_blocks(1, 128, 128, 128, 64) == 512
-    assert wgrad_blocks(1, 1, 8, 8, 8) == 1
-    # uniform chunks on request: patches x chunks; explicit groups: group x groups
-    assert wgrad_blocks(1, 350, 350, 128, 64, 175) == 1408
-    assert wgrad_blocks(1, 350, 350, 128, 64, -32) == 512
+    assert wgrad_blocks(1, 1, 8, 8, 8) == 1 and stats_blocks(1, 1, 8, 8, 64) == 1 and bwd_blocks(1, 1, 8, 8, 64) == 2
+    assert wgrad_blocks(1, 350, 350, 128, 64, 175) == 1408 and bwd_blocks(1, 350, 350, 128, 64, 175) == 2816
+    assert wgrad_blocks(1, 350, 350, 128, 64, -32) == 512 and bwd_blocks(1, 350, 350, 128, 64, -32) == 512
     # a group that is not a multiple of the two slabs of 128 channels is refused
     assert lib.kerops_dwconv_wgrad_workspace_bytes(1, 350, 350, 128, 128, 0, 0, -3, 0) == _lib.KEROPS_E_BADARG
+    assert lib.kerops_dwconv_bwd_workspace_bytes(1, 350, 350, 128, 128, -3) == _lib.KEROPS_E_BADARG
 
 
 def cl3d(*shape, dtype=torch.float16):
