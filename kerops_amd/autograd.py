@@ -6,8 +6,8 @@ wiring once.  Each `apply` takes and returns exactly what the forward op does.  
 provides the input gradient, which the reference lacks (a TODO at kerops/kernels/dw_conv.py:145):
 it is the same depthwise kernel run on the upstream gradient with the weight flipped along the
 three spatial axes.  When both gradients are wanted the wrapper calls `ops.conv.DWConvBackward`, which
-computes them in one pass over x and the upstream gradient (up to 13 % faster than the two kernels, never
-slower, the same input gradient bit for bit).
+computes them in one pass over x and the upstream gradient (4-8 % faster than the two kernels, the same input
+gradient bit for bit).
 """
 import torch
 

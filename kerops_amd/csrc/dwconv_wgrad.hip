@@ -1155,7 +1155,7 @@ static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, float* gw, hip
     return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg>, base, p, gw, stream);
 }
 
-// fused backward: one patch shape per channel count, one workgroup per CU
+// fused backward: one patch shape per channel count, two workgroups of 512 threads per CU
 static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
 {
     if (N <= 0 || H <= 0 || W <= 0 || D <= 0) {

@@ -20,7 +20,9 @@ def served(channels):
 
 @configure(H_chunk=lambda x: served(x.shape[1]), out_dtype=torch.float16)
 def DWConvBackward(x, grad, weight, *, H_chunk: ConfigurableArg, out_dtype: ConfigurableArg):
-    """x, grad (N,C,H,W,D) fp16 channels_last_3d, weight [3,3,3,C] fp16 -> (grad_x like x, grad_w [3,3,3,C])."""
+    """x, grad (N,C,H,W,D) fp16 channels_last_3d, weight [3,3,3,C] fp16 -> (grad_x like x, grad_w [3,3,3,C]).
+
+    H_chunk as in DWConvWGRAD: 0 = balanced split, > 0 = uniform chunks of that many rows, -g = groups of g."""
     channels = x.shape[1]
 
     assert x.ndim == grad.ndim == 5
