@@ -170,6 +170,54 @@ static inline bool plane_exceeds_i32(int W, int D, int C)
     return wd >= (1LL << 31) || wd * C >= (1LL << 31);
 }
 
+// Device side of the two splits of the H march: the sequence of (tile, rows [hs, he)) segments of one workgroup.
+// Tiles are numbered slab fastest, then along D, along W, then the batch.  Uniform chunks (group = 0): one segment,
+// workgroup w = (tile inside the sample, chunk, sample).  Balanced split: the workgroup is member w % group of group
+// w / group, which owns the units [u, u_end) of the (bundle of `group` tiles, row) sequence; a share that ends inside
+// a bundle continues in the next one, and members beyond the last tile of a partly filled bundle skip it.  All
+// values are wavefront-uniform and kept in scalar registers.
+struct SegmentWalk {
+    uint32_t u, u_end, member, group;
+    bool first;
+};
+// shares of q or q + 1 units: the first r groups take the longer ones
+__device__ __forceinline__ SegmentWalk segment_walk_begin(uint32_t wg, uint32_t group, uint32_t q, uint32_t r)
+{
+    SegmentWalk s{0u, 0u, 0u, group, true};
+    if (group > 0) {
+        const uint32_t g = wg / group;
+        s.member = wg - g * group;
+        s.u = __builtin_amdgcn_readfirstlane(g * q + min(g, r));
+        s.u_end = __builtin_amdgcn_readfirstlane(s.u + q + (g < r ? 1u : 0u));
+    }
+    return s;
+}
+__device__ __forceinline__ bool segment_walk_next(SegmentWalk& s, uint32_t wg, int H, uint32_t n_tiles,
+                                                  uint32_t tiles_per_sample, int n_hc, int h_chunk, uint32_t& tile,
+                                                  int& hs, int& he)
+{
+    if (s.group > 0) {
+        for (;;) {
+            if (s.u >= s.u_end) return false;
+            const uint32_t bundle = s.u / (uint32_t)H;
+            // (the quotient comes out of a vector division: back to scalar registers)
+            hs = __builtin_amdgcn_readfirstlane((int)(s.u - bundle * (uint32_t)H));
+            he = (int)min((uint32_t)H, hs + (s.u_end - s.u));
+            s.u += he - hs;
+            tile = __builtin_amdgcn_readfirstlane(bundle * s.group + s.member);
+            if (tile < n_tiles) return true;
+        }
+    }
+    if (!s.first) return false;
+    s.first = false;
+    const uint32_t rest = wg / tiles_per_sample;
+    const int hc = (int)(rest % (uint32_t)n_hc);
+    tile = __builtin_amdgcn_readfirstlane((rest / (uint32_t)n_hc) * tiles_per_sample + wg % tiles_per_sample);
+    hs = __builtin_amdgcn_readfirstlane(hc * h_chunk);
+    he = min(hs + h_chunk, H);
+    return true;
+}
+
 // The 8 XCDs of the chip receive workgroups round-robin (workgroup b runs on XCD
 // b % 8) and each XCD has a private L2.  remap_xcd turns the hardware workgroup
 // index into a logical tile index such that each XCD walks one contiguous range of

@@ -462,8 +462,11 @@ struct FmCfg {
 // pointwise GEMM [TW*TD positions][C] x [C][COUT] on the 32x32x16 matrix instruction (the product is computed
 // transposed as in pointwise_kernel, a wavefront owns 32 positions x 32 output channels; pw^T sits in LDS), the
 // [positions][COUT] result is bounced through LDS and stored as 16-byte chunks with the running max|y| fused in.
-template <class Cfg, int MODE, int COUT = 0>
-__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mfma_kernel(const FwdArgs a)
+// One segment of a workgroup's work: the march over the rows [hs, he) of one tile (patch x slab x sample).
+template <class Cfg, int MODE, int COUT>
+__device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsigned char* smem, float* amax_red,
+                                                        uint32_t wg_slot, uint32_t tile, int hs, int he,
+                                                        float (&ssum)[2], float (&ssq)[2])
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, XSLOT = Cfg::XSLOT, NLDX = Cfg::NLDX;
@@ -482,63 +485,20 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
     static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
     constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);
-    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
-    __shared__ float amax_red[Cfg::NWAVE];
-
-    const uint32_t wg_slot = remap_xcd(blockIdx.x, a.nblocks);
-    if (wg_slot >= a.nblocks) return;
-    const int H = a.H, W = a.W, D = a.D, C = a.C;
-    // Work of this workgroup: one (tile, row range) segment with uniform chunks, or, in the balanced split, its
-    // group's contiguous share [u, u_end) of the (bundle of bal_group tiles, row) sequence: the workgroups of a
-    // group march in step over neighbouring tiles (member = tile inside the bundle) and cross into the next
-    // bundle together, so that every group carries the same number of plane steps.
     constexpr bool SEGMENTS = MODE != 2;  // the fused pointwise mode always runs one segment (uniform chunks)
-    const bool balanced = SEGMENTS && a.bal_group > 0;
-    // mode 3: sums over the lane's channel pair, carried over every segment (all tiles of a workgroup belong to
-    // the same slab: the group size is a multiple of the slab count)
-    float ssum[2] = {0.0f, 0.0f}, ssq[2] = {0.0f, 0.0f};
-    uint32_t u = 0, u_end = 0, member = 0;  // wavefront-uniform, kept in scalar registers
-    if (balanced) {
-        const uint32_t group = wg_slot / a.bal_group;
-        member = wg_slot - group * a.bal_group;
-        // shares of bal_q or bal_q + 1 units: the first bal_r groups take the longer ones
-        u = __builtin_amdgcn_readfirstlane(group * a.bal_q + min(group, a.bal_r));
-        u_end = __builtin_amdgcn_readfirstlane(u + a.bal_q + (group < a.bal_r ? 1u : 0u));
-    }
-    for (bool first = true;; first = false) {
+    const int H = a.H, W = a.W, D = a.D, C = a.C;
     // The thread index is made opaque per segment: everything derived from it is then computed inside the segment
-    // and dies with the prologue, instead of being hoisted out of this loop and held in registers across the march.
+    // and dies with the prologue, instead of being hoisted out of the segment loop and held in registers across
+    // the march.
     int t = threadIdx.x;
     if constexpr (SEGMENTS) asm volatile("" : "+v"(t));
-    uint32_t L;
-    int hs, he;
-    if (balanced) {
-        if (u >= u_end) break;
-        const uint32_t bundle = u / (uint32_t)H;
-        hs = (int)(u - bundle * (uint32_t)H);
-        he = (int)min((uint32_t)H, hs + (u_end - u));
-        u += he - hs;
-        L = bundle * a.bal_group + member;
-        if (L >= a.n_tiles) continue;  // a partly filled last bundle
-    } else {
-        if (!first) break;
-        L = wg_slot;
-    }
+    uint32_t L = tile;
     const int slab = L % a.n_slab;
     L /= a.n_slab;
     const int dt = L % a.n_dt;
     L /= a.n_dt;
     const int wt_i = L % a.n_wt;
-    L /= a.n_wt;
-    int n;
-    if (balanced) {
-        n = L;
-    } else {
-        const int hc = L % a.n_hc;
-        n = L / a.n_hc;
-        hs = hc * a.h_chunk;
-        he = min(hs + a.h_chunk, H);
-    }
+    const int n = L / a.n_wt;
     const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
     const int cslab = slab * SC;
     const int64_t plane_stride = (int64_t)W * D * C;
@@ -802,10 +762,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     if constexpr (BOUNCE) {
         __syncthreads();
         flush_row(parity ^ 1);
-    } else {
-        if (balanced) __syncthreads();  // the staging buffers are free before the next segment refills them
+    } else if constexpr (SEGMENTS) {
+        __syncthreads();  // the staging buffers are free before the next segment refills them
     }
-    if constexpr (SEGMENTS) continue;  // the fused pointwise mode runs one segment and finishes here
     if constexpr (MODE == 2) {
         amax = wave_max(amax);
         if (lane == 0) amax_red[wave] = amax;
@@ -817,8 +776,48 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
             a.amax_ws[wg_slot] = m;
         }
     }
-    break;
-    }  // segments
+}
+
+template <class Cfg, int MODE, int COUT = 0>
+__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mfma_kernel(const FwdArgs a)
+{
+    constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
+    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, XSLOT = Cfg::XSLOT, NLDX = Cfg::NLDX;
+    constexpr bool EPI = MODE == 1 || MODE == 2;
+    constexpr bool STATS = MODE == 3;
+    // fused pointwise stage: t tile [NPOS][SC + 8] fp16 and y tile [NPOS][COUT + 4] fp16 behind the staging buffers
+    constexpr int NPOS = Cfg::TW * TD, RT = SC + 8, RY = COUT + 4;
+    constexpr int KS = SC / 16, MT = COUT / 32, NPT = NPOS / 32;  // k = 16 per matrix instruction
+    constexpr int T_OFF = Cfg::LDS_BYTES, Y_OFF = T_OFF + NPOS * RT * 2, A_OFF = Y_OFF + NPOS * RY * 2;
+    // modes 0 and 1 with a 64-channel slab: two output tiles [NPOS][PB] behind the staging buffers.  A wavefront
+    // owns 32 channels, i.e. 64-byte halves of the 128-byte positions; written directly they cost 10 % more HBM
+    // write traffic than the tensor holds.  So a finished plane is written to the tile as dwords and leaves one
+    // step later, behind that step's barrier, as one 16-byte chunk per thread: whole lines, one store instruction
+    // instead of RO.  Narrower slabs write runs of 256 contiguous bytes anyway and store directly.
+    constexpr bool BOUNCE = MODE != 2 && SC == 64;
+    constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
+    static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
+    constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
+    __shared__ float amax_red[Cfg::NWAVE];
+
+    const uint32_t wg_slot = remap_xcd(blockIdx.x, a.nblocks);
+    if (wg_slot >= a.nblocks) return;
+    // mode 3: sums over the lane's channel pair, carried over every segment (all tiles of a workgroup belong to
+    // the same slab: the group size of the balanced split is a multiple of the slab count)
+    float ssum[2] = {0.0f, 0.0f}, ssq[2] = {0.0f, 0.0f};
+    constexpr bool SEGMENTS = MODE != 2;  // the fused pointwise mode always runs one segment (uniform chunks)
+    SegmentWalk walk = segment_walk_begin(wg_slot, SEGMENTS ? a.bal_group : 0u, a.bal_q, a.bal_r);
+    uint32_t tile;
+    int hs, he;
+    const uint32_t per_sample = (uint32_t)(a.n_slab * a.n_dt * a.n_wt);
+    if constexpr (SEGMENTS) {
+        while (segment_walk_next(walk, wg_slot, a.H, a.n_tiles, per_sample, a.n_hc, a.h_chunk, tile, hs, he))
+            dwconv_fwd_mfma_segment<Cfg, MODE, COUT>(a, smem, amax_red, wg_slot, tile, hs, he, ssum, ssq);
+    } else {
+        segment_walk_next(walk, wg_slot, a.H, a.n_tiles, per_sample, a.n_hc, a.h_chunk, tile, hs, he);
+        dwconv_fwd_mfma_segment<Cfg, MODE, COUT>(a, smem, amax_red, wg_slot, tile, hs, he, ssum, ssq);
+    }
     if constexpr (STATS) {
         const int t = threadIdx.x;
         const int lane = t % kWave, wave = t / kWave;

@@ -390,157 +390,157 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
         u_end = __builtin_amdgcn_readfirstlane(u + a.bal_q + (group < a.bal_r ? 1u : 0u));
     }
     for (bool first = true;; first = false) {
-    // the thread index is made opaque per segment: the staging assignment derived from it is then computed inside
-    // the segment instead of being hoisted out of this loop and held in registers across the march
-    int t = threadIdx.x;
-    asm volatile("" : "+v"(t));
-    uint32_t L;
-    int hs, he;
-    if (balanced) {
-        if (u >= u_end) break;
-        const uint32_t bundle = u / (uint32_t)H;
-        hs = (int)(u - bundle * (uint32_t)H);
-        he = (int)min((uint32_t)H, hs + (u_end - u));
-        u += he - hs;
-        L = bundle * a.bal_group + member;
-        if (L >= a.n_tiles) continue;  // a partly filled last bundle
-        if (!first) __syncthreads();   // the previous segment's last plane has been read by every wavefront
-    } else {
-        if (!first) break;
-        L = ws_slot;
-    }
-    const int slab = L % a.n_slab;
-    L /= a.n_slab;
-    const int dt = L % a.n_dt;
-    L /= a.n_dt;
-    const int wt_i = L % a.n_wt;
-    L /= a.n_wt;
-    int n;
-    if (balanced) {
-        n = L;
-    } else {
-        const int hc = L % a.n_hc;
-        n = L / a.n_hc;
-        hs = hc * a.h_chunk;
-        he = min(hs + a.h_chunk, H);
-    }
-    const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
-    const int cslab = slab * SC;
-    const int64_t plane_stride = (int64_t)W * D * C;
-    const half_t* xn = a.x + (int64_t)n * H * plane_stride;
-    const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
+        // the thread index is made opaque per segment: the staging assignment derived from it is then computed inside
+        // the segment instead of being hoisted out of this loop and held in registers across the march
+        int t = threadIdx.x;
+        asm volatile("" : "+v"(t));
+        uint32_t L;
+        int hs, he;
+        if (balanced) {
+            if (u >= u_end) break;
+            const uint32_t bundle = u / (uint32_t)H;
+            hs = (int)(u - bundle * (uint32_t)H);
+            he = (int)min((uint32_t)H, hs + (u_end - u));
+            u += he - hs;
+            L = bundle * a.bal_group + member;
+            if (L >= a.n_tiles) continue;  // a partly filled last bundle
+            if (!first) __syncthreads();   // the previous segment's last plane has been read by every wavefront
+        } else {
+            if (!first) break;
+            L = ws_slot;
+        }
+        const int slab = L % a.n_slab;
+        L /= a.n_slab;
+        const int dt = L % a.n_dt;
+        L /= a.n_dt;
+        const int wt_i = L % a.n_wt;
+        L /= a.n_wt;
+        int n;
+        if (balanced) {
+            n = L;
+        } else {
+            const int hc = L % a.n_hc;
+            n = L / a.n_hc;
+            hs = hc * a.h_chunk;
+            he = min(hs + a.h_chunk, H);
+        }
+        const int w0 = wt_i * Cfg::TW, d0 = dt * TD;
+        const int cslab = slab * SC;
+        const int64_t plane_stride = (int64_t)W * D * C;
+        const half_t* xn = a.x + (int64_t)n * H * plane_stride;
+        const half_t* gn_ptr = a.g + (int64_t)n * H * plane_stride;
 
-    // everything that staging never writes must read as zero: positions outside the volume and the
-    // g planes before the chunk
-    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int o = t * 16; o < Cfg::STAGE_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
+        // everything that staging never writes must read as zero: positions outside the volume and the
+        // g planes before the chunk
+        const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int o = t * 16; o < Cfg::STAGE_BYTES; o += NT * 16) *reinterpret_cast<half8_t*>(smem + o) = z8;
 
-    // staging assignment, 16-byte chunks (8 channels of one position); lanes without a chunk inside the
-    // volume load the plane's first chunk and write it to the dump slot
-    uint32_t xgo[NLDX], ggo[NLDG];
-    int xls[NLDX], gls[NLDG];
-#pragma unroll
-    for (int j = 0; j < NLDX; ++j) {
-        const int ch = t + j * NT;
-        const int wq = ch / ((TD + 2) * CG);
-        const int rem = ch - wq * ((TD + 2) * CG);
-        const int dq = rem / CG, cq = rem - dq * CG;
-        const int w = w0 - 1 + wq, d = d0 - 1 + dq;
-        const bool ok = (ch < Cfg::NXCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
-        xgo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
-        xls[j] = ok ? Cfg::swz(wq * PDP + dq, cq * 16) : -1;
-    }
-#pragma unroll
-    for (int j = 0; j < NLDG; ++j) {
-        const int ch = t + j * NT;
-        const int wq = ch / (TD * CG);
-        const int rem = ch - wq * (TD * CG);
-        const int dq = rem / CG, cq = rem - dq * CG;
-        const int w = w0 + wq, d = d0 + dq;
-        const bool ok = (ch < Cfg::NGCH) && (w < W) && (d < D);
-        ggo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
-        gls[j] = ok ? Cfg::swz(wq * TD + dq, cq * 16) : -1;
-    }
-
-    // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
-    // They are unconditional (plane indices are clamped, values of planes that do not exist or lie
-    // outside the chunk are never used): the compiler's wait-count bookkeeping is exact only on
-    // branch-free paths, and a conservative wait would also wait for the newer set.
-    half8_t xpre0[NLDX], xpre1[NLDX], gpre0[NLDG], gpre1[NLDG];
-    auto prefetch = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {  // x plane hp, g plane hp+1
-        const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
-        const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(hp + 1, hs), he - 1) * plane_stride);
-#pragma unroll
-        for (int j = 0; j < NLDX; ++j) xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
-#pragma unroll
-        for (int j = 0; j < NLDG; ++j)
-            gpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(gplane + ggo[j]));
-    };
-
-    int parity = 0;
-    // step hp: x plane hp meets the g planes hp+1 (kh = 0), hp (kh = 1), hp-1 (kh = 2)
-    auto step = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {
-        const bool xin = (hp >= 0) && (hp < H);  // wavefront-uniform
-        const bool gin = hp + 1 < he;
-        unsigned char* xbuf = smem + Cfg::XOFF + parity * XSLOT;
-        unsigned char* gslot = smem + ((hp + 1) & 3) * GSLOT;
-#pragma unroll
+        // staging assignment, 16-byte chunks (8 channels of one position); lanes without a chunk inside the
+        // volume load the plane's first chunk and write it to the dump slot
+        uint32_t xgo[NLDX], ggo[NLDG];
+        int xls[NLDX], gls[NLDG];
+    #pragma unroll
         for (int j = 0; j < NLDX; ++j) {
-            unsigned char* dst = xls[j] >= 0 ? xbuf + xls[j] : smem + Cfg::DUMP;
-            *reinterpret_cast<half8_t*>(dst) = xpre[j];
+            const int ch = t + j * NT;
+            const int wq = ch / ((TD + 2) * CG);
+            const int rem = ch - wq * ((TD + 2) * CG);
+            const int dq = rem / CG, cq = rem - dq * CG;
+            const int w = w0 - 1 + wq, d = d0 - 1 + dq;
+            const bool ok = (ch < Cfg::NXCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
+            xgo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+            xls[j] = ok ? Cfg::swz(wq * PDP + dq, cq * 16) : -1;
         }
-        // g planes past the chunk read as zero; the slot held a plane that is no longer needed
-#pragma unroll
+    #pragma unroll
         for (int j = 0; j < NLDG; ++j) {
-            unsigned char* dst = gls[j] >= 0 ? gslot + gls[j] : smem + Cfg::DUMP;
-            *reinterpret_cast<half8_t*>(dst) = gin ? gpre[j] : z8;
+            const int ch = t + j * NT;
+            const int wq = ch / (TD * CG);
+            const int rem = ch - wq * (TD * CG);
+            const int dq = rem / CG, cq = rem - dq * CG;
+            const int w = w0 + wq, d = d0 + dq;
+            const bool ok = (ch < Cfg::NGCH) && (w < W) && (d < D);
+            ggo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
+            gls[j] = ok ? Cfg::swz(wq * TD + dq, cq * 16) : -1;
         }
-        __syncthreads();
-        prefetch(hp + 2, xpre, gpre);
-        __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
-        if (xin) {
-            const int xo = parity * XSLOT;
-            const int go = ((hp + 1 - r2) & 3) * GSLOT;  // lane j reads the slot of plane hp+1-j
-            half4_t G[RG][2];
-#pragma unroll
-            for (int xr = 0; xr < RG + 2; ++xr) {
-                if (xr < RG) {  // the g row first needed by this x row
+
+        // Global loads run two planes ahead of the arithmetic, into two register sets used alternately.
+        // They are unconditional (plane indices are clamped, values of planes that do not exist or lie
+        // outside the chunk are never used): the compiler's wait-count bookkeeping is exact only on
+        // branch-free paths, and a conservative wait would also wait for the newer set.
+        half8_t xpre0[NLDX], xpre1[NLDX], gpre0[NLDG], gpre1[NLDG];
+        auto prefetch = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {  // x plane hp, g plane hp+1
+            const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
+            const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(hp + 1, hs), he - 1) * plane_stride);
+    #pragma unroll
+            for (int j = 0; j < NLDX; ++j) xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
+    #pragma unroll
+            for (int j = 0; j < NLDG; ++j)
+                gpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(gplane + ggo[j]));
+        };
+
+        int parity = 0;
+        // step hp: x plane hp meets the g planes hp+1 (kh = 0), hp (kh = 1), hp-1 (kh = 2)
+        auto step = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {
+            const bool xin = (hp >= 0) && (hp < H);  // wavefront-uniform
+            const bool gin = hp + 1 < he;
+            unsigned char* xbuf = smem + Cfg::XOFF + parity * XSLOT;
+            unsigned char* gslot = smem + ((hp + 1) & 3) * GSLOT;
+    #pragma unroll
+            for (int j = 0; j < NLDX; ++j) {
+                unsigned char* dst = xls[j] >= 0 ? xbuf + xls[j] : smem + Cfg::DUMP;
+                *reinterpret_cast<half8_t*>(dst) = xpre[j];
+            }
+            // g planes past the chunk read as zero; the slot held a plane that is no longer needed
+    #pragma unroll
+            for (int j = 0; j < NLDG; ++j) {
+                unsigned char* dst = gls[j] >= 0 ? gslot + gls[j] : smem + Cfg::DUMP;
+                *reinterpret_cast<half8_t*>(dst) = gin ? gpre[j] : z8;
+            }
+            __syncthreads();
+            prefetch(hp + 2, xpre, gpre);
+            __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
+            if (xin) {
+                const int xo = parity * XSLOT;
+                const int go = ((hp + 1 - r2) & 3) * GSLOT;  // lane j reads the slot of plane hp+1-j
+                half4_t G[RG][2];
+    #pragma unroll
+                for (int xr = 0; xr < RG + 2; ++xr) {
+                    if (xr < RG) {  // the g row first needed by this x row
+                        uint32_t r[4];
+    #pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            r[k] = *reinterpret_cast<const uint32_t*>(smem + go + boff[k] + xr * TD * PB);
+                        split_operands(r, G[xr][0], G[xr][1]);
+                    }
                     uint32_t r[4];
-#pragma unroll
+    #pragma unroll
                     for (int k = 0; k < 4; ++k)
-                        r[k] = *reinterpret_cast<const uint32_t*>(smem + go + boff[k] + xr * TD * PB);
-                    split_operands(r, G[xr][0], G[xr][1]);
-                }
-                uint32_t r[4];
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    r[k] = *reinterpret_cast<const uint32_t*>(smem + xo + aoff[k] + xr * PDP * PB);
-                half4_t A[2];
-                split_operands(r, A[0], A[1]);
-#pragma unroll
-                for (int kw = 0; kw < 3; ++kw) {
-                    // x patch row ra-1+xr meets g row ra+xr-kw at tap kw
-                    if (xr - kw >= 0 && xr - kw < RG) {
-#pragma unroll
-                        for (int e = 0; e < 2; ++e) {
-                            acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], G[xr - kw][e], acc[kw][e], 0, 0, 0);
+                        r[k] = *reinterpret_cast<const uint32_t*>(smem + xo + aoff[k] + xr * PDP * PB);
+                    half4_t A[2];
+                    split_operands(r, A[0], A[1]);
+    #pragma unroll
+                    for (int kw = 0; kw < 3; ++kw) {
+                        // x patch row ra-1+xr meets g row ra+xr-kw at tap kw
+                        if (xr - kw >= 0 && xr - kw < RG) {
+    #pragma unroll
+                            for (int e = 0; e < 2; ++e) {
+                                acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], G[xr - kw][e], acc[kw][e], 0, 0, 0);
+                            }
                         }
                     }
                 }
             }
-        }
-        parity ^= 1;
-    };
+            parity ^= 1;
+        };
 
-    prefetch(hs - 1, xpre0, gpre0);
-    prefetch(hs, xpre1, gpre1);
-    __syncthreads();  // the one-off zero fill is complete before staging writes anything
-    for (int hp = hs - 1;;) {
-        step(hp, xpre0, gpre0);
-        if (++hp > he) break;
-        step(hp, xpre1, gpre1);
-        if (++hp > he) break;
-    }
+        prefetch(hs - 1, xpre0, gpre0);
+        prefetch(hs, xpre1, gpre1);
+        __syncthreads();  // the one-off zero fill is complete before staging writes anything
+        for (int hp = hs - 1;;) {
+            step(hp, xpre0, gpre0);
+            if (++hp > he) break;
+            step(hp, xpre1, gpre1);
+            if (++hp > he) break;
+        }
     }  // segments
 
     const int t = threadIdx.x;
@@ -760,121 +760,121 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
         }
         auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
         while (next_segment()) {
-        // lane constants from an opaque copy of the thread index: computed per segment, so that what only the
-        // segment's set-up needs is not held in registers across the march
-        int tl = t;
-        asm volatile("" : "+v"(tl));
-        const int lane = tl % kWave;
-        const int b = lane / 4, rr = lane % 4;
-        const int q = b % NQ, sub = b / NQ;
-        const int cb = half * 64 + q * 4;
-        const int c0 = cslab + half * 32 + 2 * q;
-        const int pgrp = (gd * NSUB + sub) * 4;
-        int dboff[3];
-#pragma unroll
-        for (int k = 0; k < 3; ++k) dboff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
-        int owr[RO];
-#pragma unroll
-        for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
-        // 64-channel slabs: the threads of this role store the tile, one 16-byte chunk each; narrower slabs
-        // store their dwords directly (runs of 256 contiguous bytes per instruction)
-        const int opos = tl / CG, ocq = tl % CG;
-        const int ord = ot_swz(opos, ocq * 16);
-        const int ow = w0 + opos / TD, odd = d0 + opos % TD;
-        const bool ovalid = (ow < W) && (odd < D);
-        const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
-        const int od = d0 + pgrp + rr;
-        uint32_t ooff[RO];
-        bool oval[RO];
-#pragma unroll
-        for (int o = 0; o < RO; ++o) {
-            const int w = w0 + ra + o;
-            oval[o] = (od < D) && (w < W);
-            ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
-        }
-        parity = 0;
-        prefetch(hs - 1, xpre0, gpre0);
-        prefetch(hs, xpre1, gpre1);
-        __syncthreads();  // the zero fill is complete before staging writes anything
-        int pending_row = -1;
-        auto flush_row = [&](int par) {
-            if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
-                const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + Cfg::OT_OFF + par * Cfg::OT_BYTES + ord);
-                if (ovalid)
-                    __builtin_nontemporal_store(
-                        o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(dxn + pending_row * plane_stride) + ogo));
+            // lane constants from an opaque copy of the thread index: computed per segment, so that what only the
+            // segment's set-up needs is not held in registers across the march
+            int tl = t;
+            asm volatile("" : "+v"(tl));
+            const int lane = tl % kWave;
+            const int b = lane / 4, rr = lane % 4;
+            const int q = b % NQ, sub = b / NQ;
+            const int cb = half * 64 + q * 4;
+            const int c0 = cslab + half * 32 + 2 * q;
+            const int pgrp = (gd * NSUB + sub) * 4;
+            int dboff[3];
+    #pragma unroll
+            for (int k = 0; k < 3; ++k) dboff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
+            int owr[RO];
+    #pragma unroll
+            for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
+            // 64-channel slabs: the threads of this role store the tile, one 16-byte chunk each; narrower slabs
+            // store their dwords directly (runs of 256 contiguous bytes per instruction)
+            const int opos = tl / CG, ocq = tl % CG;
+            const int ord = ot_swz(opos, ocq * 16);
+            const int ow = w0 + opos / TD, odd = d0 + opos % TD;
+            const bool ovalid = (ow < W) && (odd < D);
+            const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
+            const int od = d0 + pgrp + rr;
+            uint32_t ooff[RO];
+            bool oval[RO];
+    #pragma unroll
+            for (int o = 0; o < RO; ++o) {
+                const int w = w0 + ra + o;
+                oval[o] = (od < D) && (w < W);
+                ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
             }
-        };
-        float4_t T[RO][2];  // dx tiles: registers 0, 1, 2 = planes p+1, p, p-1
-#pragma unroll
-        for (int o = 0; o < RO; ++o)
-#pragma unroll
-            for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            parity = 0;
+            prefetch(hs - 1, xpre0, gpre0);
+            prefetch(hs, xpre1, gpre1);
+            __syncthreads();  // the zero fill is complete before staging writes anything
+            int pending_row = -1;
+            auto flush_row = [&](int par) {
+                if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
+                    const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + Cfg::OT_OFF + par * Cfg::OT_BYTES + ord);
+                    if (ovalid)
+                        __builtin_nontemporal_store(
+                            o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(dxn + pending_row * plane_stride) + ogo));
+                }
+            };
+            float4_t T[RO][2];  // dx tiles: registers 0, 1, 2 = planes p+1, p, p-1
+    #pragma unroll
+            for (int o = 0; o < RO; ++o)
+    #pragma unroll
+                for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-        auto step = [&](int p, half8_t& xpre, half8_t& gpre) {
-            const bool gin = (p >= 0) && (p < H) && (p <= he);
-            unsigned char* gslot = smem + (p & 3) * GSLOT;
-            stage(p, xpre, gpre);
-            __syncthreads();
-            flush_row(parity ^ 1);
-            prefetch(p + 2, xpre, gpre);
-            __builtin_amdgcn_sched_barrier(0);
-            if (gin) {
-#pragma unroll
-                for (int xr = 0; xr < RO + 2; ++xr) {
-                    uint32_t r[3];
-#pragma unroll
-                    for (int k = 0; k < 3; ++k)
-                        r[k] = *reinterpret_cast<const uint32_t*>(gslot + dboff[k] + xr * PDP * PB);
-                    half4_t B[2];
-                    split_operands3(r, B[0], B[1]);
-#pragma unroll
-                    for (int kw = 0; kw < 3; ++kw) {
-                        if (xr - kw >= 0 && xr - kw < RO) {
-#pragma unroll
-                            for (int e = 0; e < 2; ++e)
-                                T[xr - kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(wA[kw][e], B[e], T[xr - kw][e], 0, 0, 0);
+            auto step = [&](int p, half8_t& xpre, half8_t& gpre) {
+                const bool gin = (p >= 0) && (p < H) && (p <= he);
+                unsigned char* gslot = smem + (p & 3) * GSLOT;
+                stage(p, xpre, gpre);
+                __syncthreads();
+                flush_row(parity ^ 1);
+                prefetch(p + 2, xpre, gpre);
+                __builtin_amdgcn_sched_barrier(0);
+                if (gin) {
+    #pragma unroll
+                    for (int xr = 0; xr < RO + 2; ++xr) {
+                        uint32_t r[3];
+    #pragma unroll
+                        for (int k = 0; k < 3; ++k)
+                            r[k] = *reinterpret_cast<const uint32_t*>(gslot + dboff[k] + xr * PDP * PB);
+                        half4_t B[2];
+                        split_operands3(r, B[0], B[1]);
+    #pragma unroll
+                        for (int kw = 0; kw < 3; ++kw) {
+                            if (xr - kw >= 0 && xr - kw < RO) {
+    #pragma unroll
+                                for (int e = 0; e < 2; ++e)
+                                    T[xr - kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(wA[kw][e], B[e], T[xr - kw][e], 0, 0, 0);
+                            }
                         }
                     }
                 }
-            }
-            const int ho = p - 1;  // dx plane p-1 is complete
-            const bool store = (ho >= hs) && (ho < he);
-            pending_row = store ? ho : -1;
-            if (store) {
-                unsigned char* otile = smem + Cfg::OT_OFF + parity * Cfg::OT_BYTES;
-#pragma unroll
-                for (int o = 0; o < RO; ++o) {
-                    half2_t v;
-#pragma unroll
-                    for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
-                    if constexpr (BOUNCE) {
-                        *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
-                    } else {
-                        if (oval[o])
-                            __builtin_nontemporal_store(
-                                v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(dxn + ho * plane_stride) + ooff[o]));
+                const int ho = p - 1;  // dx plane p-1 is complete
+                const bool store = (ho >= hs) && (ho < he);
+                pending_row = store ? ho : -1;
+                if (store) {
+                    unsigned char* otile = smem + Cfg::OT_OFF + parity * Cfg::OT_BYTES;
+    #pragma unroll
+                    for (int o = 0; o < RO; ++o) {
+                        half2_t v;
+    #pragma unroll
+                        for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
+                        if constexpr (BOUNCE) {
+                            *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
+                        } else {
+                            if (oval[o])
+                                __builtin_nontemporal_store(
+                                    v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(dxn + ho * plane_stride) + ooff[o]));
+                        }
                     }
                 }
+    #pragma unroll
+                for (int o = 0; o < RO; ++o)
+    #pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        T[o][e][2] = T[o][e][1];
+                        T[o][e][1] = T[o][e][0];
+                        T[o][e][0] = 0.0f;
+                    }
+                parity ^= 1;
+            };
+            for (int p = hs - 1;;) {
+                step(p, xpre0, gpre0);
+                if (++p > he + 1) break;
+                step(p, xpre1, gpre1);
+                if (++p > he + 1) break;
             }
-#pragma unroll
-            for (int o = 0; o < RO; ++o)
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    T[o][e][2] = T[o][e][1];
-                    T[o][e][1] = T[o][e][0];
-                    T[o][e][0] = 0.0f;
-                }
-            parity ^= 1;
-        };
-        for (int p = hs - 1;;) {
-            step(p, xpre0, gpre0);
-            if (++p > he + 1) break;
-            step(p, xpre1, gpre1);
-            if (++p > he + 1) break;
-        }
-        __syncthreads();  // the last tile is written, every wavefront is done with the staging buffers
-        flush_row(parity ^ 1);
+            __syncthreads();  // the last tile is written, every wavefront is done with the staging buffers
+            flush_row(parity ^ 1);
         }  // segments
         __syncthreads();  // (the other role: staging buffers are dead)
         __syncthreads();  // (the other role: partial sums are in LDS)
