@@ -432,6 +432,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const Fwd
 // channels the cost is 3 matrix instructions, the operand comes from LDS as three dwords (two
 // channels per lane and position) split into the even and the odd channel by byte permutes.
 // The arithmetic is a fraction of the memory time; global loads run two planes ahead.
+constexpr bool kBounceNarrow = true;
+
 template <int CG_, int TW_, int TD_, int NT_>
 struct FmCfg {
     static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, NWAVE = NT_ / 64;
@@ -481,7 +483,7 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     // write traffic than the tensor holds.  So a finished plane is written to the tile as dwords and leaves one
     // step later, behind that step's barrier, as one 16-byte chunk per thread: whole lines, one store instruction
     // instead of RO.  Narrower slabs write runs of 256 contiguous bytes anyway and store directly.
-    constexpr bool BOUNCE = MODE != 2 && SC == 64;
+    constexpr bool BOUNCE = MODE != 2 && (SC == 64 || kBounceNarrow);
     constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
     static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
     constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);
@@ -578,7 +580,9 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
 #pragma unroll
     for (int k = 0; k < 3; ++k) boff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
     // output tile: the halves of odd positions are swapped so that the four positions of a write spread over all banks
-    auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
+    auto ot_swz = [](int pos, int cbyte) {
+        return PB == 128 ? pos * PB + ((cbyte + 64 * (pos & 1)) & 127) : pos * PB + cbyte;
+    };
     int owr[RO];  // the lane's dword (two channels) of position pgrp + rr in the output rows ra .. ra+RO-1
 #pragma unroll
     for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
@@ -794,7 +798,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     // write traffic than the tensor holds.  So a finished plane is written to the tile as dwords and leaves one
     // step later, behind that step's barrier, as one 16-byte chunk per thread: whole lines, one store instruction
     // instead of RO.  Narrower slabs write runs of 256 contiguous bytes anyway and store directly.
-    constexpr bool BOUNCE = MODE != 2 && SC == 64;
+    constexpr bool BOUNCE = MODE != 2 && (SC == 64 || kBounceNarrow);
     constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
     static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
     constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);

@@ -609,7 +609,7 @@ struct BsCfg {
     static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, SLOT = R * PDP * PB;
     static constexpr int GSLOT = SLOT + (SC == 8 ? 16 : 32);  // lanes j read different slots: shift their banks apart
     static constexpr int XOFF = 4 * GSLOT;
-    static constexpr bool BOUNCE = SC == 64;  // dx leaves through the output tile as whole 128-byte lines
+    static constexpr bool BOUNCE = true;  // dx leaves through an LDS output tile as 16-byte chunks (whole lines)
     static constexpr int NPOS = TW * TD, OT_BYTES = BOUNCE ? NPOS * PB : 0, OT_OFF = XOFF + 2 * SLOT;
     static constexpr int DUMP = OT_OFF + 2 * OT_BYTES, STAGE_BYTES = DUMP + 16;
     static constexpr int NCH = R * (TD + 2) * CG;  // 16-byte chunks of a staged plane: one per thread, t < NCH
@@ -758,7 +758,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
                     wA[kw][e] = v;
                 }
         }
-        auto ot_swz = [](int pos, int cbyte) { return pos * PB + ((cbyte + 64 * (pos & 1)) & 127); };
+        auto ot_swz = [](int pos, int cbyte) {
+            return PB == 128 ? pos * PB + ((cbyte + 64 * (pos & 1)) & 127) : pos * PB + cbyte;
+        };
         while (next_segment()) {
             // lane constants from an opaque copy of the thread index: computed per segment, so that what only the
             // segment's set-up needs is not held in registers across the march
