@@ -41,8 +41,8 @@ V = H * W * D
 # (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000):
 # profiles/dwconv_fwd_wgrad_c64_readme_shape.md.
 MEASURED_TRAFFIC_BYTES = {
-    ('dwconv_fwd', 64): 4321415414,    # 2.314 GB read + 2.007 GB written (1.077 x algorithmic)
-    ('dwconv_wgrad', 64): 4397211884,  # 4.394 GB read + 0.004 GB written (1.095 x algorithmic)
+    ('dwconv_fwd', 64): 4339515866,    # 2.332 GB read + 2.007 GB written (1.081 x algorithmic)
+    ('dwconv_wgrad', 64): 4376702479,  # 4.373 GB read + 0.004 GB written (1.090 x algorithmic)
 }
 
 

@@ -432,8 +432,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const Fwd
 // channels the cost is 3 matrix instructions, the operand comes from LDS as three dwords (two
 // channels per lane and position) split into the even and the odd channel by byte permutes.
 // The arithmetic is a fraction of the memory time; global loads run two planes ahead.
-constexpr bool kBounceNarrow = true;
-
 template <int CG_, int TW_, int TD_, int NT_>
 struct FmCfg {
     static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, NWAVE = NT_ / 64;
@@ -478,12 +476,13 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     constexpr int NPOS = Cfg::TW * TD, RT = SC + 8, RY = COUT + 4;
     constexpr int KS = SC / 16, MT = COUT / 32, NPT = NPOS / 32;  // k = 16 per matrix instruction
     constexpr int T_OFF = Cfg::LDS_BYTES, Y_OFF = T_OFF + NPOS * RT * 2, A_OFF = Y_OFF + NPOS * RY * 2;
-    // modes 0 and 1 with a 64-channel slab: two output tiles [NPOS][PB] behind the staging buffers.  A wavefront
-    // owns 32 channels, i.e. 64-byte halves of the 128-byte positions; written directly they cost 10 % more HBM
-    // write traffic than the tensor holds.  So a finished plane is written to the tile as dwords and leaves one
-    // step later, behind that step's barrier, as one 16-byte chunk per thread: whole lines, one store instruction
-    // instead of RO.  Narrower slabs write runs of 256 contiguous bytes anyway and store directly.
-    constexpr bool BOUNCE = MODE != 2 && (SC == 64 || kBounceNarrow);
+    // modes 0, 1 and 3: two output tiles [NPOS][PB] behind the staging buffers.  A finished plane is written to the
+    // tile as dwords and leaves one step later, behind that step's barrier, as one 16-byte chunk per thread: whole
+    // lines, one store instruction instead of RO.  With a 64-channel slab a wavefront owns 64-byte halves of the
+    // 128-byte positions, which cost 10 % more HBM write traffic when written directly; narrower slabs would write
+    // full lines either way, but the single store and the registers it frees (the RO store offsets; the 256-thread
+    // shapes then hold four wavefronts per SIMD) are worth 3-20 % there.
+    constexpr bool BOUNCE = MODE != 2;
     constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
     static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
     constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);
@@ -602,16 +601,11 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
                     o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(yn + pending_row * plane_stride) + ogo));
         }
     };
-    // direct stores (narrow slabs): the lane's dword of position pgrp + rr in the output rows ra .. ra+RO-1
+    // mode 3: whether the lane's position pgrp + rr of the output rows ra .. ra+RO-1 lies inside the volume
     const int od = d0 + pgrp + rr;
-    uint32_t ooff[RO];
     bool oval[RO];
 #pragma unroll
-    for (int o = 0; o < RO; ++o) {
-        const int w = w0 + ra + o;
-        oval[o] = (od < D) && (w < W);
-        ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
-    }
+    for (int o = 0; o < RO; ++o) oval[o] = (od < D) && (w0 + ra + o < W);
 
     float4_t T[RO][2];
 #pragma unroll
@@ -691,12 +685,8 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
                 }
                 if constexpr (MODE == 2) {
                     *reinterpret_cast<half2_t*>(tt + ((ra + o) * TD + pgrp + rr) * RT + half * 32 + 2 * q) = v;
-                } else if constexpr (BOUNCE) {
-                    *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
                 } else {
-                    if (oval[o])
-                        __builtin_nontemporal_store(
-                            v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(yn + ho * plane_stride) + ooff[o]));
+                    *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
                 }
             }
             if constexpr (MODE == 2) {
@@ -793,12 +783,13 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     constexpr int NPOS = Cfg::TW * TD, RT = SC + 8, RY = COUT + 4;
     constexpr int KS = SC / 16, MT = COUT / 32, NPT = NPOS / 32;  // k = 16 per matrix instruction
     constexpr int T_OFF = Cfg::LDS_BYTES, Y_OFF = T_OFF + NPOS * RT * 2, A_OFF = Y_OFF + NPOS * RY * 2;
-    // modes 0 and 1 with a 64-channel slab: two output tiles [NPOS][PB] behind the staging buffers.  A wavefront
-    // owns 32 channels, i.e. 64-byte halves of the 128-byte positions; written directly they cost 10 % more HBM
-    // write traffic than the tensor holds.  So a finished plane is written to the tile as dwords and leaves one
-    // step later, behind that step's barrier, as one 16-byte chunk per thread: whole lines, one store instruction
-    // instead of RO.  Narrower slabs write runs of 256 contiguous bytes anyway and store directly.
-    constexpr bool BOUNCE = MODE != 2 && (SC == 64 || kBounceNarrow);
+    // modes 0, 1 and 3: two output tiles [NPOS][PB] behind the staging buffers.  A finished plane is written to the
+    // tile as dwords and leaves one step later, behind that step's barrier, as one 16-byte chunk per thread: whole
+    // lines, one store instruction instead of RO.  With a 64-channel slab a wavefront owns 64-byte halves of the
+    // 128-byte positions, which cost 10 % more HBM write traffic when written directly; narrower slabs would write
+    // full lines either way, but the single store and the registers it frees (the RO store offsets; the 256-thread
+    // shapes then hold four wavefronts per SIMD) are worth 3-20 % there.
+    constexpr bool BOUNCE = MODE != 2;
     constexpr int OT_OFF = Cfg::LDS_BYTES, OT_BYTES = NPOS * PB;
     static_assert(!BOUNCE || NPOS * CG == NT, "one 16-byte output chunk per thread");
     constexpr int SMEM_BYTES = MODE == 2 ? A_OFF + MT * KS * 64 * 16 : (BOUNCE ? OT_OFF + 2 * OT_BYTES : Cfg::LDS_BYTES);

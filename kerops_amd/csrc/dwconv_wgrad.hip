@@ -609,14 +609,14 @@ struct BsCfg {
     static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, SLOT = R * PDP * PB;
     static constexpr int GSLOT = SLOT + (SC == 8 ? 16 : 32);  // lanes j read different slots: shift their banks apart
     static constexpr int XOFF = 4 * GSLOT;
-    static constexpr bool BOUNCE = true;  // dx leaves through an LDS output tile as 16-byte chunks (whole lines)
-    static constexpr int NPOS = TW * TD, OT_BYTES = BOUNCE ? NPOS * PB : 0, OT_OFF = XOFF + 2 * SLOT;
+    // dx leaves through two LDS output tiles as 16-byte chunks (whole lines, one store per thread and plane)
+    static constexpr int NPOS = TW * TD, OT_BYTES = NPOS * PB, OT_OFF = XOFF + 2 * SLOT;
     static constexpr int DUMP = OT_OFF + 2 * OT_BYTES, STAGE_BYTES = DUMP + 16;
     static constexpr int NCH = R * (TD + 2) * CG;  // 16-byte chunks of a staged plane: one per thread, t < NCH
     static constexpr int RED_BYTES = NPART * 27 * SC * 4;
     static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
     static_assert(NCH <= NT && RO == 4 && TD % (4 * NSUB) == 0 && NPART % GD == 0 && TW % RSPLIT == 0, "even split");
-    static_assert(!BOUNCE || NPOS * CG == RWAVES * 64, "the dx role stores the tile: one 16-byte chunk per thread");
+    static_assert(NPOS * CG == RWAVES * 64, "the dx role stores the tile: one 16-byte chunk per thread");
     static_assert(STAGE_BYTES % 16 == 0, "16-byte chunks");
 };
 
@@ -625,7 +625,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
-    constexpr bool BOUNCE = Cfg::BOUNCE;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
     const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
@@ -770,7 +769,6 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
             const int b = lane / 4, rr = lane % 4;
             const int q = b % NQ, sub = b / NQ;
             const int cb = half * 64 + q * 4;
-            const int c0 = cslab + half * 32 + 2 * q;
             const int pgrp = (gd * NSUB + sub) * 4;
             int dboff[3];
     #pragma unroll
@@ -778,29 +776,19 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
             int owr[RO];
     #pragma unroll
             for (int o = 0; o < RO; ++o) owr[o] = ot_swz((ra + o) * TD + pgrp + rr, cb);
-            // 64-channel slabs: the threads of this role store the tile, one 16-byte chunk each; narrower slabs
-            // store their dwords directly (runs of 256 contiguous bytes per instruction)
+            // the threads of this role store the output tile, one 16-byte chunk each
             const int opos = tl / CG, ocq = tl % CG;
             const int ord = ot_swz(opos, ocq * 16);
             const int ow = w0 + opos / TD, odd = d0 + opos % TD;
             const bool ovalid = (ow < W) && (odd < D);
             const uint32_t ogo = ovalid ? (uint32_t)(((ow * D + odd) * C + cslab + ocq * 8) * 2) : 0u;
-            const int od = d0 + pgrp + rr;
-            uint32_t ooff[RO];
-            bool oval[RO];
-    #pragma unroll
-            for (int o = 0; o < RO; ++o) {
-                const int w = w0 + ra + o;
-                oval[o] = (od < D) && (w < W);
-                ooff[o] = oval[o] ? (uint32_t)(((w * D + od) * C + c0) * 2) : 0u;
-            }
             parity = 0;
             prefetch(hs - 1, xpre0, gpre0);
             prefetch(hs, xpre1, gpre1);
             __syncthreads();  // the zero fill is complete before staging writes anything
             int pending_row = -1;
             auto flush_row = [&](int par) {
-                if (BOUNCE && pending_row >= 0) {  // workgroup-uniform
+                if (pending_row >= 0) {  // workgroup-uniform
                     const half8_t o8 = *reinterpret_cast<const half8_t*>(smem + Cfg::OT_OFF + par * Cfg::OT_BYTES + ord);
                     if (ovalid)
                         __builtin_nontemporal_store(
@@ -850,13 +838,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
                         half2_t v;
     #pragma unroll
                         for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
-                        if constexpr (BOUNCE) {
-                            *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
-                        } else {
-                            if (oval[o])
-                                __builtin_nontemporal_store(
-                                    v, reinterpret_cast<half2_t*>(reinterpret_cast<char*>(dxn + ho * plane_stride) + ooff[o]));
-                        }
+                        *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
                     }
                 }
     #pragma unroll
