@@ -595,7 +595,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
 // The two products run on different wavefronts: all 8 wavefronts of a workgroup stage the planes of x and g
 // (with halo) into LDS, then wavefronts 0-3 run the input-gradient scheme (and store dx) while wavefronts 4-7
 // run the weight-gradient scheme on the same LDS data, each role in its own loop with the same sequence of
-// workgroup barriers.  A role keeps only its own accumulators: 112-122 registers and 35-62 KB of LDS, so two
+// workgroup barriers.  A role keeps only its own accumulators: 123-128 registers and 42-62 KB of LDS, so two
 // workgroups (16 wavefronts) are resident per CU, where running both schemes in every wavefront needs ~190
 // registers and holds 8 wavefronts (that version took 1.55 ms at (1,64,350,350,128), this one 1.42 ms; the
 // two separate kernels 1.54-1.58 ms).  An 8x8 patch with 16 wavefronts re-reads less halo but leaves one
