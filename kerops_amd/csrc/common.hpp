@@ -11,6 +11,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cmath>
+
 #include "../../include/kerops_hip.h"
 
 namespace kerops {
@@ -104,8 +106,8 @@ static inline int pick_h_chunk(int H, int64_t per_plane, int slots, int setup)
         const int h = ceil_div(H, c);
         const int chunks = ceil_div(H, h);
         if (chunks != c) continue;  // the same split as a smaller c
-        const int64_t rounds = ceil_div64(per_plane * chunks, slots);
-        const double cost = (double)rounds * (h + 2 + setup) * (1.0 + 0.004 * c);
+        const double rounds = std::ceil((double)per_plane * chunks / slots);  // (doubles: no overflow at absurd sizes)
+        const double cost = rounds * ((double)h + 2 + setup) * (1.0 + 0.004 * c);
         if (cost < best) {
             best = cost;
             best_h = h;
@@ -130,7 +132,9 @@ static inline BalancedSplit make_balanced(int H, int64_t tiles, int slots, int g
 {
     BalancedSplit b;
     b.group = (uint32_t)group;
-    b.units = ((tiles + group - 1) / group) * H;
+    const int64_t bundles = tiles / group + (tiles % group != 0);
+    // more plane steps than the kernels' 32-bit counters hold: any value >= 2^31 makes the callers fall back
+    b.units = bundles > (1LL << 31) / H ? (1LL << 40) : bundles * H;
     // a share of fewer than 2 rows is all halo planes: use fewer groups then
     b.ngroups = (uint32_t)std::min<int64_t>(std::max(1, slots / group), std::max<int64_t>(1, b.units / 2));
     return b;
