@@ -12,8 +12,9 @@ channels_last_3d (the README-shape forward and weight-gradient target configurat
                           % of the bandwidth torch.clone reaches on the same tensor in this run
   roofline                the dominant kernel of the step, timed live with HIP events on the
                           stream the kernels run on
-  ops                     the same figures for the other ops of the path (Stats, ApplyBNReLU,
-                          AvgPoolCeilStats, QuantUint8Window) and for every C of the README table
+  ops                     the same figures for every other op of the path (statistics, BN-ReLU, pooling,
+                          quantisers, their backward ops, the fused and the linear ops) and for every C of
+                          the README table
   cpu_baseline            the CPU oracle (oracle/kerops_oracle.c, OpenMP) on a bounded crop of the
                           same workload, scaled by the voxel ratio; torch's CPU conv3d(groups=C),
                           the reference tests' ground truth, is timed beside it
