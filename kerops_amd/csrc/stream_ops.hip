@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kStreamThreads) void stats_bwd_kernel(const half_t*
         }
         return o;
     };
-    constexpr int U = ADD ? 2 : 4;  // chunks in flight per lane and input stream
+    constexpr int U = 4;  // chunks in flight per lane and input stream
     for (; i + (U - 1) * T < nchunks; i += U * T) {
         hv v[U], g[U];
 #pragma unroll
