@@ -186,7 +186,7 @@ def _same_bits_or_nan(a, b):
     return bool((eq | both_nan).all())
 
 
-@pytest.mark.parametrize('grad_scale', [1.0, 1e-30, 1e30, 3e38])
+@pytest.mark.parametrize('grad_scale', [1.0, 1e-30, 1e-37, 1e-42, 1e30, 3e38])
 def test_backward_ops_bit_exact_on_special_values(grad_scale):
     """The divisions of StatsBackward / AddStatsBackward / AvgPoolCeilStatsBackward must give the oracle's
     (IEEE) bits for every operand: signed zeros, infinities, NaNs, subnormals, huge and tiny gradients."""
