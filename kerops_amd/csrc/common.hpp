@@ -123,7 +123,8 @@ static inline int pick_h_chunk(int H, int64_t per_plane, int slots, int setup)
 // where uniform chunks leave the last round of workgroups partly filled (2-10 % slower at the shapes measured).
 // `row_len` = tiles (times slabs) in one row along D.  The group size is chosen by a cost model fitted to
 // sweeps at (1, C, 350, 350, 128), C = 8..128: time ~ plane steps of a group, 10 % / (tile rows in a bundle) for
-// the halo rows that neighbouring bundles no longer share in L2, a fixed cost per workgroup and per crossing.
+// the halo rows that neighbouring bundles no longer share in L2, 4 % for a group that does not fit one XCD, a
+// fixed cost per workgroup and per crossing.
 struct BalancedSplit {
     uint32_t group, ngroups;
     int64_t units;  // bundles * H
@@ -139,12 +140,14 @@ static inline BalancedSplit make_balanced(int H, int64_t tiles, int slots, int g
     b.ngroups = (uint32_t)std::min<int64_t>(std::max(1, slots / group), std::max<int64_t>(1, b.units / 2));
     return b;
 }
-static inline double balanced_cost(const BalancedSplit& b, int H, int row_len, int setup)
+static inline double balanced_cost(const BalancedSplit& b, int H, int row_len, int slots, int setup)
 {
     const double share = (double)((b.units + b.ngroups - 1) / b.ngroups);
     const double crossings = share / H;  // expected bundle boundaries inside a share
     const double rows = (double)b.group / row_len;
-    return (share + 2 + setup + crossings * 5.0) * (1.0 + 0.1 / rows) * (1.0 + 0.004 * H / share);
+    // a group larger than the workgroups one XCD holds is spread over several L2s (measured: 2-3 % slower)
+    const double spread = (int)b.group > slots / 8 ? 1.04 : 1.0;
+    return (share + 2 + setup + crossings * 5.0) * (1.0 + 0.1 / rows) * (1.0 + 0.004 * H / share) * spread;
 }
 // slab_mult: the group size must be a multiple of it (kernels that keep per-slab state across bundles)
 static inline BalancedSplit pick_balanced(int H, int64_t tiles, int row_len, int slots, int setup, int slab_mult)
@@ -155,7 +158,7 @@ static inline BalancedSplit pick_balanced(int H, int64_t tiles, int row_len, int
         if (g < 1 || g > slots || g % slab_mult != 0) return;
         if (g >= tiles + row_len && g > slab_mult) return;  // more than a row of idle members
         const BalancedSplit b = make_balanced(H, tiles, slots, (int)g);
-        const double c = balanced_cost(b, H, row_len, setup);
+        const double c = balanced_cost(b, H, row_len, slots, setup);
         if (c < best_cost) {
             best_cost = c;
             best = b;

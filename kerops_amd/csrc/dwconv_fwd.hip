@@ -803,6 +803,15 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     float ssum[2] = {0.0f, 0.0f}, ssq[2] = {0.0f, 0.0f};
     constexpr bool SEGMENTS = MODE != 2;  // the fused pointwise mode always runs one segment (uniform chunks)
     SegmentWalk walk = segment_walk_begin(wg_slot, SEGMENTS ? a.bal_group : 0u, a.bal_q, a.bal_r);
+    if constexpr (MODE == 0 || MODE == 1) {
+        // Two slabs (128 channels): the first half of a group's members takes slab 0 of the bundle's patches, the
+        // second half slab 1, instead of alternating.  A group of 128 spans two XCDs; this way each of them holds
+        // all four patch rows of the bundle (one slab each) and the rows share their halo voxels in its L2.
+        if (a.n_slab == 2 && walk.group > 0 && walk.group % 2 == 0) {
+            const uint32_t halfg = walk.group / 2;
+            walk.member = (walk.member % halfg) * 2 + walk.member / halfg;
+        }
+    }
     uint32_t tile;
     int hs, he;
     const uint32_t per_sample = (uint32_t)(a.n_slab * a.n_dt * a.n_wt);
