@@ -50,6 +50,7 @@ extern "C" {
 
 #define KEROPS_DTYPE_F16 0
 #define KEROPS_DTYPE_F32 1
+#define KEROPS_DTYPE_BF16 2
 
 int kerops_hip_version(void);
 const char* kerops_last_error_string(void);
@@ -182,14 +183,15 @@ int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad
 
 /* u8 = (uint8)(((clip(float(x), -window, window) + window) / (2*window)) * 255),
  * each step one IEEE fp32 operation, conversion by truncation.  dtype is the
- * KEROPS_DTYPE_* tag of x.  Flat over numel elements.
+ * KEROPS_DTYPE_* tag of x (fp16, fp32 or bf16; the reference kernel converts whatever
+ * floating type it is given to fp32 first).  Flat over numel elements.
  * Replaces `_QuantUint8Window_impl[(numblocks,)](...)`:
  * kerops/ops/quantization.py:19 (kernel kerops/kernels/quantization.py:6-27). */
 int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int64_t numel, float window, int32_t blocks,
                            void* stream);
 
 /* out = float(u8) * (2*window/255) - window (scale formed once in fp32; one
- * multiply, one subtract), stored as dtype.
+ * multiply, one subtract), stored as dtype (fp16, fp32 or bf16; one RNE rounding).
  * Replaces `_DequantUint8Window_impl[(numblocks,)](...)`:
  * kerops/ops/quantization.py:34 (kernel kerops/kernels/quantization.py:31-49). */
 int kerops_dequant_u8_window(const void* q, void* out, int32_t dtype, int64_t numel, float window, int32_t blocks,

@@ -17,7 +17,7 @@ KEROPS_E_UNSUPPORTED_C = -2
 KEROPS_E_WORKSPACE = -3
 KEROPS_E_LAUNCH = -4
 
-DTYPE_TAGS = {torch.float16: 0, torch.float32: 1}
+DTYPE_TAGS = {torch.float16: 0, torch.float32: 1, torch.bfloat16: 2}
 
 _p = ctypes.c_void_p
 _i32 = ctypes.c_int32

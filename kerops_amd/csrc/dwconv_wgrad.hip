@@ -1057,6 +1057,13 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
         }
         lane_channels = 16;
     }
+    // only the all-zero triple selects the built-in shape; anything else must name a positive patch
+    // (checked before the extents are divided by it) and is matched against the built kernels at launch
+    if (tile_w <= 0 || tile_d <= 0 || tile_w > 1024 || tile_d > 1024 || lane_channels <= 0) {
+        set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, tile_w, tile_d,
+                  lane_channels);
+        return KEROPS_E_BADARG;
+    }
     p->cl = lane_channels;
     p->tile_w = tile_w;
     p->tile_d = tile_d;

@@ -6,7 +6,7 @@
 //
 // Cout in {64, 128}: one kernel.  The matrix-core depthwise kernel hands every finished output plane of
 // its 8x8 patch (64 positions x 64 channels, rounded to fp16) through an LDS tile to the pointwise GEMM
-// on the 32x32x8 matrix instruction; t never reaches memory and the workspace only holds one max|y|
+// on the 32x32x16 matrix instruction; t never reaches memory and the workspace only holds one max|y|
 // per workgroup.  Other Cout: two kernels (depthwise with the affine+ReLU epilogue, then the
 // pointwise kernel with the running max), t goes through the caller's workspace.
 #include "common.hpp"
@@ -25,6 +25,11 @@ extern "C" int64_t kerops_dwsep_block_workspace_bytes(int32_t N, int32_t H, int3
     if (Cin != 64 || !(Cout == 16 || Cout == 32 || Cout == 64 || Cout == 128)) {
         set_error("dwsep_block: built for Cin = 64 and Cout in {16,32,64,128} (got %d -> %d)", Cin, Cout);
         return KEROPS_E_UNSUPPORTED_C;
+    }
+    // 32-bit offsets inside a plane of x and of y, 64-bit plane bases (as for every convolution entry point)
+    if (plane_exceeds_i32(W, D, Cin) || plane_exceeds_i32(W, D, Cout) || volume_exceeds_i64(N, H, W, D, Cout)) {
+        set_error("dwsep_block: one (W,D,C) plane must stay below 2^31 elements and the volume below 2^60");
+        return KEROPS_E_BADARG;
     }
     if (Cout >= 64) {
         const int nb = dwsep_fused_blocks(N, H, W, D);

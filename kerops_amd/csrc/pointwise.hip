@@ -207,6 +207,10 @@ static int launch_pw(const half_t* x, const half_t* Wm, const half_t* add, half_
                      bool relu_in, bool absmax, int blocks, hipStream_t s, const float* scale = nullptr,
                      const float* shift = nullptr)
 {
+    if (absmax && (add || scale)) {  // no instantiation keeps the running max next to a residual or the affine map
+        set_error("pointwise: the running max is built without residual add and without the affine map");
+        return KEROPS_E_BADARG;
+    }
     if (scale) {  // the affine map ends in a ReLU of its own
         if (add) {
             hipLaunchKernelGGL((pointwise_kernel<CIN, COUT, false, true, false, true>), dim3(blocks), dim3(kPwThreads), 0,

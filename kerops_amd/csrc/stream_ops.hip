@@ -215,6 +215,7 @@ __global__ __launch_bounds__(kStreamThreads) void bnrelu_bwd_kernel(const half_t
 }
 
 // ------------------------------------------------------------ quantisers
+typedef __bf16 bf16_t;
 template <typename T>
 __device__ __forceinline__ float to_f32(T v)
 {
@@ -243,8 +244,105 @@ __device__ __forceinline__ uint32_t quant_u8_one(float t, float window, float tw
     return (uint32_t)t;  // truncation toward zero
 }
 
-// The byte-wide side of the quantisers is moved 16 bytes per lane like everything else: a thread
-// handles 16 consecutive elements (two 16-byte fp16 loads or four fp32 loads per 16-byte store).
+// The quantisers move 16 bytes per lane on their wide side (8 two-byte or 4 four-byte elements) and the matching
+// 8 or 4 bytes on the byte side, consecutive lanes on consecutive pieces: every load and every store instruction of
+// a wavefront covers one contiguous run of whole 128-byte lines (1 KiB wide side, 512 or 256 bytes byte side).
+// A lane that took 16 bytes of the byte side instead would touch the wide side with two or four accesses that
+// interleave with its neighbours' (alternate 16-byte pieces per instruction): measured, that wrote 1.135x the
+// tensor size to HBM in partial lines.
+template <typename T>
+struct QuantUnit {
+    static constexpr int E = 16 / (int)sizeof(T);  // elements of one lane and step
+    typedef T wide_t __attribute__((ext_vector_type(E)));
+    typedef uint32_t bytes_t __attribute__((ext_vector_type(E / 4)));
+};
+template <>
+struct QuantUnit<float> {
+    static constexpr int E = 4;
+    typedef float wide_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t bytes_t;
+};
+__device__ __forceinline__ uint32_t bytes_word(const uint32_t& v, int) { return v; }
+__device__ __forceinline__ uint32_t bytes_word(const u32x2_t& v, int k) { return v[k]; }
+__device__ __forceinline__ void set_bytes_word(uint32_t& v, int, uint32_t w) { v = w; }
+__device__ __forceinline__ void set_bytes_word(u32x2_t& v, int k, uint32_t w) { v[k] = w; }
+
+constexpr int kQuantInFlight = 4;  // steps in flight per lane
+
+template <typename T, bool FAST>
+__global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
+                                                                  int64_t numel, float window, float r_two_w)
+{
+    typedef QuantUnit<T> QU;
+    constexpr int E = QU::E, U = kQuantInFlight;
+    const float two_w = __fmul_rn(2.0f, window);
+    const int64_t nunits = numel / E;
+    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
+    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
+    auto one = [&](const typename QU::wide_t& v) {
+        typename QU::bytes_t o;
+#pragma unroll
+        for (int k = 0; k < E / 4; ++k) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w |= quant_u8_one<FAST>(to_f32(v[4 * k + j]), window, two_w, r_two_w) << (8 * j);
+            set_bytes_word(o, k, w);
+        }
+        return o;
+    };
+    const typename QU::wide_t* xv = reinterpret_cast<const typename QU::wide_t*>(x);
+    typename QU::bytes_t* qv = reinterpret_cast<typename QU::bytes_t*>(q);
+    int64_t i = gid;
+    for (; i + (U - 1) * Tn < nunits; i += U * Tn) {
+        typename QU::wide_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(xv + i + u * Tn);
+#pragma unroll
+        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(v[u]), qv + i + u * Tn);
+    }
+    for (; i < nunits; i += Tn) __builtin_nontemporal_store(one(__builtin_nontemporal_load(xv + i)), qv + i);
+    if (gid == 0) {
+        for (int64_t k = nunits * E; k < numel; ++k)
+            q[k] = (uint8_t)quant_u8_one<FAST>(to_f32(x[k]), window, two_w, r_two_w);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kStreamThreads) void dequant_u8_kernel(const uint8_t* __restrict__ q,
+                                                                    T* __restrict__ out, int64_t numel, float window)
+{
+    typedef QuantUnit<T> QU;
+    constexpr int E = QU::E, U = kQuantInFlight;
+    const float scale = __fdiv_rn(__fmul_rn(2.0f, window), 255.0f);
+    const int64_t nunits = numel / E;
+    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
+    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
+    auto one = [&](const typename QU::bytes_t& b) {
+        typename QU::wide_t o;
+#pragma unroll
+        for (int j = 0; j < E; ++j)
+            o[j] = (T)__fsub_rn(__fmul_rn((float)((bytes_word(b, j / 4) >> (8 * (j % 4))) & 0xffu), scale), window);
+        return o;
+    };
+    const typename QU::bytes_t* qv = reinterpret_cast<const typename QU::bytes_t*>(q);
+    typename QU::wide_t* ov = reinterpret_cast<typename QU::wide_t*>(out);
+    int64_t i = gid;
+    for (; i + (U - 1) * Tn < nunits; i += U * Tn) {
+        typename QU::bytes_t b[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) b[u] = __builtin_nontemporal_load(qv + i + u * Tn);
+#pragma unroll
+        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(b[u]), ov + i + u * Tn);
+    }
+    for (; i < nunits; i += Tn) __builtin_nontemporal_store(one(__builtin_nontemporal_load(qv + i)), ov + i);
+    if (gid == 0) {
+        for (int64_t k = nunits * E; k < numel; ++k)
+            out[k] = (T)__fsub_rn(__fmul_rn((float)q[k], scale), window);
+    }
+}
+
+// 16 consecutive fp16 values per lane (two 16-byte loads) for one 16-byte store of bytes: the int8 pass
 template <typename T>
 __device__ __forceinline__ void load16(const T* p, float (&f)[16])
 {
@@ -257,69 +355,12 @@ __device__ __forceinline__ void load16(const T* p, float (&f)[16])
         f[8 + j] = (float)b[j];
     }
 }
-template <typename T>
-__device__ __forceinline__ void store16(T* p, const float (&f)[16])
-{
-    typedef T tv8 __attribute__((ext_vector_type(8)));
-    tv8 a, b;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        a[j] = (T)f[j];
-        b[j] = (T)f[8 + j];
-    }
-    __builtin_nontemporal_store(a, reinterpret_cast<tv8*>(p));
-    __builtin_nontemporal_store(b, reinterpret_cast<tv8*>(p + 8));
-}
 __device__ __forceinline__ u32x4_t pack16(const uint32_t (&b)[16])
 {
     u32x4_t o;
 #pragma unroll
     for (int w = 0; w < 4; ++w) o[w] = b[4 * w] | (b[4 * w + 1] << 8) | (b[4 * w + 2] << 16) | (b[4 * w + 3] << 24);
     return o;
-}
-
-template <typename T, bool FAST>
-__global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
-                                                                  int64_t numel, float window, float r_two_w)
-{
-    const float two_w = __fmul_rn(2.0f, window);
-    const int64_t ngroups = numel / 16;
-    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
-    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    for (int64_t i = gid; i < ngroups; i += Tn) {
-        float f[16];
-        load16<T>(x + i * 16, f);
-        uint32_t b[16];
-#pragma unroll
-        for (int j = 0; j < 16; ++j) b[j] = quant_u8_one<FAST>(f[j], window, two_w, r_two_w);
-        __builtin_nontemporal_store(pack16(b), reinterpret_cast<u32x4_t*>(q + i * 16));
-    }
-    if (gid == 0) {
-        for (int64_t k = ngroups * 16; k < numel; ++k)
-            q[k] = (uint8_t)quant_u8_one<FAST>(to_f32(x[k]), window, two_w, r_two_w);
-    }
-}
-
-template <typename T>
-__global__ __launch_bounds__(kStreamThreads) void dequant_u8_kernel(const uint8_t* __restrict__ q,
-                                                                    T* __restrict__ out, int64_t numel, float window)
-{
-    const float scale = __fdiv_rn(__fmul_rn(2.0f, window), 255.0f);
-    const int64_t ngroups = numel / 16;
-    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
-    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    for (int64_t i = gid; i < ngroups; i += Tn) {
-        const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(q + i * 16));
-        float f[16];
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-            f[j] = __fsub_rn(__fmul_rn((float)((v[j / 4] >> (8 * (j % 4))) & 0xffu), scale), window);
-        store16<T>(out + i * 16, f);
-    }
-    if (gid == 0) {
-        for (int64_t k = ngroups * 16; k < numel; ++k)
-            out[k] = (T)__fsub_rn(__fmul_rn((float)q[k], scale), window);
-    }
 }
 
 __global__ __launch_bounds__(kStreamThreads) void absmax_kernel(const half_t* __restrict__ y, float* __restrict__ ws,
@@ -605,6 +646,9 @@ extern "C" int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int
     if (dtype == KEROPS_DTYPE_F16) {
         if (fast) KEROPS_QU8_GO(half_t, true);
         else KEROPS_QU8_GO(half_t, false);
+    } else if (dtype == KEROPS_DTYPE_BF16) {
+        if (fast) KEROPS_QU8_GO(bf16_t, true);
+        else KEROPS_QU8_GO(bf16_t, false);
     } else if (dtype == KEROPS_DTYPE_F32) {
         if (fast) KEROPS_QU8_GO(float, true);
         else KEROPS_QU8_GO(float, false);
@@ -625,6 +669,9 @@ extern "C" int kerops_dequant_u8_window(const void* q, void* out, int32_t dtype,
     if (dtype == KEROPS_DTYPE_F16) {
         hipLaunchKernelGGL((dequant_u8_kernel<half_t>), dim3(blocks), dim3(kStreamThreads), 0, s, (const uint8_t*)q,
                            (half_t*)out, numel, window);
+    } else if (dtype == KEROPS_DTYPE_BF16) {
+        hipLaunchKernelGGL((dequant_u8_kernel<bf16_t>), dim3(blocks), dim3(kStreamThreads), 0, s, (const uint8_t*)q,
+                           (bf16_t*)out, numel, window);
     } else if (dtype == KEROPS_DTYPE_F32) {
         hipLaunchKernelGGL((dequant_u8_kernel<float>), dim3(blocks), dim3(kStreamThreads), 0, s, (const uint8_t*)q,
                            (float*)out, numel, window);

@@ -24,8 +24,9 @@ def PointwiseLinear(x, weight, relu_in=False):
     assert x.shape[1] == cin
     require_cuda(x, weight)
     n, _, h, w, d = x.shape
+    weight = weight.contiguous()  # bound to a name: a copy must outlive the launch
     out = torch.empty([n, h, w, d, cout], dtype=torch.float16, device=x.device).permute(0, 4, 1, 2, 3)
-    _lib.call('kerops_pointwise_f16', x.data_ptr(), weight.contiguous().data_ptr(), None, out.data_ptr(),
+    _lib.call('kerops_pointwise_f16', x.data_ptr(), weight.data_ptr(), None, out.data_ptr(),
               n * h * w * d, cin, cout, 1 if relu_in else 0, _lib.stream_of(x))
     return out
 
@@ -44,12 +45,15 @@ def DWSepBlock(x, dw_weight, scale, shift, pw_weight, *, reserved: ConfigurableA
 
     scale = scale.to(torch.float32).contiguous()
     shift = shift.to(torch.float32).contiguous()
+    # bound to names: copies of non-contiguous weights must outlive the launch
+    dw_weight = dw_weight.contiguous()
+    pw_weight = pw_weight.contiguous()
     ws_bytes = _lib.query('kerops_dwsep_block_workspace_bytes', n, h, w, d, cin, cout)
     ws = _lib.workspace(ws_bytes, x.device)
     y = torch.empty([n, h, w, d, cout], dtype=torch.float16, device=x.device).permute(0, 4, 1, 2, 3)
     absmax = torch.empty(1, dtype=torch.float32, device=x.device)
-    _lib.call('kerops_dwsep_block_f16', x.data_ptr(), dw_weight.contiguous().data_ptr(), scale.data_ptr(),
-              shift.data_ptr(), pw_weight.contiguous().data_ptr(), y.data_ptr(), absmax.data_ptr(), n, h, w, d, cin,
+    _lib.call('kerops_dwsep_block_f16', x.data_ptr(), dw_weight.data_ptr(), scale.data_ptr(),
+              shift.data_ptr(), pw_weight.data_ptr(), y.data_ptr(), absmax.data_ptr(), n, h, w, d, cin,
               cout, ws.data_ptr(), ws_bytes, _lib.stream_of(x))
     return y, absmax
 

@@ -27,7 +27,7 @@ def QuantUint8Window(x, window, *, num_warps: ConfigurableArg, l1_cache_bytes: C
                      blocks: ConfigurableArg):
     """u8 = trunc((clip(x, -window, window) + window) / (2*window) * 255), fp32 arithmetic."""
     require_cuda(x)
-    assert x.dtype in _lib.DTYPE_TAGS, 'fp16 or fp32 input'
+    assert x.dtype in _lib.DTYPE_TAGS, 'fp16, bf16 or fp32 input'
     assert _dense(x)
     output = torch.empty_like(x, dtype=torch.uint8)
     _lib.call('kerops_quant_u8_window', x.data_ptr(), _lib.DTYPE_TAGS[x.dtype], output.data_ptr(), x.numel(),
@@ -41,7 +41,7 @@ def DequantUint8Window(x, init_dtype, window, *, num_warps: ConfigurableArg, l1_
     """x_hat = float(u8) * (2*window/255) - window, stored as `init_dtype`."""
     require_cuda(x)
     assert x.dtype == torch.uint8
-    assert init_dtype in _lib.DTYPE_TAGS, 'fp16 or fp32 output'
+    assert init_dtype in _lib.DTYPE_TAGS, 'fp16, bf16 or fp32 output'
     assert _dense(x)
     output = torch.empty_like(x, dtype=init_dtype)
     _lib.call('kerops_dequant_u8_window', x.data_ptr(), output.data_ptr(), _lib.DTYPE_TAGS[init_dtype], x.numel(),

@@ -184,7 +184,8 @@ def quant_u8_window(x, window):
     q = torch.empty(xc.shape, dtype=torch.uint8)
     if xc.dtype == torch.float16:
         lib().oracle_quant_u8_window_f16(_p(xc), _p(q), _i64(xc.numel()), _f32(window))
-    elif xc.dtype == torch.float32:
+    elif xc.dtype in (torch.float32, torch.bfloat16):
+        xc = xc.float()  # bf16 -> fp32 is exact: the same first step as the kernel's
         lib().oracle_quant_u8_window_f32(_p(xc), _p(q), _i64(xc.numel()), _f32(window))
     else:
         raise TypeError(xc.dtype)
@@ -193,6 +194,8 @@ def quant_u8_window(x, window):
 
 def dequant_u8_window(q, init_dtype, window):
     qc = q.contiguous()
+    if init_dtype == torch.bfloat16:  # the fp32 value, rounded once to nearest-even by torch's conversion
+        return dequant_u8_window(q, torch.float32, window).to(torch.bfloat16)
     out = torch.empty(qc.shape, dtype=init_dtype)
     if init_dtype == torch.float16:
         lib().oracle_dequant_u8_window_f16(_p(qc), _p(out), _i64(qc.numel()), _f32(window))

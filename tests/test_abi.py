@@ -95,6 +95,22 @@ def test_workspace_queries():
     assert lib.kerops_absmax_workspace_bytes(10) == 40
 
 
+def test_wgrad_launch_knobs_are_checked_before_any_division():
+    # a zero or negative patch extent beside non-zero knobs used to divide by zero on the host
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    addr = (ctypes.addressof(buf) + 15) & ~15
+    for tw, td, cl in [(0, 8, 16), (8, 0, 16), (0, 8, 0), (-8, 8, 16), (8, -8, 16), (8, 8, -16), (8, 8, 0),
+                       (2 ** 31 - 1, 8, 16)]:
+        assert lib.kerops_dwconv_wgrad_workspace_bytes(1, 16, 16, 16, 64, tw, td, 0, cl) == _lib.KEROPS_E_BADARG
+        assert 'no kernel built' in _lib.last_error()
+        rc = lib.kerops_dwconv_wgrad_f16(addr, addr, addr, addr, 1 << 40, 1, 16, 16, 16, 64, tw, td, 0, cl, None)
+        assert rc == _lib.KEROPS_E_BADARG
+    # the fused block checks plane and volume limits like the other convolution entry points
+    assert lib.kerops_dwsep_block_workspace_bytes(1, 4, 2 ** 20, 2 ** 20, 64, 128) == _lib.KEROPS_E_BADARG
+    assert lib.kerops_dwsep_block_workspace_bytes(2 ** 31 - 1, 2 ** 31 - 1, 256, 256, 64, 128) == _lib.KEROPS_E_BADARG
+
+
 def test_split_of_the_h_march():
     # workgroup counts of the built-in launch shapes, read back from the workspace sizes (one partial per
     # workgroup).  The matrix-core convolution kernels use the balanced split by default: never more workgroups than

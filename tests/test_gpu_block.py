@@ -307,6 +307,27 @@ def test_dwsep_block_matches_oracle(shape, cout):
     assert qscale.item() == torch.tensor(amax.item(), dtype=torch.float32).div(127.0).item()
 
 
+@pytest.mark.parametrize('cout', [128, 32])
+def test_dwsep_block_noncontiguous_weights(cout):
+    """Both weights handed over as non-contiguous views (the torch (C,1,3,3,3) layout permuted, a transposed linear
+    weight): the op's contiguous copies must stay alive until the launch, the result equals the contiguous call."""
+    g = cpu_gen(77)
+    x = rand_cl3d(g, 1, 64, 6, 9, 10).to(DEV)
+    wt, wk = rand_dw_weight(g, 64)
+    scale = (torch.rand(64, generator=g) + 0.5).to(DEV)
+    shift = (torch.randn(64, generator=g) * math.sqrt(0.1)).to(DEV)
+    Wm = rand_pw(g, 64, cout)
+    dw_view = wt.to(DEV)[:, 0].permute(1, 2, 3, 0)
+    pw_view = Wm.t().contiguous().to(DEV).t()
+    assert not dw_view.is_contiguous() and not pw_view.is_contiguous()
+    y0, a0 = DWSepBlock(x, wk.to(DEV), scale, shift, Wm.to(DEV))
+    for _ in range(3):
+        y1, a1 = DWSepBlock(x, dw_view, scale, shift, pw_view)
+        assert torch.equal(y1, y0) and a1.item() == a0.item()
+    p0 = PointwiseLinear(x, Wm.to(DEV))
+    assert torch.equal(PointwiseLinear(x, pw_view), p0)
+
+
 def test_config5_full_shape():
     """(1,64,128,128,128) -> y (1,128,128,128,128) -> int8: slab comparison with the oracle,
     absmax against torch, int8 against the closed form on the build's own y."""

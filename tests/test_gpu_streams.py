@@ -269,6 +269,38 @@ def test_quant_u8_division_is_ieee_exact(window):
     assert torch.equal(QuantUint8Window(x32.to(DEV), window).cpu(), oracle.quant_u8_window(x32, window))
 
 
+@pytest.mark.parametrize('window', [1.0, 0.3, 7.77, 1e-3, 4097.0, 2.0 ** -59, 3e17])
+def test_quant_u8_fp32_every_bin_edge(window):
+    """fp32 inputs on and around every one of the 256 bin edges (the exact edge and the 16 fp32 neighbours on each
+    side), the window's ends and the values just outside it: the launch-constant division must give the oracle's
+    IEEE quotient on all of them, also where the quotient sits next to an integer multiple of 1/255."""
+    w = torch.tensor(window, dtype=torch.float32)
+    k = torch.arange(0, 256, dtype=torch.float64)
+    edges = ((k / 255.0 * 2.0 - 1.0) * float(w)).float()
+    edges = torch.cat([edges, torch.stack([-w, w, -w * 1.5, w * 1.5, torch.zeros(())])])
+    ulps = torch.arange(-16, 17, dtype=torch.int32)
+    x = (edges.view(torch.int32)[:, None] + ulps[None, :]).view(torch.float32).reshape(-1)
+    x = x[torch.isfinite(x)]
+    assert torch.equal(QuantUint8Window(x.to(DEV), window).cpu(), oracle.quant_u8_window(x, window))
+
+
+@pytest.mark.parametrize('window', [1.0, 3.0, 0.37, 6.5, 1e-4])
+def test_quant_u8_window_bf16_exhaustive(window):
+    """Every bf16 bit pattern (the reference kernel converts whatever floating type it is given to fp32 first,
+    kerops/kernels/quantization.py:21); the inverse stores bf16 with one rounding to nearest-even."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    x = bits[~torch.isnan(bits)]
+    q = QuantUint8Window(x.to(DEV), window)
+    rq = oracle.quant_u8_window(x, window)
+    assert q.dtype == torch.uint8 and torch.equal(q.cpu(), rq)
+    assert torch.equal(q.cpu(), torch.from_numpy(oracle.np_quant_u8_window(x.float().numpy(), window)))
+    allq = torch.arange(256, dtype=torch.uint8).repeat(37)[:9001]  # ragged length
+    dq = DequantUint8Window(allq.to(DEV), torch.bfloat16, window)
+    assert dq.dtype == torch.bfloat16
+    ref = oracle.dequant_u8_window(allq, torch.bfloat16, window)
+    assert torch.equal(dq.cpu().view(torch.int16), ref.view(torch.int16))
+
+
 def test_quant_u8_ragged_lengths_and_layouts():
     g = cpu_gen(5)
     for n in (1, 7, 8, 9, 1023, 100003):
