@@ -96,6 +96,19 @@ int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* works
                             int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d,
                             int32_t h_chunk, int32_t lane_channels, void* stream);
 
+/* kerops_dwconv_wgrad_f16 at its built-in launch shape for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * op allocates its partial buffer with torch on every call, kerops/ops/conv/dwconv_wgrad.py:54).  No workspace
+ * argument: the per-workgroup partials go to a 4 MiB device array that is part of the library (each GPU the
+ * library runs on holds its copy until the process ends); the entry point calls no hipMalloc, hipFree or other
+ * allocating routine.  The built-in launch shapes need at most 3.5 MB whatever the tensor size; a shape that
+ * would need more than 4 MiB returns KEROPS_E_WORKSPACE.  Same result, bit for bit, as kerops_dwconv_wgrad_f16
+ * with tile_w = tile_d = h_chunk = lane_channels = 0.  Calls on one GPU share the array: calls that overlap on
+ * one GPU (different streams) race.  The first call on a device looks up the array's address
+ * (hipGetSymbolAddress) and should be made outside graph capture. */
+int kerops_dwconv_wgrad_noalloc_f16(const void* x, const void* g, float* gw, int32_t N, int32_t H, int32_t W,
+                                    int32_t D, int32_t C, void* stream);
+
 /* Backward of the depthwise convolution in one pass over x and g (no reference counterpart: the reference has
  * no input gradient, TODO at kerops/kernels/dw_conv.py:145, and computes the weight gradient separately,
  * kerops/ops/conv/dwconv_wgrad.py:25-79):

@@ -36,6 +36,7 @@ SIGNATURES = {
     'kerops_dwconv_wgrad_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_dwconv_wgrad_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32,
                                                _i32, _p]),
+    'kerops_dwconv_wgrad_noalloc_f16': (ctypes.c_int, [_p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_stats_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'kerops_stats_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p, _i64, _i32, _p]),
     'kerops_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _p]),
