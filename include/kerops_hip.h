@@ -15,16 +15,23 @@
  *  - Every pointer is a device pointer, 16-byte aligned.  C is a power of two.
  *  - The caller owns every buffer, including the workspace whose size the
  *    matching *_workspace_bytes function returns.  The library allocates nothing
- *    and keeps no device state; workspaces need not be zeroed.
+ *    and keeps no device state (the one exception is the fixed array behind
+ *    kerops_dwconv_wgrad_noalloc_f16); workspaces need not be zeroed.  A workspace
+ *    query with blocks = 0 returns a size that covers every built-in launch shape.
  *  - All work is enqueued on `stream` (a hipStream_t, NULL = default stream); no
  *    entry point synchronises with the host.
  *  - Return value: KEROPS_OK or a negative KEROPS_E_* code; the text of the last
  *    failure on the calling thread is available from kerops_last_error_string().
  *    Nothing throws.
- *  - Trailing `tile_*`, `h_chunk`, `lane_channels` and `blocks` arguments are
- *    launch-shape knobs (patch extents along W and D, rows of H one workgroup
- *    marches over, channels one lane owns, workgroup count); 0 selects the built-in
- *    choice for gfx950, an unbuilt combination returns KEROPS_E_BADARG.
+ *  - Trailing `tile_*`, `h_chunk`, `lane_channels`, `blocks`, `waves` and `segment`
+ *    arguments are launch-shape knobs (patch extents along W and D, rows of H one
+ *    workgroup marches over, channels one lane owns; for the flat stream kernels the
+ *    workgroup count, the wavefronts per workgroup (4, 8 or 16) and the walk: segment
+ *    1 = a workgroup's 16-byte chunks are interleaved with the other workgroups',
+ *    4 or 8 = every step of a workgroup covers one contiguous run of that many chunks
+ *    per thread; the pooling kernels count output chunks and take 1 or 2);
+ *    0 selects the built-in choice for gfx950, an unbuilt combination
+ *    returns KEROPS_E_BADARG.
  *    For kerops_dwconv_fwd_f16 and kerops_dwconv_wgrad_f16 with the matrix-core
  *    kernels, h_chunk > 0 cuts H into uniform chunks of that many rows, one per
  *    workgroup; h_chunk = 0 is the balanced split: as many workgroups as the GPU
@@ -127,32 +134,34 @@ int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* wt, void* dx
  * Two-pass and deterministic instead of float atomics. */
 int64_t kerops_stats_workspace_bytes(int64_t M, int32_t C, int32_t blocks);
 int kerops_stats_f16(const void* x, float* mean, float* sqmean, int64_t M, int32_t C, void* workspace,
-                     int64_t workspace_bytes, int32_t blocks, void* stream);
+                     int64_t workspace_bytes, int32_t blocks, int32_t waves, int32_t segment, void* stream);
 
 /* dx = 2*x*sqmean_grad[c]/M + mean_grad[c]/M, fp16.
  * Replaces `_Stats_cl3d_backward_impl[(grid,)](...)`: kerops/ops/stats.py:52-63
  * (kernel kerops/kernels/stats.py:26-51). */
 int kerops_stats_bwd_f16(const void* x, const float* mean_grad, const float* sqmean_grad, void* dx, int64_t M,
-                         int32_t C, int32_t blocks, void* stream);
+                         int32_t C, int32_t blocks, int32_t waves, int32_t segment, void* stream);
 
 /* z = fp16(x + y) and the per-channel mean / mean of squares of z.
  * Replaces `_AddStats_cl3d_impl[(grid,)](...)`: kerops/ops/addition.py:35-48
  * (kernel kerops/kernels/addition.py:6-37).  z may alias x (the inplace mode).
  * Workspace as for kerops_stats_f16. */
 int kerops_add_stats_f16(const void* x, const void* y, void* z, float* mean, float* sqmean, int64_t M, int32_t C,
-                         void* workspace, int64_t workspace_bytes, int32_t blocks, void* stream);
+                         void* workspace, int64_t workspace_bytes, int32_t blocks, int32_t waves, int32_t segment,
+                         void* stream);
 
 /* out = fp16(add_grad + 2*add_result*sqmean_grad[c]/M + mean_grad[c]/M).
  * Replaces `_AddStats_cl3d_backward_impl[(grid,)](...)`: kerops/ops/addition.py:75-88
  * (kernel kerops/kernels/addition.py:41-75). */
 int kerops_add_stats_bwd_f16(const void* add_grad, const float* mean_grad, const float* sqmean_grad,
-                             const void* add_result, void* out, int64_t M, int32_t C, int32_t blocks, void* stream);
+                             const void* add_result, void* out, int64_t M, int32_t C, int32_t blocks, int32_t waves,
+                             int32_t segment, void* stream);
 
 /* y = fp16(max(float(x) * wv[c] + bv[c], 0)); wv, bv are fp32 [C].
  * Replaces `_ApplyBNReLU_cl3d_impl[(grid,)](...)`: kerops/ops/bnrelu.py:30-41
  * (kernel kerops/kernels/bnrelu.py:6-31). */
 int kerops_bnrelu_fwd_f16(const void* x, const float* wv, const float* bv, void* y, int64_t M, int32_t C,
-                          int32_t blocks, void* stream);
+                          int32_t blocks, int32_t waves, int32_t segment, void* stream);
 
 /* keep = (x*wv[c] > -bv[c]); g' = g*keep; dx = fp16(wv[c]*g'); dW[c] = sum x*g';
  * dB[c] = sum g' (fp32, deterministic two-pass).
@@ -161,7 +170,7 @@ int kerops_bnrelu_fwd_f16(const void* x, const float* wv, const float* bv, void*
  * (kernel kerops/kernels/bnrelu.py:35-71).  Workspace as for kerops_stats_f16. */
 int kerops_bnrelu_bwd_f16(const void* x, const float* wv, const float* bv, const void* g, void* dx, float* dW,
                           float* dB, int64_t M, int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks,
-                          void* stream);
+                          int32_t waves, int32_t segment, void* stream);
 
 /* 2x2x2 stride-2 average pool with ceil_mode (edge windows divide by the number
  * of existing voxels), y dense [N][ceil(H/2)][ceil(W/2)][ceil(D/2)][C] fp16, plus
@@ -171,9 +180,9 @@ int kerops_bnrelu_bwd_f16(const void* x, const float* wv, const float* bv, const
  * (kernel kerops/kernels/avgpool.py:6-93). */
 int64_t kerops_avgpool_ceil_stats_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
                                                   int32_t blocks);
-int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H, int32_t W,
-                                  int32_t D, int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks,
-                                  void* stream);
+int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H,
+                                  int32_t W, int32_t D, int32_t C, void* workspace, int64_t workspace_bytes,
+                                  int32_t blocks, int32_t waves, int32_t segment, void* stream);
 
 /* ApplyBNReLU and AvgPoolCeilStats in one pass (no single reference counterpart; the reference composes
  * the two ops, tests/ops/test_bn_relu.py:26-30 and tests/ops/test_avgpool.py): every existing voxel is
@@ -182,7 +191,8 @@ int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sq
  * kerops_avgpool_ceil_stats_f16. */
 int kerops_bnrelu_avgpool_ceil_stats_f16(const void* x, const float* weight, const float* bias, void* y, float* mean,
                                          float* sqmean, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
-                                         void* workspace, int64_t workspace_bytes, int32_t blocks, void* stream);
+                                         void* workspace, int64_t workspace_bytes, int32_t blocks, int32_t waves,
+                                         int32_t segment, void* stream);
 
 /* dx[every existing voxel of a window] =
  *   fp16((inpgrad + meangrad[c]/Mo + 2*output*sqmeangrad[c]/Mo) / count),
@@ -192,7 +202,7 @@ int kerops_bnrelu_avgpool_ceil_stats_f16(const void* x, const float* weight, con
  * kerops/ops/avgpool.py:93-122 (kernel kerops/kernels/avgpool.py:97-185). */
 int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad, const float* sqmeangrad,
                                       const void* output, void* dx, int32_t N, int32_t H, int32_t W, int32_t D,
-                                      int32_t C, int32_t blocks, void* stream);
+                                      int32_t C, int32_t blocks, int32_t waves, int32_t segment, void* stream);
 
 /* u8 = (uint8)(((clip(float(x), -window, window) + window) / (2*window)) * 255),
  * each step one IEEE fp32 operation, conversion by truncation.  dtype is the
@@ -201,14 +211,14 @@ int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad
  * Replaces `_QuantUint8Window_impl[(numblocks,)](...)`:
  * kerops/ops/quantization.py:19 (kernel kerops/kernels/quantization.py:6-27). */
 int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int64_t numel, float window, int32_t blocks,
-                           void* stream);
+                           int32_t waves, int32_t segment, void* stream);
 
 /* out = float(u8) * (2*window/255) - window (scale formed once in fp32; one
  * multiply, one subtract), stored as dtype (fp16, fp32 or bf16; one RNE rounding).
  * Replaces `_DequantUint8Window_impl[(numblocks,)](...)`:
  * kerops/ops/quantization.py:34 (kernel kerops/kernels/quantization.py:31-49). */
 int kerops_dequant_u8_window(const void* q, void* out, int32_t dtype, int64_t numel, float window, int32_t blocks,
-                             void* stream);
+                             int32_t waves, int32_t segment, void* stream);
 
 /* max |y| over numel fp16 values, written to *absmax (device fp32).  No reference
  * counterpart: first pass of the symmetric int8 quantiser of the fused-block
@@ -220,7 +230,8 @@ int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, void* workspa
 /* q = clamp(rint_half_even(float(y) / (absmax/127)), -127, 127) as int8, with
  * absmax read from device memory; absmax == 0 gives q = 0.  No reference
  * counterpart: second pass of the symmetric int8 quantiser. */
-int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t numel, int32_t blocks, void* stream);
+int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t numel, int32_t blocks,
+                            int32_t waves, int32_t segment, void* stream);
 
 /* Pointwise (1x1x1) channel mixing on MFMA:
  *   out[v, co] = fp16(sum_ci act(x[v, ci]) * Wm[ci, co]) (+ add[v, co], fp16 add)

@@ -38,23 +38,25 @@ SIGNATURES = {
                                                _i32, _p]),
     'kerops_dwconv_wgrad_noalloc_f16': (ctypes.c_int, [_p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_stats_workspace_bytes': (_i64, [_i64, _i32, _i32]),
-    'kerops_stats_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p, _i64, _i32, _p]),
-    'kerops_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _p]),
-    'kerops_add_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i32, _p, _i64, _i32, _p]),
-    'kerops_add_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
-    'kerops_bnrelu_fwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _p]),
-    'kerops_bnrelu_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _i64, _i32, _p, _i64, _i32, _p]),
+    'kerops_stats_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p, _i64, _i32, _i32, _i32, _p]),
+    'kerops_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _p]),
+    'kerops_add_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i32, _p, _i64, _i32, _i32, _i32, _p]),
+    'kerops_add_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _p]),
+    'kerops_bnrelu_fwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _p]),
+    'kerops_bnrelu_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _i64, _i32, _p, _i64, _i32, _i32, _i32,
+                                             _p]),
     'kerops_avgpool_ceil_stats_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_avgpool_ceil_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _i64, _i32,
-                                                     _p]),
-    'kerops_bnrelu_avgpool_ceil_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _i64, _i32,
-                                                     _p]),
-    'kerops_avgpool_ceil_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _i32, _p]),
-    'kerops_quant_u8_window': (ctypes.c_int, [_p, _i32, _p, _i64, _f32, _i32, _p]),
-    'kerops_dequant_u8_window': (ctypes.c_int, [_p, _p, _i32, _i64, _f32, _i32, _p]),
+                                                     _i32, _i32, _p]),
+    'kerops_bnrelu_avgpool_ceil_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p,
+                                                            _i64, _i32, _i32, _i32, _p]),
+    'kerops_avgpool_ceil_stats_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _i32, _i32,
+                                                         _i32, _p]),
+    'kerops_quant_u8_window': (ctypes.c_int, [_p, _i32, _p, _i64, _f32, _i32, _i32, _i32, _p]),
+    'kerops_dequant_u8_window': (ctypes.c_int, [_p, _p, _i32, _i64, _f32, _i32, _i32, _i32, _p]),
     'kerops_absmax_workspace_bytes': (_i64, [_i32]),
     'kerops_absmax_f16': (ctypes.c_int, [_p, _p, _i64, _p, _i64, _i32, _p]),
-    'kerops_quant_i8_sym_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p]),
+    'kerops_quant_i8_sym_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _i32, _i32, _p]),
     'kerops_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p]),
     'kerops_bnrelu_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
     'kerops_lin_brelu_lin_add_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _p]),

@@ -19,23 +19,24 @@ struct PoolDims {
 // BNRELU: every voxel that exists is first mapped to fp16(max(x * bw[c] + bb[c], 0)), exactly what
 // bnrelu_fwd_kernel would have stored, so the fused op equals ApplyBNReLU followed by the pool bit for bit
 // while the full-size intermediate is neither written nor read.
-template <int V, bool BNRELU>
-__global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_t* __restrict__ x,
-                                                                     const float* __restrict__ bw,
-                                                                     const float* __restrict__ bb,
-                                                                     half_t* __restrict__ y, float* __restrict__ ws,
-                                                                     const PoolDims p, int64_t nchunks)
+template <int V, int U, bool BNRELU>
+__global__ __launch_bounds__(kStreamMaxThreads) void avgpool_fwd_kernel(const half_t* __restrict__ x,
+                                                                        const float* __restrict__ bw,
+                                                                        const float* __restrict__ bb,
+                                                                        half_t* __restrict__ y, float* __restrict__ ws,
+                                                                        const PoolDims p, int64_t nchunks,
+                                                                        int segments)
 {
     typedef typename HVec<V>::type hv;
-    __shared__ float red[kStreamWaves * 2 * 64 * V];
-    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
+    __shared__ float red[4 * 2 * 64 * V];
+    const ChunkWalk<U> wk(nchunks, segments != 0);
     float acc[2][V];
 #pragma unroll
     for (int j = 0; j < V; ++j) acc[0][j] = acc[1][j] = 0.0f;
-    // the grid stride is a multiple of the number of channel groups: a thread keeps its channel group
+    // every stride of the walk is a multiple of the number of channel groups: a thread keeps its channel group
     float cw[V], cb[V];
     if (BNRELU) {
-        const int cg0 = (int)(((int64_t)blockIdx.x * kStreamThreads + threadIdx.x) % p.CG);
+        const int cg0 = (int)(wk.first % p.CG);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
             cw[j] = bw[cg0 * V + j];
@@ -44,7 +45,12 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
     }
     const int64_t sD = p.CG, sW = (int64_t)p.D * p.CG, sH = (int64_t)p.W * sW, sN = (int64_t)p.H * sH;  // in chunks
 
-    for (int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x; i < nchunks; i += T) {
+    struct Window {
+        hv v[2][2][2];
+        bool h1, w1, d1;
+    };
+    // all eight loads of a window are issued before the first value is touched
+    auto load_window = [&](int64_t i, Window& wn) {
         int64_t r = i;
         const int cg = (int)(r % p.CG);
         r /= p.CG;
@@ -54,39 +60,42 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
         r /= p.Wo;
         const int hO = (int)(r % p.Ho);
         const int n = (int)(r / p.Ho);
-        const bool h1 = 2 * hO + 1 < p.H, w1 = 2 * wO + 1 < p.W, d1 = 2 * dO + 1 < p.D;
+        wn.h1 = 2 * hO + 1 < p.H;
+        wn.w1 = 2 * wO + 1 < p.W;
+        wn.d1 = 2 * dO + 1 < p.D;
         const int64_t base = n * sN + (2 * hO) * sH + (2 * wO) * sW + (2 * dO) * sD + cg;
-        hv v[2][2][2];
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
+                    const bool ok = (a == 0 || wn.h1) && (b == 0 || wn.w1) && (e == 0 || wn.d1);
                     hv t;
 #pragma unroll
                     for (int j = 0; j < V; ++j) t[j] = (half_t)0;
                     if (ok) t = ld_stream<V>(x, base + a * sH + b * sW + e * sD);
-                    v[a][b][e] = t;
+                    wn.v[a][b][e] = t;
                 }
+    };
+    auto finish_window = [&](int64_t i, Window& wn) {
         if (BNRELU) {
-            // a second pass, so that all eight loads are in flight before the first value is touched
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
                 for (int b = 0; b < 2; ++b)
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
-                        const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
+                        const bool ok = (a == 0 || wn.h1) && (b == 0 || wn.w1) && (e == 0 || wn.d1);
 #pragma unroll
                         for (int j = 0; j < V; ++j) {
-                            const half_t r = (half_t)fmaxf(__builtin_fmaf((float)v[a][b][e][j], cw[j], cb[j]), 0.0f);
-                            v[a][b][e][j] = ok ? r : (half_t)0;
+                            const half_t r =
+                                (half_t)fmaxf(__builtin_fmaf((float)wn.v[a][b][e][j], cw[j], cb[j]), 0.0f);
+                            wn.v[a][b][e][j] = ok ? r : (half_t)0;
                         }
                     }
         }
-        const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
+        const float cnt = (float)((wn.h1 ? 2 : 1) * (wn.w1 ? 2 : 1) * (wn.d1 ? 2 : 1));
         hv o;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -94,37 +103,49 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_fwd_kernel(const half_
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
-                for (int b = 0; b < 2; ++b) s += (float)v[a][b][0][j] + (float)v[a][b][1][j];
+                for (int b = 0; b < 2; ++b) s += (float)wn.v[a][b][0][j] + (float)wn.v[a][b][1][j];
             const float m = __fdiv_rn(s, cnt);
             o[j] = (half_t)m;
             acc[0][j] += m;
             acc[1][j] = __builtin_fmaf(m, m, acc[1][j]);
         }
         st_stream<V>(y, i, o);
+    };
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
+        Window wn[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_window(i + u * wk.su, wn[u]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) finish_window(i + u * wk.su, wn[u]);
     }
-    block_channel_partials<2, V>(acc, p.CG, red, ws + (int64_t)blockIdx.x * 2 * p.CG * V);
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T) {
+        Window wn;
+        load_window(i, wn);
+        finish_window(i, wn);
+    }
+    block_channel_partials_any<2, V>(acc, p.CG, red, ws + (int64_t)blockIdx.x * 2 * p.CG * V);
 }
 
-template <int V>
-__global__ __launch_bounds__(kStreamThreads) void avgpool_bwd_kernel(const half_t* __restrict__ inpgrad,
-                                                                     const float* __restrict__ meangrad,
-                                                                     const float* __restrict__ sqmeangrad,
-                                                                     const half_t* __restrict__ output,
-                                                                     half_t* __restrict__ dx, const PoolDims p,
-                                                                     int64_t nchunks, float fMo)
+template <int V, int U>
+__global__ __launch_bounds__(kStreamMaxThreads) void avgpool_bwd_kernel(const half_t* __restrict__ inpgrad,
+                                                                        const float* __restrict__ meangrad,
+                                                                        const float* __restrict__ sqmeangrad,
+                                                                        const half_t* __restrict__ output,
+                                                                        half_t* __restrict__ dx, const PoolDims p,
+                                                                        int64_t nchunks, float fMo, int segments)
 {
     typedef typename HVec<V>::type hv;
-    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
+    const ChunkWalk<U> wk(nchunks, segments != 0);
     const int64_t sD = p.CG, sW = (int64_t)p.D * p.CG, sH = (int64_t)p.W * sW, sN = (int64_t)p.H * sH;
-    int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    const int cg0 = (int)(i % p.CG);
+    const int cg0 = (int)(wk.first % p.CG);
     float mg[V], sg[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
         mg[j] = __fdiv_rn(meangrad[cg0 * V + j], fMo);
         sg[j] = sqmeangrad[cg0 * V + j];
     }
-    for (; i < nchunks; i += T) {
+    auto one = [&](int64_t i, const hv& g, const hv& o) {
         int64_t r = i / p.CG;
         const int dO = (int)(r % p.Do);
         r /= p.Do;
@@ -134,7 +155,6 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_bwd_kernel(const half_
         const int n = (int)(r / p.Ho);
         const bool h1 = 2 * hO + 1 < p.H, w1 = 2 * wO + 1 < p.W, d1 = 2 * dO + 1 < p.D;
         const float cnt = (float)((h1 ? 2 : 1) * (w1 ? 2 : 1) * (d1 ? 2 : 1));
-        const hv g = ld_stream<V>(inpgrad, i), o = ld_stream<V>(output, i);
         hv res;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -152,11 +172,34 @@ __global__ __launch_bounds__(kStreamThreads) void avgpool_bwd_kernel(const half_
                     const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
                     if (ok) st_stream<V>(dx, base + a * sH + b * sW + e * sD, res);
                 }
+    };
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
+        hv g[U], o[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            g[u] = ld_stream<V>(inpgrad, i + u * wk.su);
+            o[u] = ld_stream<V>(output, i + u * wk.su);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) one(i + u * wk.su, g[u], o[u]);
     }
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T) one(i, ld_stream<V>(inpgrad, i), ld_stream<V>(output, i));
 }
 
-static int pool_plan(const char* op, int N, int H, int W, int D, int C, int* blocks, PoolDims* p, int64_t* nchunks,
-                     int64_t* need)
+// Launch shape (blocks, waves, segment) as for the flat stream kernels; segment counts output chunks per thread and
+// step: 1 = interleaved (one window per thread in flight), 2 = contiguous runs of two chunks per thread (two
+// windows, 16 loads, in flight).  Built-in choices measured at (1,64,350,350,128).
+struct PoolDefault {
+    int blocks, waves, segment;
+};
+constexpr PoolDefault kDefPoolFwd{256, 4, 2};
+constexpr PoolDefault kDefPoolFwdBnRelu{512, 4, 1};
+constexpr PoolDefault kDefPoolBwd{256, 4, 2};
+constexpr int kMaxDefaultBlocks = 4096;  // workspace queries with blocks = 0 size for this many partials
+
+static int pool_plan(const char* op, const PoolDefault& def, int N, int H, int W, int D, int C, int blocks, int waves,
+                     int segment, PoolDims* p, int64_t* nchunks, StreamShape* sh)
 {
     if (N <= 0 || H <= 0 || W <= 0 || D <= 0 || C <= 0 || !is_pow2(C)) {
         set_error("%s: extents must be positive and C a power of two", op);
@@ -170,6 +213,20 @@ static int pool_plan(const char* op, int N, int H, int W, int D, int C, int* blo
         set_error("%s: tensor too large", op);
         return KEROPS_E_BADARG;
     }
+    if (waves == 0) waves = def.waves;
+    if (segment == 0) segment = def.segment;
+    if (!(waves == 4 || waves == 8 || waves == 16)) {
+        set_error("%s: waves must be 4, 8 or 16 wavefronts per workgroup (got %d)", op, waves);
+        return KEROPS_E_BADARG;
+    }
+    if (!(segment == 1 || segment == 2)) {
+        set_error("%s: segment must be 1 (interleaved) or 2 (got %d)", op, segment);
+        return KEROPS_E_BADARG;
+    }
+    if (blocks > 65536) {
+        set_error("%s: blocks must be <= 65536", op);
+        return KEROPS_E_BADARG;
+    }
     const int V = C >= 8 ? 8 : C;
     p->N = N;
     p->H = H;
@@ -181,12 +238,10 @@ static int pool_plan(const char* op, int N, int H, int W, int D, int C, int* blo
     p->C = C;
     p->CG = C / V;
     *nchunks = (int64_t)N * p->Ho * p->Wo * p->Do * p->CG;
-    if (*blocks <= 0) *blocks = stream_blocks_default(*nchunks, 512);
-    if (*blocks > 65536) {
-        set_error("%s: blocks must be <= 65536", op);
-        return KEROPS_E_BADARG;
-    }
-    *need = (int64_t)(*blocks) * 2 * C * (int64_t)sizeof(float);
+    sh->threads = waves * kWave;
+    sh->segment = segment;
+    if (blocks <= 0) blocks = def.blocks;
+    sh->blocks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(*nchunks, (int64_t)sh->threads * segment), blocks));
     return KEROPS_OK;
 }
 
@@ -198,75 +253,87 @@ extern "C" int64_t kerops_avgpool_ceil_stats_workspace_bytes(int32_t N, int32_t 
                                                              int32_t blocks)
 {
     PoolDims p;
-    int64_t nchunks = 0, need = 0;
-    int rc = pool_plan("avgpool_ceil_stats", N, H, W, D, C, &blocks, &p, &nchunks, &need);
-    return rc != KEROPS_OK ? rc : need;
+    int64_t nchunks = 0;
+    StreamShape sh;
+    int rc = pool_plan("avgpool_ceil_stats", kDefPoolFwd, N, H, W, D, C, blocks, 0, 0, &p, &nchunks, &sh);
+    if (rc != KEROPS_OK) return rc;
+    if (blocks <= 0) blocks = kMaxDefaultBlocks;
+    return (int64_t)blocks * 2 * C * (int64_t)sizeof(float);
 }
 
 static int pool_fwd_run(const char* op, const void* x, const float* bw, const float* bb, void* y, float* mean,
                         float* sqmean, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, void* workspace,
-                        int64_t workspace_bytes, int32_t blocks, void* stream)
+                        int64_t workspace_bytes, int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
     PoolDims p;
-    int64_t nchunks = 0, need = 0;
-    int rc = pool_plan(op, N, H, W, D, C, &blocks, &p, &nchunks, &need);
+    int64_t nchunks = 0;
+    StreamShape sh;
+    int rc = pool_plan(op, bw ? kDefPoolFwdBnRelu : kDefPoolFwd, N, H, W, D, C, blocks, waves, segment, &p, &nchunks,
+                       &sh);
     if (rc != KEROPS_OK) return rc;
     if (!x || !y || !mean || !sqmean || !aligned16(x) || !aligned16(y)) {
         set_error("%s: null or misaligned pointer", op);
         return KEROPS_E_BADARG;
     }
+    const int64_t need = (int64_t)sh.blocks * 2 * C * (int64_t)sizeof(float);
     if (!workspace || !aligned16(workspace) || workspace_bytes < need) {
         set_error("%s: workspace of %lld bytes required, %lld given", op, (long long)need, (long long)workspace_bytes);
         return KEROPS_E_WORKSPACE;
     }
     hipStream_t s = (hipStream_t)stream;
     float* ws = (float*)workspace;
+    const int seg = sh.segment != 1;
+#define KEROPS_POOL_GO(Uv, B)                                                                                      \
+    KEROPS_DISPATCH_V(C, {                                                                                         \
+        hipLaunchKernelGGL((avgpool_fwd_kernel<V, Uv, B>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const half_t*)x, \
+                           bw, bb, (half_t*)y, ws, p, nchunks, seg);                                               \
+    })
     if (bw) {
-        KEROPS_DISPATCH_V(C, {
-            hipLaunchKernelGGL((avgpool_fwd_kernel<V, true>), dim3(blocks), dim3(kStreamThreads), 0, s,
-                               (const half_t*)x, bw, bb, (half_t*)y, ws, p, nchunks);
-        });
+        if (sh.segment == 2) KEROPS_POOL_GO(2, true);
+        else KEROPS_POOL_GO(1, true);
     } else {
-        KEROPS_DISPATCH_V(C, {
-            hipLaunchKernelGGL((avgpool_fwd_kernel<V, false>), dim3(blocks), dim3(kStreamThreads), 0, s,
-                               (const half_t*)x, bw, bb, (half_t*)y, ws, p, nchunks);
-        });
+        if (sh.segment == 2) KEROPS_POOL_GO(2, false);
+        else KEROPS_POOL_GO(1, false);
     }
+#undef KEROPS_POOL_GO
     rc = check_launch(op);
     if (rc != KEROPS_OK) return rc;
     const double Mo = (double)N * p.Ho * p.Wo * p.Do;
-    launch_reduce_rows(ws, blocks, 2 * C, mean, sqmean, C, 1.0 / Mo, s);
+    launch_reduce_rows(ws, sh.blocks, 2 * C, mean, sqmean, C, 1.0 / Mo, s);
     return check_launch(op);
 }
 
 extern "C" int kerops_avgpool_ceil_stats_f16(const void* x, void* y, float* mean, float* sqmean, int32_t N, int32_t H,
                                              int32_t W, int32_t D, int32_t C, void* workspace,
-                                             int64_t workspace_bytes, int32_t blocks, void* stream)
+                                             int64_t workspace_bytes, int32_t blocks, int32_t waves, int32_t segment,
+                                             void* stream)
 {
     return pool_fwd_run("avgpool_ceil_stats", x, nullptr, nullptr, y, mean, sqmean, N, H, W, D, C, workspace,
-                        workspace_bytes, blocks, stream);
+                        workspace_bytes, blocks, waves, segment, stream);
 }
 
 extern "C" int kerops_bnrelu_avgpool_ceil_stats_f16(const void* x, const float* weight, const float* bias, void* y,
                                                     float* mean, float* sqmean, int32_t N, int32_t H, int32_t W,
                                                     int32_t D, int32_t C, void* workspace, int64_t workspace_bytes,
-                                                    int32_t blocks, void* stream)
+                                                    int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
     if (!weight || !bias) {
         set_error("bnrelu_avgpool_ceil_stats: null weight or bias");
         return KEROPS_E_BADARG;
     }
     return pool_fwd_run("bnrelu_avgpool_ceil_stats", x, weight, bias, y, mean, sqmean, N, H, W, D, C, workspace,
-                        workspace_bytes, blocks, stream);
+                        workspace_bytes, blocks, waves, segment, stream);
 }
 
 extern "C" int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const float* meangrad, const float* sqmeangrad,
                                                  const void* output, void* dx, int32_t N, int32_t H, int32_t W,
-                                                 int32_t D, int32_t C, int32_t blocks, void* stream)
+                                                 int32_t D, int32_t C, int32_t blocks, int32_t waves, int32_t segment,
+                                                 void* stream)
 {
     PoolDims p;
-    int64_t nchunks = 0, need = 0;
-    int rc = pool_plan("avgpool_ceil_stats_bwd", N, H, W, D, C, &blocks, &p, &nchunks, &need);
+    int64_t nchunks = 0;
+    StreamShape sh;
+    int rc = pool_plan("avgpool_ceil_stats_bwd", kDefPoolBwd, N, H, W, D, C, blocks, waves, segment, &p, &nchunks, &sh);
     if (rc != KEROPS_OK) return rc;
     if (!inpgrad || !meangrad || !sqmeangrad || !output || !dx || !aligned16(inpgrad) || !aligned16(output) ||
         !aligned16(dx)) {
@@ -274,10 +341,15 @@ extern "C" int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const floa
         return KEROPS_E_BADARG;
     }
     const float fMo = (float)((int64_t)N * p.Ho * p.Wo * p.Do);
-    KEROPS_DISPATCH_V(C, {
-        hipLaunchKernelGGL((avgpool_bwd_kernel<V>), dim3(blocks), dim3(kStreamThreads), 0, (hipStream_t)stream,
-                           (const half_t*)inpgrad, meangrad, sqmeangrad, (const half_t*)output, (half_t*)dx, p,
-                           nchunks, fMo);
-    });
+    const int seg = sh.segment != 1;
+#define KEROPS_POOLB_GO(Uv)                                                                                          \
+    KEROPS_DISPATCH_V(C, {                                                                                           \
+        hipLaunchKernelGGL((avgpool_bwd_kernel<V, Uv>), dim3(sh.blocks), dim3(sh.threads), 0, (hipStream_t)stream,   \
+                           (const half_t*)inpgrad, meangrad, sqmeangrad, (const half_t*)output, (half_t*)dx, p,      \
+                           nchunks, fMo, seg);                                                                       \
+    })
+    if (sh.segment == 2) KEROPS_POOLB_GO(2);
+    else KEROPS_POOLB_GO(1);
+#undef KEROPS_POOLB_GO
     return check_launch("avgpool_ceil_stats_bwd");
 }

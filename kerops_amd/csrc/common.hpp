@@ -393,6 +393,79 @@ __device__ __forceinline__ void block_channel_partials(float (&acc)[NACC][V], in
     }
 }
 
+// ---- launch shape of the flat stream kernels ------------------------------------------------------------
+// A stream kernel walks its 16-byte chunks in steps of U chunks per thread (all U loads of a stream are issued
+// before the first value is used).  With T = workgroups * threads, step k of a thread covers
+//   interleaved (segment = 1): chunks k*U*T + u*T + b*threads + t          (a workgroup's chunks are T apart)
+//   segments    (segment = U): chunks k*U*T + b*U*threads + u*threads + t  (a workgroup reads and writes one
+//                                                                           contiguous run of U*threads chunks)
+// for u < U; what is left after the last full step (< U*T chunks) is walked one chunk at a time.  Measured on
+// MI355X with a plain copy of 2 GB: interleaved 256-thread workgroups reach 5.4-5.8 TB/s depending on the
+// workgroup count (power-of-two counts such as 1024 fall to 4.4 TB/s: all accesses in flight then sit a
+// power-of-two stride apart), 1024-thread workgroups on 128 KiB segments (U = 8) reach 6.0-6.3 TB/s whatever
+// the count.  Both T and threads are multiples of the number of channel groups, so a thread keeps its group.
+struct StreamShape {
+    int blocks, threads, segment;  // segment: 1 = interleaved (U = 4), 4 or 8 = contiguous segments with that U
+    int unroll() const { return segment == 8 ? 8 : 4; }
+};
+template <int U>
+struct ChunkWalk {
+    int64_t T, step, su, first, nfull, tail;
+    __device__ __forceinline__ ChunkWalk(int64_t nchunks, bool segments)
+    {
+        const int64_t nthr = blockDim.x;
+        T = (int64_t)gridDim.x * nthr;
+        step = U * T;
+        nfull = nchunks / step;
+        su = segments ? nthr : T;
+        first = (segments ? (int64_t)blockIdx.x * U * nthr : (int64_t)blockIdx.x * nthr) + threadIdx.x;
+        tail = nfull * step + (int64_t)blockIdx.x * nthr + threadIdx.x;
+    }
+};
+constexpr int kStreamMaxThreads = 1024;
+
+// block_channel_partials for any workgroup size up to 1024 threads: the wavefronts hand their sums over in
+// rounds of four through the same 4-slot LDS buffer; thread o keeps the running sums of the outputs
+// o, o + threads, ... (at most NACC*512 / 256 = 2*NACC of them) and adds the rounds in a fixed order.
+template <int NACC, int V>
+__device__ __forceinline__ void block_channel_partials_any(float (&acc)[NACC][V], int CG, float* red, float* dst)
+{
+    const int t = threadIdx.x, lane = t % kWave, wave = t / kWave, nthr = blockDim.x, nwaves = nthr / kWave;
+    const int cols = CG * V, nout = NACC * cols;
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            float v = acc[a][j];
+            for (int off = 32; off >= CG; off >>= 1) v += __shfl_xor(v, off, 64);
+            acc[a][j] = v;
+        }
+    constexpr int kMine = 2 * NACC;
+    float run[kMine];
+#pragma unroll
+    for (int m = 0; m < kMine; ++m) run[m] = 0.0f;
+    for (int r = 0; r < nwaves; r += 4) {
+        if (wave >= r && wave < r + 4 && lane < CG) {
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+#pragma unroll
+                for (int j = 0; j < V; ++j) red[((wave - r) * NACC + a) * cols + lane * V + j] = acc[a][j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < kMine; ++m) {
+            const int o = t + m * nthr;
+            if (o < nout) run[m] += (red[o] + red[nout + o]) + (red[2 * nout + o] + red[3 * nout + o]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int m = 0; m < kMine; ++m) {
+        const int o = t + m * nthr;
+        if (o < nout) dst[o] = run[m];
+    }
+}
+
 // out[j] = scale * sum_r ws[r*ncols + j] for j < ncols, summed in fp64 in a fixed order;
 // columns [0, split) go to out0, the rest to out1.  (Kernel lives in core.hip.)
 void launch_reduce_rows(const float* ws, int nrows, int ncols, float* out0, float* out1, int split, double scale,

@@ -2,12 +2,13 @@
 // statistics, BN-ReLU forward/backward, residual add with statistics, the uint8 window
 // quantiser pair and the symmetric int8 quantiser.
 //
-// All of them are HBM-bound.  Each is a persistent grid-stride loop of 256-thread
-// workgroups: a thread moves V = min(8, C) consecutive channels per access (16 bytes for
-// C >= 8), consecutive lanes take consecutive chunks, and the grid stride is a multiple
-// of the number of channel groups, so a thread keeps one channel group for its whole
-// life: per-channel parameters sit in registers and per-channel sums are plain
-// per-thread fp32 accumulators.  Reductions finish with wavefront shuffles, one LDS
+// All of them are HBM-bound.  Each is a persistent loop of 256- or 1024-thread workgroups
+// over steps of U chunks per thread (ChunkWalk in common.hpp: interleaved, or one contiguous
+// segment per workgroup and step): a thread moves V = min(8, C) consecutive channels per
+// access (16 bytes for C >= 8), consecutive lanes take consecutive chunks, and every stride
+// of the walk is a multiple of the number of channel groups, so a thread keeps one channel
+// group for its whole life: per-channel parameters sit in registers and per-channel sums
+// are plain per-thread fp32 accumulators.  Reductions finish with wavefront shuffles, one LDS
 // hop per workgroup, a [workgroups][..] partial buffer and a small fp64 second pass:
 // no float atomics, identical bits on every run.
 #include "common.hpp"
@@ -15,13 +16,14 @@
 namespace kerops {
 
 // ------------------------------------------------------------------ Stats
-template <int V, bool ADD>
-__global__ __launch_bounds__(kStreamThreads) void stats_kernel(const half_t* x, const half_t* y, half_t* z,
-                                                               float* __restrict__ ws, int64_t nchunks, int CG)
+template <int V, int U, bool ADD>
+__global__ __launch_bounds__(kStreamMaxThreads) void stats_kernel(const half_t* x, const half_t* y, half_t* z,
+                                                                  float* __restrict__ ws, int64_t nchunks, int CG,
+                                                                  int segments)
 {
     typedef typename HVec<V>::type hv;
-    __shared__ float red[kStreamWaves * 2 * 64 * V];
-    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
+    __shared__ float red[4 * 2 * 64 * V];
+    const ChunkWalk<U> wk(nchunks, segments != 0);
     float acc[2][V];
 #pragma unroll
     for (int j = 0; j < V; ++j) acc[0][j] = acc[1][j] = 0.0f;
@@ -41,70 +43,49 @@ __global__ __launch_bounds__(kStreamThreads) void stats_kernel(const half_t* x, 
             acc[1][j] = __builtin_fmaf(f, f, acc[1][j]);
         }
     };
-    int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    for (; i + 3 * T < nchunks; i += 4 * T) {
-        if (!ADD) {
-            const hv v0 = ld_stream<V>(x, i), v1 = ld_stream<V>(x, i + T), v2 = ld_stream<V>(x, i + 2 * T),
-                     v3 = ld_stream<V>(x, i + 3 * T);
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
+        hv v[U], w[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v[u] = ld_stream<V>(x, i + u * wk.su);
+            w[u] = ADD ? ld_stream<V>(y, i + u * wk.su) : v[u];
+        }
+        if (ADD) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) v[u][j] = (half_t)((float)v[u][j] + (float)w[u][j]);  // fp16 sum, RNE
+                st_stream<V>(z, i + u * wk.su, v[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u += 4) {
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                const float f0 = (float)v0[j], f1 = (float)v1[j], f2 = (float)v2[j], f3 = (float)v3[j];
+                const float f0 = (float)v[u][j], f1 = (float)v[u + 1][j], f2 = (float)v[u + 2][j],
+                            f3 = (float)v[u + 3][j];
                 acc[0][j] += (f0 + f1) + (f2 + f3);
                 acc[1][j] += __builtin_fmaf(f0, f0, f1 * f1) + __builtin_fmaf(f2, f2, f3 * f3);
             }
-        } else {
-            body(i);
-            body(i + T);
-            body(i + 2 * T);
-            body(i + 3 * T);
         }
     }
-    for (; i < nchunks; i += T) body(i);
-    block_channel_partials<2, V>(acc, CG, red, ws + (int64_t)blockIdx.x * 2 * CG * V);
-}
-
-static int check_reduce_args(const char* op, int64_t M, int C, int* blocks, int64_t* need)
-{
-    if (M <= 0 || C <= 0 || !is_pow2(C)) {
-        set_error("%s: M must be positive and C a power of two (M=%lld C=%d)", op, (long long)M, C);
-        return KEROPS_E_BADARG;
-    }
-    if (C > kMaxReduceChannels) {
-        set_error("%s: per-channel reductions are built for C <= %d (got %d)", op, kMaxReduceChannels, C);
-        return KEROPS_E_UNSUPPORTED_C;
-    }
-    const int V = C >= 8 ? 8 : C;
-    if (*blocks <= 0) *blocks = stream_blocks_default(M * (C / V));
-    if (*blocks > 65536) {
-        set_error("%s: blocks must be <= 65536", op);
-        return KEROPS_E_BADARG;
-    }
-    *need = (int64_t)(*blocks) * 2 * C * (int64_t)sizeof(float);
-    return KEROPS_OK;
-}
-
-static int check_ws(const char* op, const void* ws, int64_t have, int64_t need)
-{
-    if (!ws || !aligned16(ws) || have < need) {
-        set_error("%s: workspace of %lld bytes required, %lld given", op, (long long)need, (long long)have);
-        return KEROPS_E_WORKSPACE;
-    }
-    return KEROPS_OK;
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T) body(i);
+    block_channel_partials_any<2, V>(acc, CG, red, ws + (int64_t)blockIdx.x * 2 * CG * V);
 }
 
 // ---------------------------------------------------------- stats backward
-template <int V, bool ADD>
-__global__ __launch_bounds__(kStreamThreads) void stats_bwd_kernel(const half_t* __restrict__ x,
-                                                                   const half_t* __restrict__ add_grad,
-                                                                   const float* __restrict__ mean_grad,
-                                                                   const float* __restrict__ sqmean_grad,
-                                                                   half_t* __restrict__ dx, int64_t nchunks, int CG,
-                                                                   float fm)
+template <int V, int U, bool ADD>
+__global__ __launch_bounds__(kStreamMaxThreads) void stats_bwd_kernel(const half_t* __restrict__ x,
+                                                                      const half_t* __restrict__ add_grad,
+                                                                      const float* __restrict__ mean_grad,
+                                                                      const float* __restrict__ sqmean_grad,
+                                                                      half_t* __restrict__ dx, int64_t nchunks, int CG,
+                                                                      float fm, int segments)
 {
     typedef typename HVec<V>::type hv;
-    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
-    int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    const int cg = (int)(i % CG);
+    const ChunkWalk<U> wk(nchunks, segments != 0);
+    const int cg = (int)(wk.first % CG);
     float sg[V], mg[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
@@ -120,34 +101,34 @@ __global__ __launch_bounds__(kStreamThreads) void stats_bwd_kernel(const half_t*
         }
         return o;
     };
-    constexpr int U = 4;  // chunks in flight per lane and input stream
-    for (; i + (U - 1) * T < nchunks; i += U * T) {
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
         hv v[U], g[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            v[u] = ld_stream<V>(x, i + u * T);
-            g[u] = ADD ? ld_stream<V>(add_grad, i + u * T) : v[u];
+            v[u] = ld_stream<V>(x, i + u * wk.su);
+            g[u] = ADD ? ld_stream<V>(add_grad, i + u * wk.su) : v[u];
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) st_stream<V>(dx, i + u * T, one(v[u], g[u]));
+        for (int u = 0; u < U; ++u) st_stream<V>(dx, i + u * wk.su, one(v[u], g[u]));
     }
-    for (; i < nchunks; i += T) {
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T) {
         const hv v = ld_stream<V>(x, i);
         st_stream<V>(dx, i, one(v, ADD ? ld_stream<V>(add_grad, i) : v));
     }
 }
 
 // ---------------------------------------------------------------- BN-ReLU
-template <int V>
-__global__ __launch_bounds__(kStreamThreads) void bnrelu_fwd_kernel(const half_t* __restrict__ x,
-                                                                    const float* __restrict__ wv,
-                                                                    const float* __restrict__ bv,
-                                                                    half_t* __restrict__ y, int64_t nchunks, int CG)
+template <int V, int U>
+__global__ __launch_bounds__(kStreamMaxThreads) void bnrelu_fwd_kernel(const half_t* __restrict__ x,
+                                                                       const float* __restrict__ wv,
+                                                                       const float* __restrict__ bv,
+                                                                       half_t* __restrict__ y, int64_t nchunks, int CG,
+                                                                       int segments)
 {
     typedef typename HVec<V>::type hv;
-    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
-    int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    const int cg = (int)(i % CG);
+    const ChunkWalk<U> wk(nchunks, segments != 0);
+    const int cg = (int)(wk.first % CG);
     float w[V], b[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
@@ -160,29 +141,29 @@ __global__ __launch_bounds__(kStreamThreads) void bnrelu_fwd_kernel(const half_t
         for (int j = 0; j < V; ++j) o[j] = (half_t)fmaxf(__builtin_fmaf((float)v[j], w[j], b[j]), 0.0f);
         return o;
     };
-    for (; i + 3 * T < nchunks; i += 4 * T) {
-        const hv v0 = ld_stream<V>(x, i), v1 = ld_stream<V>(x, i + T), v2 = ld_stream<V>(x, i + 2 * T), v3 = ld_stream<V>(x, i + 3 * T);
-        st_stream<V>(y, i, act(v0));
-        st_stream<V>(y, i + T, act(v1));
-        st_stream<V>(y, i + 2 * T, act(v2));
-        st_stream<V>(y, i + 3 * T, act(v3));
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
+        hv v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = ld_stream<V>(x, i + u * wk.su);
+#pragma unroll
+        for (int u = 0; u < U; ++u) st_stream<V>(y, i + u * wk.su, act(v[u]));
     }
-    for (; i < nchunks; i += T) st_stream<V>(y, i, act(ld_stream<V>(x, i)));
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T) st_stream<V>(y, i, act(ld_stream<V>(x, i)));
 }
 
-template <int V>
-__global__ __launch_bounds__(kStreamThreads) void bnrelu_bwd_kernel(const half_t* __restrict__ x,
-                                                                    const float* __restrict__ wv,
-                                                                    const float* __restrict__ bv,
-                                                                    const half_t* __restrict__ g,
-                                                                    half_t* __restrict__ dx, float* __restrict__ ws,
-                                                                    int64_t nchunks, int CG)
+template <int V, int U>
+__global__ __launch_bounds__(kStreamMaxThreads) void bnrelu_bwd_kernel(const half_t* __restrict__ x,
+                                                                       const float* __restrict__ wv,
+                                                                       const float* __restrict__ bv,
+                                                                       const half_t* __restrict__ g,
+                                                                       half_t* __restrict__ dx, float* __restrict__ ws,
+                                                                       int64_t nchunks, int CG, int segments)
 {
     typedef typename HVec<V>::type hv;
-    __shared__ float red[kStreamWaves * 2 * 64 * V];
-    const int64_t T = (int64_t)gridDim.x * kStreamThreads;
-    int64_t i = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    const int cg = (int)(i % CG);
+    __shared__ float red[4 * 2 * 64 * V];
+    const ChunkWalk<U> wk(nchunks, segments != 0);
+    const int cg = (int)(wk.first % CG);
     float w[V], nb[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
@@ -204,14 +185,19 @@ __global__ __launch_bounds__(kStreamThreads) void bnrelu_bwd_kernel(const half_t
         }
         st_stream<V>(dx, k, o);
     };
-    for (; i + T < nchunks; i += 2 * T) {
-        const hv x0 = ld_stream<V>(x, i), x1 = ld_stream<V>(x, i + T);
-        const hv g0 = ld_stream<V>(g, i), g1 = ld_stream<V>(g, i + T);
-        body(i, x0, g0);
-        body(i + T, x1, g1);
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
+        hv xv[U], gv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            xv[u] = ld_stream<V>(x, i + u * wk.su);
+            gv[u] = ld_stream<V>(g, i + u * wk.su);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) body(i + u * wk.su, xv[u], gv[u]);
     }
-    for (; i < nchunks; i += T) body(i, ld_stream<V>(x, i), ld_stream<V>(g, i));
-    block_channel_partials<2, V>(acc, CG, red, ws + (int64_t)blockIdx.x * 2 * CG * V);
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T) body(i, ld_stream<V>(x, i), ld_stream<V>(g, i));
+    block_channel_partials_any<2, V>(acc, CG, red, ws + (int64_t)blockIdx.x * 2 * CG * V);
 }
 
 // ------------------------------------------------------------ quantisers
@@ -267,18 +253,16 @@ __device__ __forceinline__ uint32_t bytes_word(const u32x2_t& v, int k) { return
 __device__ __forceinline__ void set_bytes_word(uint32_t& v, int, uint32_t w) { v = w; }
 __device__ __forceinline__ void set_bytes_word(u32x2_t& v, int k, uint32_t w) { v[k] = w; }
 
-constexpr int kQuantInFlight = 4;  // steps in flight per lane
-
-template <typename T, bool FAST>
-__global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
-                                                                  int64_t numel, float window, float r_two_w)
+template <typename T, int U, bool FAST>
+__global__ __launch_bounds__(kStreamMaxThreads) void quant_u8_kernel(const T* __restrict__ x, uint8_t* __restrict__ q,
+                                                                     int64_t numel, float window, float r_two_w,
+                                                                     int segments)
 {
     typedef QuantUnit<T> QU;
-    constexpr int E = QU::E, U = kQuantInFlight;
+    constexpr int E = QU::E;
     const float two_w = __fmul_rn(2.0f, window);
     const int64_t nunits = numel / E;
-    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
-    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
+    const ChunkWalk<U> wk(nunits, segments != 0);
     auto one = [&](const typename QU::wide_t& v) {
         typename QU::bytes_t o;
 #pragma unroll
@@ -293,31 +277,32 @@ __global__ __launch_bounds__(kStreamThreads) void quant_u8_kernel(const T* __res
     };
     const typename QU::wide_t* xv = reinterpret_cast<const typename QU::wide_t*>(x);
     typename QU::bytes_t* qv = reinterpret_cast<typename QU::bytes_t*>(q);
-    int64_t i = gid;
-    for (; i + (U - 1) * Tn < nunits; i += U * Tn) {
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
         typename QU::wide_t v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(xv + i + u * Tn);
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(xv + i + u * wk.su);
 #pragma unroll
-        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(v[u]), qv + i + u * Tn);
+        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(v[u]), qv + i + u * wk.su);
     }
-    for (; i < nunits; i += Tn) __builtin_nontemporal_store(one(__builtin_nontemporal_load(xv + i)), qv + i);
-    if (gid == 0) {
+    for (int64_t i = wk.tail; i < nunits; i += wk.T)
+        __builtin_nontemporal_store(one(__builtin_nontemporal_load(xv + i)), qv + i);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
         for (int64_t k = nunits * E; k < numel; ++k)
             q[k] = (uint8_t)quant_u8_one<FAST>(to_f32(x[k]), window, two_w, r_two_w);
     }
 }
 
-template <typename T>
-__global__ __launch_bounds__(kStreamThreads) void dequant_u8_kernel(const uint8_t* __restrict__ q,
-                                                                    T* __restrict__ out, int64_t numel, float window)
+template <typename T, int U>
+__global__ __launch_bounds__(kStreamMaxThreads) void dequant_u8_kernel(const uint8_t* __restrict__ q,
+                                                                       T* __restrict__ out, int64_t numel,
+                                                                       float window, int segments)
 {
     typedef QuantUnit<T> QU;
-    constexpr int E = QU::E, U = kQuantInFlight;
+    constexpr int E = QU::E;
     const float scale = __fdiv_rn(__fmul_rn(2.0f, window), 255.0f);
     const int64_t nunits = numel / E;
-    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
-    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
+    const ChunkWalk<U> wk(nunits, segments != 0);
     auto one = [&](const typename QU::bytes_t& b) {
         typename QU::wide_t o;
 #pragma unroll
@@ -327,40 +312,20 @@ __global__ __launch_bounds__(kStreamThreads) void dequant_u8_kernel(const uint8_
     };
     const typename QU::bytes_t* qv = reinterpret_cast<const typename QU::bytes_t*>(q);
     typename QU::wide_t* ov = reinterpret_cast<typename QU::wide_t*>(out);
-    int64_t i = gid;
-    for (; i + (U - 1) * Tn < nunits; i += U * Tn) {
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
         typename QU::bytes_t b[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) b[u] = __builtin_nontemporal_load(qv + i + u * Tn);
+        for (int u = 0; u < U; ++u) b[u] = __builtin_nontemporal_load(qv + i + u * wk.su);
 #pragma unroll
-        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(b[u]), ov + i + u * Tn);
+        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(b[u]), ov + i + u * wk.su);
     }
-    for (; i < nunits; i += Tn) __builtin_nontemporal_store(one(__builtin_nontemporal_load(qv + i)), ov + i);
-    if (gid == 0) {
+    for (int64_t i = wk.tail; i < nunits; i += wk.T)
+        __builtin_nontemporal_store(one(__builtin_nontemporal_load(qv + i)), ov + i);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
         for (int64_t k = nunits * E; k < numel; ++k)
             out[k] = (T)__fsub_rn(__fmul_rn((float)q[k], scale), window);
     }
-}
-
-// 16 consecutive fp16 values per lane (two 16-byte loads) for one 16-byte store of bytes: the int8 pass
-template <typename T>
-__device__ __forceinline__ void load16(const T* p, float (&f)[16])
-{
-    typedef T tv8 __attribute__((ext_vector_type(8)));
-    const tv8 a = __builtin_nontemporal_load(reinterpret_cast<const tv8*>(p));
-    const tv8 b = __builtin_nontemporal_load(reinterpret_cast<const tv8*>(p + 8));
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        f[j] = (float)a[j];
-        f[8 + j] = (float)b[j];
-    }
-}
-__device__ __forceinline__ u32x4_t pack16(const uint32_t (&b)[16])
-{
-    u32x4_t o;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) o[w] = b[4 * w] | (b[4 * w + 1] << 8) | (b[4 * w + 2] << 16) | (b[4 * w + 3] << 24);
-    return o;
 }
 
 __global__ __launch_bounds__(kStreamThreads) void absmax_kernel(const half_t* __restrict__ y, float* __restrict__ ws,
@@ -425,26 +390,42 @@ __device__ __forceinline__ uint32_t quant_i8_one(float v, float scale, float rsc
     return (uint32_t)((int)t) & 0xffu;
 }
 
-__global__ __launch_bounds__(kStreamThreads) void quant_i8_kernel(const half_t* __restrict__ y,
-                                                                  const float* __restrict__ absmax,
-                                                                  int8_t* __restrict__ q, int64_t numel)
+template <int U>
+__global__ __launch_bounds__(kStreamMaxThreads) void quant_i8_kernel(const half_t* __restrict__ y,
+                                                                     const float* __restrict__ absmax,
+                                                                     int8_t* __restrict__ q, int64_t numel,
+                                                                     int segments)
 {
     const float scale = __fdiv_rn(absmax[0], 127.0f);
     const bool zero = (scale == 0.0f);
     const float rscale = __fdiv_rn(1.0f, zero ? 1.0f : scale);  // correctly rounded reciprocal, once per thread
-    const int64_t ngroups = numel / 16;
-    const int64_t Tn = (int64_t)gridDim.x * kStreamThreads;
-    const int64_t gid = (int64_t)blockIdx.x * kStreamThreads + threadIdx.x;
-    for (int64_t i = gid; i < ngroups; i += Tn) {
-        float f[16];
-        load16<half_t>(y + i * 16, f);
-        uint32_t b[16];
+    const int64_t nunits = numel / 8;  // 16 bytes in, 8 bytes out per lane and access
+    const ChunkWalk<U> wk(nunits, segments != 0);
+    auto one = [&](const half8_t& v) {
+        u32x2_t o;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) b[j] = zero ? 0u : quant_i8_one(f[j], scale, rscale);
-        __builtin_nontemporal_store(pack16(b), reinterpret_cast<u32x4_t*>(q + i * 16));
+        for (int k = 0; k < 2; ++k) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w |= (zero ? 0u : quant_i8_one((float)v[4 * k + j], scale, rscale)) << (8 * j);
+            o[k] = w;
+        }
+        return o;
+    };
+    const half8_t* yv = reinterpret_cast<const half8_t*>(y);
+    u32x2_t* qv = reinterpret_cast<u32x2_t*>(q);
+    for (int64_t k = 0; k < wk.nfull; ++k) {
+        const int64_t i = k * wk.step + wk.first;
+        half8_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(yv + i + u * wk.su);
+#pragma unroll
+        for (int u = 0; u < U; ++u) __builtin_nontemporal_store(one(v[u]), qv + i + u * wk.su);
     }
-    if (gid == 0) {
-        for (int64_t k = ngroups * 16; k < numel; ++k)
+    for (int64_t i = wk.tail; i < nunits; i += wk.T)
+        __builtin_nontemporal_store(one(__builtin_nontemporal_load(yv + i)), qv + i);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        for (int64_t k = nunits * 8; k < numel; ++k)
             q[k] = zero ? (int8_t)0 : (int8_t)quant_i8_one((float)y[k], scale, rscale);
     }
 }
@@ -454,84 +435,175 @@ __global__ __launch_bounds__(kStreamThreads) void quant_i8_kernel(const half_t* 
 using namespace kerops;
 
 // ------------------------------------------------------------------ C ABI
+//
+// Launch shape of an entry point: (blocks, waves, segment), 0 = the built-in choice below.
+//   blocks   workgroups of the persistent loop
+//   waves    wavefronts per workgroup: 4, 8 or 16
+//   segment  1 = interleaved walk, 4 or 8 = each workgroup step covers one contiguous run of that many
+//            chunks per thread (8 needs C >= 8)
+// Built-in choices: measured on MI355X at (1,64,350,350,128) with `python -m kerops_amd.tune --streams`.
+namespace {
+
+struct StreamDefault {
+    int blocks, waves, segment;
+};
+constexpr StreamDefault kDefStats{512, 4, 4};
+constexpr StreamDefault kDefAddStats{256, 4, 1};
+constexpr StreamDefault kDefStatsBwd{4096, 16, 4};
+constexpr StreamDefault kDefAddStatsBwd{512, 4, 4};
+constexpr StreamDefault kDefBnReluFwd{4096, 16, 4};
+constexpr StreamDefault kDefBnReluBwd{1280, 16, 4};
+constexpr StreamDefault kDefQuantU8{256, 4, 8};
+constexpr StreamDefault kDefDequantU8{512, 4, 4};
+constexpr StreamDefault kDefQuantI8{4096, 16, 4};
+constexpr int kMaxStreamBlocks = 65536;
+constexpr int kMaxDefaultBlocks = 4096;  // workspace queries with blocks = 0 size for this many partials
+
+int resolve_shape(const char* op, const StreamDefault& def, int64_t work_items, bool wide8, int blocks, int waves,
+                  int segment, StreamShape* out)
+{
+    if (waves == 0) waves = def.waves;
+    if (segment == 0) segment = (def.segment == 8 && !wide8) ? 4 : def.segment;
+    if (!(waves == 4 || waves == 8 || waves == 16)) {
+        set_error("%s: waves must be 4, 8 or 16 wavefronts per workgroup (got %d)", op, waves);
+        return KEROPS_E_BADARG;
+    }
+    if (!(segment == 1 || segment == 4 || (segment == 8 && wide8))) {
+        set_error("%s: segment must be 1 (interleaved), 4 or 8 (8 only with 16-byte chunks; got %d)", op, segment);
+        return KEROPS_E_BADARG;
+    }
+    out->threads = waves * kWave;
+    out->segment = segment;
+    if (blocks > kMaxStreamBlocks) {
+        set_error("%s: blocks must be <= %d", op, kMaxStreamBlocks);
+        return KEROPS_E_BADARG;
+    }
+    if (blocks <= 0) blocks = def.blocks;
+    // never more workgroups than steps of work (small tensors)
+    const int64_t per_step = (int64_t)out->threads * out->unroll();
+    out->blocks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(work_items, per_step), blocks));
+    return KEROPS_OK;
+}
+
+int check_channels(const char* op, int64_t M, int C, bool reduces)
+{
+    if (M <= 0 || C <= 0 || !is_pow2(C)) {
+        set_error("%s: M must be positive and C a power of two (M=%lld C=%d)", op, (long long)M, C);
+        return KEROPS_E_BADARG;
+    }
+    if (reduces && C > kMaxReduceChannels) {
+        set_error("%s: per-channel reductions are built for C <= %d (got %d)", op, kMaxReduceChannels, C);
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    if (C / (C >= 8 ? 8 : C) > 256) {  // a thread keeps its channel group: threads % (C/8) == 0
+        set_error("%s: built for C <= 2048 (got %d)", op, C);
+        return KEROPS_E_UNSUPPORTED_C;
+    }
+    return KEROPS_OK;
+}
+
+int check_ws(const char* op, const void* ws, int64_t have, int64_t need)
+{
+    if (!ws || !aligned16(ws) || have < need) {
+        set_error("%s: workspace of %lld bytes required, %lld given", op, (long long)need, (long long)have);
+        return KEROPS_E_WORKSPACE;
+    }
+    return KEROPS_OK;
+}
+
+// Runs the statement list with constexpr V = min(8, C) and U = 4 or 8 (8 only with V = 8) in scope.
+#define KEROPS_DISPATCH_VU(C, shape, ...)          \
+    do {                                           \
+        if ((C) >= 8 && (shape).unroll() == 8) {   \
+            constexpr int V = 8, U = 8;            \
+            __VA_ARGS__;                           \
+        } else {                                   \
+            constexpr int U = 4;                   \
+            KEROPS_DISPATCH_V(C, __VA_ARGS__);     \
+        }                                          \
+    } while (0)
+
+}  // namespace
 
 extern "C" int64_t kerops_stats_workspace_bytes(int64_t M, int32_t C, int32_t blocks)
 {
-    int64_t need = 0;
-    int rc = check_reduce_args("stats", M, C, &blocks, &need);
-    return rc != KEROPS_OK ? rc : need;
+    int rc = check_channels("stats", M, C, true);
+    if (rc != KEROPS_OK) return rc;
+    if (blocks > kMaxStreamBlocks) {
+        set_error("stats: blocks must be <= %d", kMaxStreamBlocks);
+        return KEROPS_E_BADARG;
+    }
+    if (blocks <= 0) blocks = kMaxDefaultBlocks;
+    return (int64_t)blocks * 2 * C * (int64_t)sizeof(float);
 }
 
-static int stats_common(const char* op, const void* x, const void* y, void* z, float* mean, float* sqmean, int64_t M,
-                        int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks, void* stream)
+static int stats_common(const char* op, const StreamDefault& def, const void* x, const void* y, void* z, float* mean,
+                        float* sqmean, int64_t M, int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks,
+                        int32_t waves, int32_t segment, void* stream)
 {
-    int64_t need = 0;
-    int rc = check_reduce_args(op, M, C, &blocks, &need);
+    int rc = check_channels(op, M, C, true);
+    if (rc != KEROPS_OK) return rc;
+    const int Vr = C >= 8 ? 8 : C;
+    const int CG = C / Vr;
+    const int64_t nchunks = M * CG;
+    StreamShape sh;
+    rc = resolve_shape(op, def, nchunks, Vr == 8, blocks, waves, segment, &sh);
     if (rc != KEROPS_OK) return rc;
     const bool add = (y != nullptr);
     if (!x || !mean || !sqmean || !aligned16(x) || (add && (!z || !aligned16(y) || !aligned16(z)))) {
         set_error("%s: null or misaligned pointer", op);
         return KEROPS_E_BADARG;
     }
-    rc = check_ws(op, workspace, workspace_bytes, need);
+    rc = check_ws(op, workspace, workspace_bytes, (int64_t)sh.blocks * 2 * C * (int64_t)sizeof(float));
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
-    const int Vr = C >= 8 ? 8 : C;
-    const int CG = C / Vr;
-    const int64_t nchunks = M * CG;
     float* ws = (float*)workspace;
-    KEROPS_DISPATCH_V(C, {
+    const int seg = sh.segment != 1;
+    KEROPS_DISPATCH_VU(C, sh, {
         if (add) {
-            hipLaunchKernelGGL((stats_kernel<V, true>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x,
-                               (const half_t*)y, (half_t*)z, ws, nchunks, CG);
+            hipLaunchKernelGGL((stats_kernel<V, U, true>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const half_t*)x,
+                               (const half_t*)y, (half_t*)z, ws, nchunks, CG, seg);
         } else {
-            hipLaunchKernelGGL((stats_kernel<V, false>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x,
-                               (const half_t*)nullptr, (half_t*)nullptr, ws, nchunks, CG);
+            hipLaunchKernelGGL((stats_kernel<V, U, false>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const half_t*)x,
+                               (const half_t*)nullptr, (half_t*)nullptr, ws, nchunks, CG, seg);
         }
     });
     rc = check_launch(op);
     if (rc != KEROPS_OK) return rc;
-    launch_reduce_rows(ws, blocks, 2 * C, mean, sqmean, C, 1.0 / (double)M, s);
+    launch_reduce_rows(ws, sh.blocks, 2 * C, mean, sqmean, C, 1.0 / (double)M, s);
     return check_launch(op);
 }
 
 extern "C" int kerops_stats_f16(const void* x, float* mean, float* sqmean, int64_t M, int32_t C, void* workspace,
-                                int64_t workspace_bytes, int32_t blocks, void* stream)
+                                int64_t workspace_bytes, int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
-    return stats_common("stats", x, nullptr, nullptr, mean, sqmean, M, C, workspace, workspace_bytes, blocks, stream);
+    return stats_common("stats", kDefStats, x, nullptr, nullptr, mean, sqmean, M, C, workspace, workspace_bytes, blocks,
+                        waves, segment, stream);
 }
 
 extern "C" int kerops_add_stats_f16(const void* x, const void* y, void* z, float* mean, float* sqmean, int64_t M,
-                                    int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks, void* stream)
+                                    int32_t C, void* workspace, int64_t workspace_bytes, int32_t blocks, int32_t waves,
+                                    int32_t segment, void* stream)
 {
     if (!y) {
         set_error("add_stats: null pointer");
         return KEROPS_E_BADARG;
     }
-    return stats_common("add_stats", x, y, z, mean, sqmean, M, C, workspace, workspace_bytes, blocks, stream);
+    return stats_common("add_stats", kDefAddStats, x, y, z, mean, sqmean, M, C, workspace, workspace_bytes, blocks,
+                        waves, segment, stream);
 }
 
-static int check_stream_args(const char* op, int64_t M, int C, int* blocks)
+static int stats_bwd_common(const char* op, const StreamDefault& def, const void* x, const void* add_grad,
+                            const float* mean_grad, const float* sqmean_grad, void* dx, int64_t M, int32_t C,
+                            int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
-    if (M <= 0 || C <= 0 || !is_pow2(C)) {
-        set_error("%s: M must be positive and C a power of two (M=%lld C=%d)", op, (long long)M, C);
-        return KEROPS_E_BADARG;
-    }
-    const int V = C >= 8 ? 8 : C;
-    if (*blocks <= 0) *blocks = stream_blocks_default(M * (C / V));
-    // a thread keeps one channel group only if the grid stride is a multiple of C/V
-    const int CG = C / V;
-    if (((int64_t)(*blocks) * kStreamThreads) % CG != 0) {
-        set_error("%s: blocks*256 must be a multiple of C/8", op);
-        return KEROPS_E_BADARG;
-    }
-    return KEROPS_OK;
-}
-
-static int stats_bwd_common(const char* op, const void* x, const void* add_grad, const float* mean_grad,
-                            const float* sqmean_grad, void* dx, int64_t M, int32_t C, int32_t blocks, void* stream)
-{
-    int rc = check_stream_args(op, M, C, &blocks);
+    int rc = check_channels(op, M, C, false);
+    if (rc != KEROPS_OK) return rc;
+    const int Vr = C >= 8 ? 8 : C;
+    const int CG = C / Vr;
+    const int64_t nchunks = M * CG;
+    StreamShape sh;
+    rc = resolve_shape(op, def, nchunks, Vr == 8, blocks, waves, segment, &sh);
     if (rc != KEROPS_OK) return rc;
     if (!x || !mean_grad || !sqmean_grad || !dx || !aligned16(x) || !aligned16(dx) ||
         (add_grad && !aligned16(add_grad))) {
@@ -539,100 +611,114 @@ static int stats_bwd_common(const char* op, const void* x, const void* add_grad,
         return KEROPS_E_BADARG;
     }
     hipStream_t s = (hipStream_t)stream;
-    const int Vr = C >= 8 ? 8 : C;
-    const int CG = C / Vr;
-    const int64_t nchunks = M * CG;
-    KEROPS_DISPATCH_V(C, {
+    const int seg = sh.segment != 1;
+    KEROPS_DISPATCH_VU(C, sh, {
         if (add_grad) {
-            hipLaunchKernelGGL((stats_bwd_kernel<V, true>), dim3(blocks), dim3(kStreamThreads), 0, s,
+            hipLaunchKernelGGL((stats_bwd_kernel<V, U, true>), dim3(sh.blocks), dim3(sh.threads), 0, s,
                                (const half_t*)x, (const half_t*)add_grad, mean_grad, sqmean_grad, (half_t*)dx,
-                               nchunks, CG, (float)M);
+                               nchunks, CG, (float)M, seg);
         } else {
-            hipLaunchKernelGGL((stats_bwd_kernel<V, false>), dim3(blocks), dim3(kStreamThreads), 0, s,
+            hipLaunchKernelGGL((stats_bwd_kernel<V, U, false>), dim3(sh.blocks), dim3(sh.threads), 0, s,
                                (const half_t*)x, (const half_t*)nullptr, mean_grad, sqmean_grad, (half_t*)dx, nchunks,
-                               CG, (float)M);
+                               CG, (float)M, seg);
         }
     });
     return check_launch(op);
 }
 
 extern "C" int kerops_stats_bwd_f16(const void* x, const float* mean_grad, const float* sqmean_grad, void* dx,
-                                    int64_t M, int32_t C, int32_t blocks, void* stream)
+                                    int64_t M, int32_t C, int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
-    return stats_bwd_common("stats_bwd", x, nullptr, mean_grad, sqmean_grad, dx, M, C, blocks, stream);
+    return stats_bwd_common("stats_bwd", kDefStatsBwd, x, nullptr, mean_grad, sqmean_grad, dx, M, C, blocks, waves,
+                            segment, stream);
 }
 
 extern "C" int kerops_add_stats_bwd_f16(const void* add_grad, const float* mean_grad, const float* sqmean_grad,
                                         const void* add_result, void* out, int64_t M, int32_t C, int32_t blocks,
-                                        void* stream)
+                                        int32_t waves, int32_t segment, void* stream)
 {
     if (!add_grad) {
         set_error("add_stats_bwd: null pointer");
         return KEROPS_E_BADARG;
     }
-    return stats_bwd_common("add_stats_bwd", add_result, add_grad, mean_grad, sqmean_grad, out, M, C, blocks, stream);
+    return stats_bwd_common("add_stats_bwd", kDefAddStatsBwd, add_result, add_grad, mean_grad, sqmean_grad, out, M, C,
+                            blocks, waves, segment, stream);
 }
 
 extern "C" int kerops_bnrelu_fwd_f16(const void* x, const float* wv, const float* bv, void* y, int64_t M, int32_t C,
-                                     int32_t blocks, void* stream)
+                                     int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
-    int rc = check_stream_args("bnrelu_fwd", M, C, &blocks);
+    int rc = check_channels("bnrelu_fwd", M, C, false);
+    if (rc != KEROPS_OK) return rc;
+    const int Vr = C >= 8 ? 8 : C;
+    const int CG = C / Vr;
+    StreamShape sh;
+    rc = resolve_shape("bnrelu_fwd", kDefBnReluFwd, M * CG, Vr == 8, blocks, waves, segment, &sh);
     if (rc != KEROPS_OK) return rc;
     if (!x || !wv || !bv || !y || !aligned16(x) || !aligned16(y)) {
         set_error("bnrelu_fwd: null or misaligned pointer");
         return KEROPS_E_BADARG;
     }
     hipStream_t s = (hipStream_t)stream;
-    const int Vr = C >= 8 ? 8 : C;
-    const int CG = C / Vr;
-    KEROPS_DISPATCH_V(C, {
-        hipLaunchKernelGGL((bnrelu_fwd_kernel<V>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x, wv, bv,
-                           (half_t*)y, M * CG, CG);
+    const int seg = sh.segment != 1;
+    KEROPS_DISPATCH_VU(C, sh, {
+        hipLaunchKernelGGL((bnrelu_fwd_kernel<V, U>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const half_t*)x, wv,
+                           bv, (half_t*)y, M * CG, CG, seg);
     });
     return check_launch("bnrelu_fwd");
 }
 
 extern "C" int kerops_bnrelu_bwd_f16(const void* x, const float* wv, const float* bv, const void* g, void* dx,
                                      float* dW, float* dB, int64_t M, int32_t C, void* workspace,
-                                     int64_t workspace_bytes, int32_t blocks, void* stream)
+                                     int64_t workspace_bytes, int32_t blocks, int32_t waves, int32_t segment,
+                                     void* stream)
 {
-    int64_t need = 0;
-    int rc = check_reduce_args("bnrelu_bwd", M, C, &blocks, &need);
+    int rc = check_channels("bnrelu_bwd", M, C, true);
+    if (rc != KEROPS_OK) return rc;
+    const int Vr = C >= 8 ? 8 : C;
+    const int CG = C / Vr;
+    StreamShape sh;
+    rc = resolve_shape("bnrelu_bwd", kDefBnReluBwd, M * CG, Vr == 8, blocks, waves, segment, &sh);
     if (rc != KEROPS_OK) return rc;
     if (!x || !wv || !bv || !g || !dx || !dW || !dB || !aligned16(x) || !aligned16(g) || !aligned16(dx)) {
         set_error("bnrelu_bwd: null or misaligned pointer");
         return KEROPS_E_BADARG;
     }
-    rc = check_ws("bnrelu_bwd", workspace, workspace_bytes, need);
+    rc = check_ws("bnrelu_bwd", workspace, workspace_bytes, (int64_t)sh.blocks * 2 * C * (int64_t)sizeof(float));
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
-    const int Vr = C >= 8 ? 8 : C;
-    const int CG = C / Vr;
     float* ws = (float*)workspace;
-    KEROPS_DISPATCH_V(C, {
-        hipLaunchKernelGGL((bnrelu_bwd_kernel<V>), dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)x, wv, bv,
-                           (const half_t*)g, (half_t*)dx, ws, M * CG, CG);
+    const int seg = sh.segment != 1;
+    KEROPS_DISPATCH_VU(C, sh, {
+        hipLaunchKernelGGL((bnrelu_bwd_kernel<V, U>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const half_t*)x, wv,
+                           bv, (const half_t*)g, (half_t*)dx, ws, M * CG, CG, seg);
     });
     rc = check_launch("bnrelu_bwd");
     if (rc != KEROPS_OK) return rc;
-    launch_reduce_rows(ws, blocks, 2 * C, dW, dB, C, 1.0, s);
+    launch_reduce_rows(ws, sh.blocks, 2 * C, dW, dB, C, 1.0, s);
     return check_launch("bnrelu_bwd");
 }
 
-static int check_flat(const char* op, const void* a, const void* b, int64_t numel, int* blocks)
+static int check_flat(const char* op, const StreamDefault& def, const void* a, const void* b, int64_t numel,
+                      int64_t units, int blocks, int waves, int segment, StreamShape* sh)
 {
     if (!a || !b || !aligned16(a) || !aligned16(b) || numel <= 0) {
         set_error("%s: null or misaligned pointer, or non-positive numel", op);
         return KEROPS_E_BADARG;
     }
-    if (*blocks <= 0) *blocks = stream_blocks_default(ceil_div64(numel, 16), 768);
-    return KEROPS_OK;
+    return resolve_shape(op, def, units, true, blocks, waves, segment, sh);
 }
 
 extern "C" int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int64_t numel, float window,
-                                      int32_t blocks, void* stream)
+                                      int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
-    int rc = check_flat("quant_u8_window", x, q, numel, &blocks);
+    if (!(dtype == KEROPS_DTYPE_F16 || dtype == KEROPS_DTYPE_BF16 || dtype == KEROPS_DTYPE_F32)) {
+        set_error("quant_u8_window: unknown dtype tag %d", dtype);
+        return KEROPS_E_BADARG;
+    }
+    StreamShape sh;
+    int rc = check_flat("quant_u8_window", kDefQuantU8, x, q, numel, numel / (dtype == KEROPS_DTYPE_F32 ? 4 : 8), blocks,
+                        waves, segment, &sh);
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
     // 1/(2w) correctly rounded to fp32: the double quotient rounded once more is exact for division
@@ -640,45 +726,59 @@ extern "C" int kerops_quant_u8_window(const void* x, int32_t dtype, void* q, int
     const float two_w = 2.0f * window;
     const bool fast = window >= 0x1p-60f && window <= 0x1p60f;
     const float r_two_w = fast ? (float)(1.0 / (double)two_w) : 0.0f;
-#define KEROPS_QU8_GO(T, F)                                                                                     \
-    hipLaunchKernelGGL((quant_u8_kernel<T, F>), dim3(blocks), dim3(kStreamThreads), 0, s, (const T*)x, (uint8_t*)q, \
-                       numel, window, r_two_w)
-    if (dtype == KEROPS_DTYPE_F16) {
-        if (fast) KEROPS_QU8_GO(half_t, true);
-        else KEROPS_QU8_GO(half_t, false);
-    } else if (dtype == KEROPS_DTYPE_BF16) {
-        if (fast) KEROPS_QU8_GO(bf16_t, true);
-        else KEROPS_QU8_GO(bf16_t, false);
-    } else if (dtype == KEROPS_DTYPE_F32) {
-        if (fast) KEROPS_QU8_GO(float, true);
-        else KEROPS_QU8_GO(float, false);
-    } else {
-        set_error("quant_u8_window: unknown dtype tag %d", dtype);
-        return KEROPS_E_BADARG;
+    const int seg = sh.segment != 1;
+#define KEROPS_QU8_GO(T, Uv, F)                                                                                  \
+    hipLaunchKernelGGL((quant_u8_kernel<T, Uv, F>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const T*)x, (uint8_t*)q, \
+                       numel, window, r_two_w, seg)
+#define KEROPS_QU8_T(T)                            \
+    if (sh.unroll() == 8) {                        \
+        if (fast) KEROPS_QU8_GO(T, 8, true);       \
+        else KEROPS_QU8_GO(T, 8, false);           \
+    } else {                                       \
+        if (fast) KEROPS_QU8_GO(T, 4, true);       \
+        else KEROPS_QU8_GO(T, 4, false);           \
     }
+    if (dtype == KEROPS_DTYPE_F16) {
+        KEROPS_QU8_T(half_t)
+    } else if (dtype == KEROPS_DTYPE_BF16) {
+        KEROPS_QU8_T(bf16_t)
+    } else {
+        KEROPS_QU8_T(float)
+    }
+#undef KEROPS_QU8_T
 #undef KEROPS_QU8_GO
     return check_launch("quant_u8_window");
 }
 
 extern "C" int kerops_dequant_u8_window(const void* q, void* out, int32_t dtype, int64_t numel, float window,
-                                        int32_t blocks, void* stream)
+                                        int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
-    int rc = check_flat("dequant_u8_window", q, out, numel, &blocks);
-    if (rc != KEROPS_OK) return rc;
-    hipStream_t s = (hipStream_t)stream;
-    if (dtype == KEROPS_DTYPE_F16) {
-        hipLaunchKernelGGL((dequant_u8_kernel<half_t>), dim3(blocks), dim3(kStreamThreads), 0, s, (const uint8_t*)q,
-                           (half_t*)out, numel, window);
-    } else if (dtype == KEROPS_DTYPE_BF16) {
-        hipLaunchKernelGGL((dequant_u8_kernel<bf16_t>), dim3(blocks), dim3(kStreamThreads), 0, s, (const uint8_t*)q,
-                           (bf16_t*)out, numel, window);
-    } else if (dtype == KEROPS_DTYPE_F32) {
-        hipLaunchKernelGGL((dequant_u8_kernel<float>), dim3(blocks), dim3(kStreamThreads), 0, s, (const uint8_t*)q,
-                           (float*)out, numel, window);
-    } else {
+    if (!(dtype == KEROPS_DTYPE_F16 || dtype == KEROPS_DTYPE_BF16 || dtype == KEROPS_DTYPE_F32)) {
         set_error("dequant_u8_window: unknown dtype tag %d", dtype);
         return KEROPS_E_BADARG;
     }
+    StreamShape sh;
+    int rc = check_flat("dequant_u8_window", kDefDequantU8, q, out, numel, numel / (dtype == KEROPS_DTYPE_F32 ? 4 : 8),
+                        blocks, waves, segment, &sh);
+    if (rc != KEROPS_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const int seg = sh.segment != 1;
+#define KEROPS_DQ_T(T)                                                                                              \
+    if (sh.unroll() == 8) {                                                                                         \
+        hipLaunchKernelGGL((dequant_u8_kernel<T, 8>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const uint8_t*)q,   \
+                           (T*)out, numel, window, seg);                                                            \
+    } else {                                                                                                        \
+        hipLaunchKernelGGL((dequant_u8_kernel<T, 4>), dim3(sh.blocks), dim3(sh.threads), 0, s, (const uint8_t*)q,   \
+                           (T*)out, numel, window, seg);                                                            \
+    }
+    if (dtype == KEROPS_DTYPE_F16) {
+        KEROPS_DQ_T(half_t)
+    } else if (dtype == KEROPS_DTYPE_BF16) {
+        KEROPS_DQ_T(bf16_t)
+    } else {
+        KEROPS_DQ_T(float)
+    }
+#undef KEROPS_DQ_T
     return check_launch("dequant_u8_window");
 }
 
@@ -692,10 +792,15 @@ extern "C" int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, vo
                                  int64_t workspace_bytes, int32_t blocks, void* stream)
 {
     if (blocks <= 0) blocks = 768;
-    int b = blocks;
-    int rc = check_flat("absmax", y, absmax, numel, &b);
-    if (rc != KEROPS_OK) return rc;
-    rc = check_ws("absmax", workspace, workspace_bytes, (int64_t)blocks * 4);
+    if (!y || !absmax || !aligned16(y) || numel <= 0) {
+        set_error("absmax: null or misaligned pointer, or non-positive numel");
+        return KEROPS_E_BADARG;
+    }
+    if (blocks > kMaxStreamBlocks) {
+        set_error("absmax: blocks must be <= %d", kMaxStreamBlocks);
+        return KEROPS_E_BADARG;
+    }
+    int rc = check_ws("absmax", workspace, workspace_bytes, (int64_t)blocks * 4);
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(kStreamThreads), 0, s, (const half_t*)y, (float*)workspace,
@@ -708,15 +813,22 @@ extern "C" int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, vo
 }
 
 extern "C" int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t numel, int32_t blocks,
-                                       void* stream)
+                                       int32_t waves, int32_t segment, void* stream)
 {
-    int rc = check_flat("quant_i8_sym", y, q, numel, &blocks);
+    StreamShape sh;
+    int rc = check_flat("quant_i8_sym", kDefQuantI8, y, q, numel, numel / 8, blocks, waves, segment, &sh);
     if (rc != KEROPS_OK) return rc;
     if (!absmax) {
         set_error("quant_i8_sym: null absmax");
         return KEROPS_E_BADARG;
     }
-    hipLaunchKernelGGL(quant_i8_kernel, dim3(blocks), dim3(kStreamThreads), 0, (hipStream_t)stream,
-                       (const half_t*)y, absmax, (int8_t*)q, numel);
+    const int seg = sh.segment != 1;
+    if (sh.unroll() == 8) {
+        hipLaunchKernelGGL(quant_i8_kernel<8>, dim3(sh.blocks), dim3(sh.threads), 0, (hipStream_t)stream,
+                           (const half_t*)y, absmax, (int8_t*)q, numel, seg);
+    } else {
+        hipLaunchKernelGGL(quant_i8_kernel<4>, dim3(sh.blocks), dim3(sh.threads), 0, (hipStream_t)stream,
+                           (const half_t*)y, absmax, (int8_t*)q, numel, seg);
+    }
     return check_launch("quant_i8_sym");
 }

@@ -7,14 +7,20 @@ import torch
 
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
+from ..settings.stream_table import stream_knob
 from ._common import next_power_of_2, numel_no_channels, require_cuda
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=8, blocks=0)
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AddStats', 'num_warps'),
+           blocks=stream_knob('AddStats', 'blocks'), segment=stream_knob('AddStats', 'segment'))
 def AddStats(
-    x, y, inplace=False, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg
+    x, y, inplace=False, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg,
+    segment: ConfigurableArg
 ):
-    """Returns (x + y as fp16, mean, sqmean); with inplace=True the sum overwrites x."""
+    """Returns (x + y as fp16, mean, sqmean); with inplace=True the sum overwrites x.
+    Launch knobs: `num_warps` = wavefronts per workgroup (4, 8, 16), `blocks` = workgroups, `segment` = walk of the
+    stream (1 interleaved, 4 / 8 contiguous chunks per thread); 0 = the library's choice.  `l1_cache_bytes` is
+    accepted and not used."""
     num_channels = x.shape[1]
     assert x.shape == y.shape
     assert x.ndim == y.ndim == 5
@@ -31,11 +37,13 @@ def AddStats(
     mean = torch.empty(num_channels, dtype=torch.float32, device=x.device)
     sqmean = torch.empty(num_channels, dtype=torch.float32, device=x.device)
     _lib.call('kerops_add_stats_f16', x.data_ptr(), y.data_ptr(), output.data_ptr(), mean.data_ptr(),
-              sqmean.data_ptr(), m, num_channels, ws.data_ptr(), ws_bytes, int(blocks), _lib.stream_of(x))
+              sqmean.data_ptr(), m, num_channels, ws.data_ptr(), ws_bytes, int(blocks), int(num_warps), int(segment),
+              _lib.stream_of(x))
     return output, mean, sqmean
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=8, blocks=0)
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AddStatsBackward', 'num_warps'),
+           blocks=stream_knob('AddStatsBackward', 'blocks'), segment=stream_knob('AddStatsBackward', 'segment'))
 def AddStatsBackward(
     add_grad,
     mean_grad,
@@ -45,8 +53,9 @@ def AddStatsBackward(
     l1_cache_bytes: ConfigurableArg,
     num_warps: ConfigurableArg,
     blocks: ConfigurableArg,
+    segment: ConfigurableArg,
 ):
-    """grad = add_grad + 2*add_result*sqmean_grad/M + mean_grad/M as fp16."""
+    """grad = add_grad + 2*add_result*sqmean_grad/M + mean_grad/M as fp16.  Launch knobs as for AddStats."""
     num_channels = add_grad.shape[1]
     assert add_result.shape == add_grad.shape
     assert add_grad.ndim == add_result.ndim == 5
@@ -62,5 +71,5 @@ def AddStatsBackward(
     output_grad = torch.empty_like(add_grad)
     _lib.call('kerops_add_stats_bwd_f16', add_grad.data_ptr(), mean_grad.data_ptr(), sqmean_grad.data_ptr(),
               add_result.data_ptr(), output_grad.data_ptr(), numel_no_channels(add_grad), num_channels, int(blocks),
-              _lib.stream_of(add_grad))
+              int(num_warps), int(segment), _lib.stream_of(add_grad))
     return output_grad

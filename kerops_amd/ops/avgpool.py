@@ -10,12 +10,19 @@ import torch
 
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
+from ..settings.stream_table import stream_knob
 from ._common import next_power_of_2, require_cuda
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=2, blocks=0)
-def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg):
-    """Returns (pooled fp16 (N,C,ceil(H/2),ceil(W/2),ceil(D/2)) channels_last_3d, mean, sqmean)."""
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AvgPoolCeilStats', 'num_warps'),
+           blocks=stream_knob('AvgPoolCeilStats', 'blocks'), segment=stream_knob('AvgPoolCeilStats', 'segment'))
+def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg,
+                     segment: ConfigurableArg):
+    """Returns (pooled fp16 (N,C,ceil(H/2),ceil(W/2),ceil(D/2)) channels_last_3d, mean, sqmean).
+
+    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (4, 8 or 16), `blocks` = workgroups, `segment` =
+    pooled chunks per thread and step (1 or 2); 0 = the library's choice.  `l1_cache_bytes` only feeds the
+    reference's row-size assert below."""
     num_channels = x.shape[1]
     input_d = x.shape[-1]
     MAX_SIZE = l1_cache_bytes // x.element_size()
@@ -37,12 +44,16 @@ def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: Configura
     ws_bytes = _lib.query('kerops_avgpool_ceil_stats_workspace_bytes', n, h, w, d, num_channels, int(blocks))
     ws = _lib.workspace(ws_bytes, x.device)
     _lib.call('kerops_avgpool_ceil_stats_f16', x.data_ptr(), output.data_ptr(), mean.data_ptr(), sqmean.data_ptr(),
-              n, h, w, d, num_channels, ws.data_ptr(), ws_bytes, int(blocks), _lib.stream_of(x))
+              n, h, w, d, num_channels, ws.data_ptr(), ws_bytes, int(blocks), int(num_warps), int(segment),
+              _lib.stream_of(x))
     return output, mean, sqmean
 
 
-@configure(blocks=0)
-def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg):
+@configure(blocks=stream_knob('ApplyBNReLUAvgPoolCeilStats', 'blocks'),
+           num_warps=stream_knob('ApplyBNReLUAvgPoolCeilStats', 'num_warps'),
+           segment=stream_knob('ApplyBNReLUAvgPoolCeilStats', 'segment'))
+def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg, num_warps: ConfigurableArg,
+                                segment: ConfigurableArg):
     """ApplyBNReLU(x, weight, bias) followed by AvgPoolCeilStats in one pass over x (no reference counterpart:
     the reference composes kerops/ops/bnrelu.py:11-41 and kerops/ops/avgpool.py:11-60).  Bit-identical to the
     composition; the full-size activation is neither written nor read.  Returns (pooled, mean, sqmean)."""
@@ -65,11 +76,13 @@ def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg):
     ws = _lib.workspace(ws_bytes, x.device)
     _lib.call('kerops_bnrelu_avgpool_ceil_stats_f16', x.data_ptr(), weight.data_ptr(), bias.data_ptr(),
               output.data_ptr(), mean.data_ptr(), sqmean.data_ptr(), n, h, w, d, num_channels, ws.data_ptr(),
-              ws_bytes, int(blocks), _lib.stream_of(x))
+              ws_bytes, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
     return output, mean, sqmean
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=4, blocks=0)
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AvgPoolCeilStatsBackward', 'num_warps'),
+           blocks=stream_knob('AvgPoolCeilStatsBackward', 'blocks'),
+           segment=stream_knob('AvgPoolCeilStatsBackward', 'segment'))
 def AvgPoolCeilStatsBackward(
     inpgrad,
     meangrad,
@@ -80,8 +93,10 @@ def AvgPoolCeilStatsBackward(
     l1_cache_bytes: ConfigurableArg,
     num_warps: ConfigurableArg,
     blocks: ConfigurableArg,
+    segment: ConfigurableArg,
 ):
-    """Gradient w.r.t. the pooling input, fp16, shape `outgrad_shape`, channels_last_3d."""
+    """Gradient w.r.t. the pooling input, fp16, shape `outgrad_shape`, channels_last_3d.
+    Launch knobs as for AvgPoolCeilStats."""
     MAX_SIZE = l1_cache_bytes // inpgrad.element_size()
     bsize, num_channels, h_outgrad, w_outgrad, d_outgrad = outgrad_shape
 
@@ -106,5 +121,5 @@ def AvgPoolCeilStatsBackward(
     sqmeangrad = sqmeangrad.contiguous()
     _lib.call('kerops_avgpool_ceil_stats_bwd_f16', inpgrad.data_ptr(), meangrad.data_ptr(), sqmeangrad.data_ptr(),
               output.data_ptr(), outgrad.data_ptr(), bsize, h_outgrad, w_outgrad, d_outgrad, num_channels,
-              int(blocks), _lib.stream_of(inpgrad))
+              int(blocks), int(num_warps), int(segment), _lib.stream_of(inpgrad))
     return outgrad

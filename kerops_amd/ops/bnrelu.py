@@ -9,13 +9,21 @@ import torch
 
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
+from ..settings.stream_table import stream_knob
 from ._common import next_power_of_2, numel_no_channels, require_cuda
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=8, blocks=0)
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('ApplyBNReLU', 'num_warps'),
+           blocks=stream_knob('ApplyBNReLU', 'blocks'), segment=stream_knob('ApplyBNReLU', 'segment'))
 def ApplyBNReLU(
-    x, weight, bias, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg
+    x, weight, bias, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg,
+    segment: ConfigurableArg
 ):
+    """y = fp16(max(x * weight[c] + bias[c], 0)).
+
+    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (4, 8 or 16), `blocks` = workgroups, `segment` =
+    walk of the stream (1 interleaved, 4 / 8 contiguous chunks per thread); 0 = the library's choice.
+    `l1_cache_bytes` is accepted for compatibility and not used: the reference sized its blocks with it."""
     num_channels = x.shape[1]
     assert x.ndim == 5
     assert num_channels == next_power_of_2(num_channels)
@@ -28,15 +36,18 @@ def ApplyBNReLU(
     bias = bias.to(torch.float32).contiguous()
     output = torch.empty_like(x)
     _lib.call('kerops_bnrelu_fwd_f16', x.data_ptr(), weight.data_ptr(), bias.data_ptr(), output.data_ptr(),
-              numel_no_channels(x), num_channels, int(blocks), _lib.stream_of(x))
+              numel_no_channels(x), num_channels, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
     return output
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=8, blocks=0)
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('ApplyBNReLUBackward', 'num_warps'),
+           blocks=stream_knob('ApplyBNReLUBackward', 'blocks'), segment=stream_knob('ApplyBNReLUBackward', 'segment'))
 def ApplyBNReLUBackward(
-    x, weight, bias, grad, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg
+    x, weight, bias, grad, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blocks: ConfigurableArg,
+    segment: ConfigurableArg
 ):
-    """Returns (dx fp16, weight_grad fp32, bias_grad fp32); the two gradients keep weight's shape."""
+    """Returns (dx fp16, weight_grad fp32, bias_grad fp32); the two gradients keep weight's shape.
+    Launch knobs as for ApplyBNReLU (`l1_cache_bytes` accepted, not used)."""
     num_channels = x.shape[1]
     assert x.ndim == 5
     assert x.shape == grad.shape
@@ -58,5 +69,5 @@ def ApplyBNReLUBackward(
     ws = _lib.workspace(ws_bytes, x.device)
     _lib.call('kerops_bnrelu_bwd_f16', x.data_ptr(), wflat.data_ptr(), bflat.data_ptr(), grad.data_ptr(),
               outgrad.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(), m, num_channels, ws.data_ptr(),
-              ws_bytes, int(blocks), _lib.stream_of(x))
+              ws_bytes, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
     return outgrad, weight_grad, bias_grad

@@ -12,6 +12,7 @@ import torch
 
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
+from ..settings.stream_table import stream_knob
 from ._common import require_cuda
 
 
@@ -22,30 +23,37 @@ def _dense(x):
     )
 
 
-@configure(num_warps=4, l1_cache_bytes=get_l1_cache, blocks=0)
+@configure(num_warps=stream_knob('QuantUint8Window', 'num_warps'), l1_cache_bytes=get_l1_cache,
+           blocks=stream_knob('QuantUint8Window', 'blocks'), segment=stream_knob('QuantUint8Window', 'segment'))
 def QuantUint8Window(x, window, *, num_warps: ConfigurableArg, l1_cache_bytes: ConfigurableArg,
-                     blocks: ConfigurableArg):
-    """u8 = trunc((clip(x, -window, window) + window) / (2*window) * 255), fp32 arithmetic."""
+                     blocks: ConfigurableArg, segment: ConfigurableArg):
+    """u8 = trunc((clip(x, -window, window) + window) / (2*window) * 255), fp32 arithmetic; x fp16, bf16 or fp32.
+
+    Launch knobs: `num_warps` = wavefronts per workgroup (4, 8, 16), `blocks` = workgroups, `segment` = walk of the
+    stream (1 interleaved, 4 / 8 contiguous pieces per thread); 0 = the library's choice.  `l1_cache_bytes` is
+    accepted and not used."""
     require_cuda(x)
     assert x.dtype in _lib.DTYPE_TAGS, 'fp16, bf16 or fp32 input'
     assert _dense(x)
     output = torch.empty_like(x, dtype=torch.uint8)
     _lib.call('kerops_quant_u8_window', x.data_ptr(), _lib.DTYPE_TAGS[x.dtype], output.data_ptr(), x.numel(),
-              float(window), int(blocks), _lib.stream_of(x))
+              float(window), int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
     return output
 
 
-@configure(num_warps=4, l1_cache_bytes=get_l1_cache, blocks=0)
+@configure(num_warps=stream_knob('DequantUint8Window', 'num_warps'), l1_cache_bytes=get_l1_cache,
+           blocks=stream_knob('DequantUint8Window', 'blocks'), segment=stream_knob('DequantUint8Window', 'segment'))
 def DequantUint8Window(x, init_dtype, window, *, num_warps: ConfigurableArg, l1_cache_bytes: ConfigurableArg,
-                       blocks: ConfigurableArg):
-    """x_hat = float(u8) * (2*window/255) - window, stored as `init_dtype`."""
+                       blocks: ConfigurableArg, segment: ConfigurableArg):
+    """x_hat = float(u8) * (2*window/255) - window, stored as `init_dtype` (fp16, bf16 or fp32).
+    Launch knobs as for QuantUint8Window."""
     require_cuda(x)
     assert x.dtype == torch.uint8
     assert init_dtype in _lib.DTYPE_TAGS, 'fp16, bf16 or fp32 output'
     assert _dense(x)
     output = torch.empty_like(x, dtype=init_dtype)
     _lib.call('kerops_dequant_u8_window', x.data_ptr(), output.data_ptr(), _lib.DTYPE_TAGS[init_dtype], x.numel(),
-              float(window), int(blocks), _lib.stream_of(x))
+              float(window), int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
     return output
 
 
@@ -63,8 +71,9 @@ def AbsMax(y, *, blocks: ConfigurableArg):
     return out
 
 
-@configure(blocks=0)
-def QuantInt8Sym(y, absmax=None, *, blocks: ConfigurableArg):
+@configure(blocks=stream_knob('QuantInt8Sym', 'blocks'), num_warps=stream_knob('QuantInt8Sym', 'num_warps'),
+           segment=stream_knob('QuantInt8Sym', 'segment'))
+def QuantInt8Sym(y, absmax=None, *, blocks: ConfigurableArg, num_warps: ConfigurableArg, segment: ConfigurableArg):
     """Symmetric per-tensor int8: scale = absmax/127, q = clamp(rint(y/scale), -127, 127).
 
     Rounding is half-to-even.  `absmax` is a 1-element fp32 device tensor (computed with
@@ -78,5 +87,5 @@ def QuantInt8Sym(y, absmax=None, *, blocks: ConfigurableArg):
     assert absmax.dtype == torch.float32 and absmax.numel() == 1 and absmax.is_cuda
     q = torch.empty_like(y, dtype=torch.int8)
     _lib.call('kerops_quant_i8_sym_f16', y.data_ptr(), absmax.data_ptr(), q.data_ptr(), y.numel(), int(blocks),
-              _lib.stream_of(y))
+              int(num_warps), int(segment), _lib.stream_of(y))
     return q, absmax / 127.0

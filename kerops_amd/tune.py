@@ -1,4 +1,4 @@
-"""Measure the built launch shapes of DWConv / DWConvWGRAD on the GPU at hand and install the winners.
+"""Measure the built launch shapes of the ops on the GPU at hand and install the winners.
 
 The reference ships static per-channel tables tuned for one card (kerops/ops/conv/dwconv.py:10-17,
 kerops/ops/conv/dwconv_wgrad.py:10-22); the tables in kerops_amd/ops/conv were measured on an MI355X at
@@ -7,8 +7,13 @@ kerops/ops/conv/dwconv_wgrad.py:10-22); the tables in kerops_amd/ops/conv were m
     python -m kerops_amd.tune --shape 1 64 350 350 128          # print the timings
     python -m kerops_amd.tune --channels 32 64 --apply          # and reconfigure the ops of this process
 
+    python -m kerops_amd.tune --streams                         # the flat stream ops: (blocks, num_warps, segment)
+    python -m kerops_amd.tune --streams --write                 # ... and rewrite settings/stream_shapes.json
+
 `tune(...)` returns {op: {C: (W_block, D_block, lane_channels, H_chunk, ms)}}; `apply(result)` installs the
 choices through the ops' `reconfigure`, the same mechanism a user of the reference has for overriding its tables.
+`tune_streams(...)` returns {op: (blocks, num_warps, segment, ms)}; `apply_streams(result)` puts them into the live
+table of `kerops_amd.settings.stream_table`, which the stream ops read on every call.
 """
 import argparse
 import math
@@ -93,13 +98,90 @@ def apply(result):
         op.reconfigure(**conf)
 
 
+STREAM_BLOCKS = (256, 512, 768, 1024, 1280, 1536, 2048, 3072, 4096)
+STREAM_SHAPES = ((4, 1), (4, 4), (4, 8), (16, 1), (16, 4), (16, 8))  # (num_warps, segment)
+POOL_SHAPES = ((4, 1), (4, 2), (16, 1), (16, 2))
+
+
+def stream_cases(shape, device='cuda'):
+    """{op name: callable(**knobs)} on synthetic tensors of the given (N, C, H, W, D)."""
+    from .ops.addition import AddStats, AddStatsBackward
+    from .ops.avgpool import ApplyBNReLUAvgPoolCeilStats, AvgPoolCeilStats, AvgPoolCeilStatsBackward
+    from .ops.bnrelu import ApplyBNReLU, ApplyBNReLUBackward
+    from .ops.quantization import DequantUint8Window, QuantInt8Sym, QuantUint8Window
+    from .ops.stats import Stats, StatsBackward
+
+    n, c, h, w, d = shape
+    x = torch.randn(n, h, w, d, c, device=device, dtype=torch.float16).permute(0, 4, 1, 2, 3)
+    y = torch.randn(n, h, w, d, c, device=device, dtype=torch.float16).permute(0, 4, 1, 2, 3)
+    z = torch.empty_like(x)
+    wv = torch.rand(c, device=device) + 0.5
+    bv = torch.randn(c, device=device)
+    q = torch.randint(0, 256, x.shape, device=device, dtype=torch.uint8).permute(0, 2, 3, 4, 1).contiguous().permute(0, 4, 1, 2, 3)
+    amax = torch.full((1,), 5.0, device=device)
+    del z
+    pooled = AvgPoolCeilStats(x)[0]
+    return {
+        'AvgPoolCeilStats': lambda **kw: AvgPoolCeilStats(x, **kw),
+        'ApplyBNReLUAvgPoolCeilStats': lambda **kw: ApplyBNReLUAvgPoolCeilStats(x, wv, bv, **kw),
+        'AvgPoolCeilStatsBackward': lambda **kw: AvgPoolCeilStatsBackward(pooled, wv, bv, pooled, list(x.shape), **kw),
+        'Stats': lambda **kw: Stats(x, **kw),
+        'StatsBackward': lambda **kw: StatsBackward(x, wv, bv, **kw),
+        'AddStats': lambda **kw: AddStats(x, y, **kw),
+        'AddStatsBackward': lambda **kw: AddStatsBackward(x, wv, bv, y, **kw),
+        'ApplyBNReLU': lambda **kw: ApplyBNReLU(x, wv, bv, **kw),
+        'ApplyBNReLUBackward': lambda **kw: ApplyBNReLUBackward(x, wv, bv, y, **kw),
+        'QuantUint8Window': lambda **kw: QuantUint8Window(x, 3.0, **kw),
+        'DequantUint8Window': lambda **kw: DequantUint8Window(q, torch.float16, 3.0, **kw),
+        'QuantInt8Sym': lambda **kw: QuantInt8Sym(x, amax, **kw),
+    }
+
+
+def tune_streams(shape=(1, 64, 350, 350, 128), ops=None, iters=12, warmup=3, device='cuda', verbose=False):
+    """Times every (blocks, num_warps, segment) of the built stream kernels; returns {op: (blocks, warps, segment, ms)}."""
+    result = {}
+    for name, run in stream_cases(shape, device).items():
+        if ops and name not in ops:
+            continue
+        best = None
+        for warps, segment in (POOL_SHAPES if 'AvgPool' in name else STREAM_SHAPES):
+            for blocks in STREAM_BLOCKS:
+                kw = dict(blocks=blocks, num_warps=warps, segment=segment)
+                ms = _time(lambda: run(**kw), iters, warmup)
+                if verbose:
+                    print(f'{name:20s} blocks {blocks:5d} num_warps {warps:2d} segment {segment}: {ms:.4f} ms', flush=True)
+                if best is None or ms < best[3]:
+                    best = (blocks, warps, segment, ms)
+        result[name] = best
+    return result
+
+
+def apply_streams(result, write=False, note=''):
+    from .settings import stream_table
+    for op, (blocks, warps, segment, _) in result.items():
+        stream_table.set_stream_shape(op, blocks=blocks, num_warps=warps, segment=segment)
+    if write:
+        stream_table.save(note=note)
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split('\n')[0])
+    ap.add_argument('--streams', action='store_true', help='tune the flat stream ops instead of the convolution pair')
+    ap.add_argument('--write', action='store_true', help='with --streams: rewrite settings/stream_shapes.json')
+    ap.add_argument('--ops', nargs='*', default=None, help='with --streams: only these ops')
     ap.add_argument('--shape', type=int, nargs=5, default=[1, 64, 350, 350, 128], metavar=('N', 'C', 'H', 'W', 'D'))
     ap.add_argument('--channels', type=int, nargs='*', default=None)
     ap.add_argument('--h-chunks', type=int, nargs='*', default=[0])
     ap.add_argument('--apply', action='store_true')
     args = ap.parse_args()
+    if args.streams:
+        res = tune_streams(tuple(args.shape), ops=args.ops, verbose=True)
+        for op, (blocks, warps, segment, ms) in res.items():
+            print(f'best {op:20s}: blocks={blocks} num_warps={warps} segment={segment}  {ms:.4f} ms')
+        shape = ','.join(str(v) for v in args.shape)
+        apply_streams(res, write=args.write, note=f'measured by kerops_amd.tune --streams at ({shape}) on '
+                                                  f'{torch.cuda.get_device_name(0)}')
+        return
     res = tune(tuple(args.shape), args.channels, tuple(args.h_chunks), verbose=True)
     for op, table in res.items():
         for c, (tw, td, cl, hc, ms) in table.items():

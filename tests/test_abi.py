@@ -47,12 +47,20 @@ def test_argument_validation_needs_no_device():
     assert rc == _lib.KEROPS_E_BADARG
     rc = lib.kerops_dwconv_wgrad_f16(addr, addr, addr, addr, 16, 1, 4, 4, 4, 64, 0, 0, 0, 0, None)
     assert rc == _lib.KEROPS_E_WORKSPACE
-    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 1024, addr, 1 << 30, 0, None)
+    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 1024, addr, 1 << 30, 0, 0, 0, None)
     assert rc == _lib.KEROPS_E_UNSUPPORTED_C
-    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 12, addr, 1 << 30, 0, None)
+    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 12, addr, 1 << 30, 0, 0, 0, None)
     assert rc == _lib.KEROPS_E_BADARG
-    rc = lib.kerops_quant_u8_window(addr, 7, addr, 16, 1.0, 0, None)
+    rc = lib.kerops_quant_u8_window(addr, 7, addr, 16, 1.0, 0, 0, 0, None)
     assert rc == _lib.KEROPS_E_BADARG and 'dtype' in _lib.last_error()
+    # launch-shape knobs of the stream kernels: wavefronts per workgroup in {4, 8, 16}, segment in {1, 4, 8}
+    for waves, segment, word in [(5, 0, 'waves'), (32, 1, 'waves'), (4, 2, 'segment'), (16, 16, 'segment')]:
+        rc = lib.kerops_bnrelu_fwd_f16(addr, addr, addr, addr, 64, 64, 0, waves, segment, None)
+        assert rc == _lib.KEROPS_E_BADARG and word in _lib.last_error()
+    rc = lib.kerops_bnrelu_fwd_f16(addr, addr, addr, addr, 64, 4, 0, 4, 8, None)  # 8 pieces need 16-byte chunks
+    assert rc == _lib.KEROPS_E_BADARG and 'segment' in _lib.last_error()
+    rc = lib.kerops_stats_f16(addr, addr, addr, 64, 64, addr, 1 << 30, 70000, 0, 0, None)
+    assert rc == _lib.KEROPS_E_BADARG and 'blocks' in _lib.last_error()
 
 
 def test_every_entry_point_rejects_null_pointers_before_touching_the_device():
@@ -87,6 +95,7 @@ def test_extreme_sizes_never_reach_a_launch():
 def test_workspace_queries():
     lib = _lib.load()
     assert lib.kerops_stats_workspace_bytes(1000, 64, 16) == 16 * 2 * 64 * 4
+    assert lib.kerops_stats_workspace_bytes(1000, 64, 0) == 4096 * 2 * 64 * 4  # covers every built-in shape
     assert lib.kerops_stats_workspace_bytes(1000, 24, 16) == _lib.KEROPS_E_BADARG
     n = lib.kerops_dwconv_wgrad_workspace_bytes(1, 350, 350, 128, 64, 0, 0, 0, 0)
     assert n > 0 and n % (27 * 64 * 4) == 0  # one [27][64] fp32 partial per workgroup

@@ -137,3 +137,39 @@ def test_tuner_apply_installs_and_falls_back():
             shape = (conf['W_block'], conf['D_block'], conf['lane_channels'])
             assert shape in table[c], (op, c, shape)
             assert conf['num_warps'] * 64 == threads_per_workgroup(c, *shape)
+
+
+def test_stream_table_feeds_the_stream_ops_live():
+    """The launch shapes of the stream ops come from settings/stream_shapes.json through zero-argument
+    configurators: the ops see a changed table on their next call, an op missing from the table gets zeros
+    (the library's built-in choice)."""
+    from kerops_amd.ops.bnrelu import ApplyBNReLU
+    from kerops_amd.settings import stream_table
+
+    table = stream_table.load()
+    assert set(table['ApplyBNReLU']) == {'blocks', 'num_warps', 'segment'}
+    for op, entry in table.items():
+        assert entry['num_warps'] in (0, 4, 8, 16) and entry['segment'] in (0, 1, 2, 4, 8) and 0 <= entry['blocks'] <= 65536
+    knob = ApplyBNReLU.configurators['num_warps']
+    assert callable(knob) and knob() == table['ApplyBNReLU']['num_warps']
+    saved = stream_table.stream_shape('ApplyBNReLU')
+    try:
+        stream_table.set_stream_shape('ApplyBNReLU', blocks=7, num_warps=4, segment=1)
+        assert ApplyBNReLU.configurators['blocks']() == 7 and ApplyBNReLU.configurators['segment']() == 1
+    finally:
+        stream_table.set_stream_shape('ApplyBNReLU', **saved)
+    assert stream_table.stream_shape('NoSuchOp') == {'blocks': 0, 'num_warps': 0, 'segment': 0}
+    assert stream_table.stream_knob('NoSuchOp', 'blocks')() == 0
+
+
+def test_stream_table_round_trips_through_its_file(tmp_path):
+    from kerops_amd.settings import stream_table
+
+    before = {op: dict(e) for op, e in stream_table.load().items()}
+    path = str(tmp_path / 'shapes.json')
+    try:
+        stream_table.set_stream_shape('Stats', blocks=123, num_warps=16, segment=8)
+        stream_table.save(path, note='test')
+        assert stream_table.load(path)['Stats'] == {'blocks': 123, 'num_warps': 16, 'segment': 8}
+    finally:
+        assert stream_table.load() == before
