@@ -43,6 +43,16 @@ __device__ __forceinline__ void split_operands(const uint32_t (&r)[4], half4_t& 
     even = __builtin_bit_cast(half4_t, e);
     odd = __builtin_bit_cast(half4_t, o);
 }
+// the same with per-lane byte selectors (0x05040100 / 0x07060302 for live lanes): a lane whose results are never
+// used passes 0x0c0c0c0c twice and gets all-zero operands, so that its share of the multipliers does not toggle
+__device__ __forceinline__ void split_operands_sel(const uint32_t (&r)[4], uint32_t sel_even, uint32_t sel_odd,
+                                                   half4_t& even, half4_t& odd)
+{
+    const u32x2_t e = {__builtin_amdgcn_perm(r[1], r[0], sel_even), __builtin_amdgcn_perm(r[3], r[2], sel_even)};
+    const u32x2_t o = {__builtin_amdgcn_perm(r[1], r[0], sel_odd), __builtin_amdgcn_perm(r[3], r[2], sel_odd)};
+    even = __builtin_bit_cast(half4_t, e);
+    odd = __builtin_bit_cast(half4_t, o);
+}
 // same with three positions; the fourth operand element is zero (selector byte 0x0c yields 0x00)
 __device__ __forceinline__ void split_operands3(const uint32_t (&r)[3], half4_t& even, half4_t& odd)
 {

@@ -617,7 +617,11 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     // They are unconditional (plane indices are clamped; planes that do not exist are never used):
     // the compiler's wait-count bookkeeping is exact only on branch-free paths.
     // (the fused pointwise mode has no registers to spare for the second set and runs one plane ahead)
-    constexpr int AHEAD = MODE == 2 ? 1 : 2;
+    // Planes in flight per workgroup: measured at (1,C,350,350,128), one plane ahead is faster with 8 and with 64
+    // channels per slab (C = 8: 4 % for the plain kernel, 10 % with the statistics; C = 64, 128: 1 %), two planes
+    // ahead with 16 and 32 (1-2 %), and three are slower everywhere: more planes in flight spread the workgroups
+    // of a group further apart, and the halo lines they share leave the L2 before the neighbour asks for them.
+    constexpr int AHEAD = MODE == 2 ? 1 : (SC == 8 || (SC == 64 && MODE != 3)) ? 1 : 2;
     half8_t xpre0[NLDX], xpre1[NLDX];
     auto prefetch = [&](int hp, half8_t(&xpre)[NLDX]) {
         const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
@@ -626,8 +630,8 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     };
 
     int parity = 0;
-    auto step = [&](int hp, half8_t(&xpre)[NLDX]) {
-        const bool xin = (hp >= 0) && (hp < H);  // wavefront-uniform
+    auto step = [&](int hp, half8_t(&xpre)[NLDX], bool live) {
+        const bool xin = live && (hp >= 0) && (hp < H);  // wavefront-uniform
         unsigned char* xbuf = smem + parity * XSLOT;
 #pragma unroll
         for (int j = 0; j < NLDX; ++j) {
@@ -660,8 +664,9 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
         }
         // register 2 of every tile is the finished output plane hp-1
         const int ho = hp - 1;
-        pending_row = (ho >= hs) ? ho : -1;
-        if (ho >= hs) {  // workgroup-uniform
+        const bool finished = live && (ho >= hs);
+        pending_row = finished ? ho : -1;
+        if (finished) {  // workgroup-uniform
             unsigned char* otile = smem + OT_OFF + parity * OT_BYTES;
             half_t* tt = reinterpret_cast<half_t*>(smem + T_OFF);
 #pragma unroll
@@ -743,14 +748,18 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     };
 
     prefetch(hs - 1, xpre0);
-    if (AHEAD == 2) prefetch(hs, xpre1);
+    if (AHEAD >= 2) prefetch(hs, xpre1);
     __syncthreads();  // the one-off zero fill is complete before staging writes anything
-    for (int hp = hs - 1;;) {
-        step(hp, xpre0);
-        if (++hp > he) break;
-        if (AHEAD == 2) {
-            step(hp, xpre1);
-            if (++hp > he) break;
+    // The steps hp = hs-1 .. he run in groups of AHEAD, one per register set, in a loop whose only exit is at its end:
+    // an exit between two steps would give the loop a second way into its first step, on which the newest set is
+    // the oldest, and the compiler's wait before that step's staging writes would cover every load in flight.  A
+    // count that does not divide ends with steps that stage planes nobody reads, compute and store nothing.
+    if constexpr (AHEAD == 1) {
+        for (int hp = hs - 1; hp <= he; ++hp) step(hp, xpre0, true);
+    } else {
+        for (int hp = hs - 1; hp <= he; hp += 2) {
+            step(hp, xpre0, true);
+            step(hp + 1, xpre1, hp + 1 <= he);
         }
     }
     if constexpr (BOUNCE) {

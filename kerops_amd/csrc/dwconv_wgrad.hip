@@ -363,6 +363,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
     const int b = lane / 4, rr = lane % 4;
     const int q = b % NQ, sub = b / NQ;
     const int r2 = min(rr, 2);  // index 3 repeats index 2: its results are never used
+    // ... and its operands are made zero by the byte selectors of the operand split: the quarter of the multipliers
+    // that works for index 3 of either operand then does not toggle (measured: 1738 -> 1765 MHz sustained core clock
+    // under this kernel and 2.5 % less time; the kernel follows the core clock, which the power management lowers
+    // under matrix-core load)
+    const uint32_t sel_e = rr < 3 ? 0x05040100u : 0x0c0c0c0cu, sel_o = rr < 3 ? 0x07060302u : 0x0c0c0c0cu;
     const int cb = half * 64 + q * 4;
     const int pgrp = (gd * NSUB + sub) * 4;  // first position of the lane's group inside a row
     int aoff[4], boff[4];
@@ -488,8 +493,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
 
         int parity = 0;
         // step hp: x plane hp meets the g planes hp+1 (kh = 0), hp (kh = 1), hp-1 (kh = 2)
-        auto step = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG]) {
-            const bool xin = (hp >= 0) && (hp < H);  // wavefront-uniform
+        auto step = [&](int hp, half8_t(&xpre)[NLDX], half8_t(&gpre)[NLDG], bool live) {
+            const bool xin = live && (hp >= 0) && (hp < H);  // wavefront-uniform
             const bool gin = hp + 1 < he;
             unsigned char* xbuf = smem + Cfg::XOFF + parity * XSLOT;
             unsigned char* gslot = smem + ((hp + 1) & 3) * GSLOT;
@@ -518,14 +523,14 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
     #pragma unroll
                         for (int k = 0; k < 4; ++k)
                             r[k] = *reinterpret_cast<const uint32_t*>(smem + go + boff[k] + xr * TD * PB);
-                        split_operands(r, G[xr][0], G[xr][1]);
+                        split_operands_sel(r, sel_e, sel_o, G[xr][0], G[xr][1]);
                     }
                     uint32_t r[4];
     #pragma unroll
                     for (int k = 0; k < 4; ++k)
                         r[k] = *reinterpret_cast<const uint32_t*>(smem + xo + aoff[k] + xr * PDP * PB);
                     half4_t A[2];
-                    split_operands(r, A[0], A[1]);
+                    split_operands_sel(r, sel_e, sel_o, A[0], A[1]);
     #pragma unroll
                     for (int kw = 0; kw < 3; ++kw) {
                         // x patch row ra-1+xr meets g row ra+xr-kw at tap kw
@@ -544,11 +549,13 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
         prefetch(hs - 1, xpre0, gpre0);
         prefetch(hs, xpre1, gpre1);
         __syncthreads();  // the one-off zero fill is complete before staging writes anything
-        for (int hp = hs - 1;;) {
-            step(hp, xpre0, gpre0);
-            if (++hp > he) break;
-            step(hp, xpre1, gpre1);
-            if (++hp > he) break;
+        // The steps hp = hs-1 .. he run in pairs, one per register set, in a loop whose only exit is at its end: an
+        // exit between the two steps would give the loop a second way into its first step, on which the newer set
+        // is the older one, and the compiler's wait before that step's staging writes would cover both sets.  An odd
+        // count ends with a step that stages planes nobody reads and computes nothing.
+        for (int hp = hs - 1; hp <= he; hp += 2) {
+            step(hp, xpre0, gpre0, true);
+            step(hp + 1, xpre1, gpre1, hp + 1 <= he);
         }
     }  // segments
 
@@ -630,7 +637,7 @@ struct BsCfg {
 };
 
 template <class Cfg>
-__global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_split_kernel(const WgArgs a)
+__global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
@@ -817,8 +824,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
     #pragma unroll
                 for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-            auto step = [&](int p, half8_t& xpre, half8_t& gpre) {
-                const bool gin = (p >= 0) && (p < H) && (p <= he);
+            auto step = [&](int p, half8_t& xpre, half8_t& gpre, bool live) {
+                const bool gin = live && (p >= 0) && (p < H) && (p <= he);
                 unsigned char* gslot = smem + (p & 3) * GSLOT;
                 stage(p, xpre, gpre);
                 __syncthreads();
@@ -845,7 +852,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
                     }
                 }
                 const int ho = p - 1;  // dx plane p-1 is complete
-                const bool store = (ho >= hs) && (ho < he);
+                const bool store = live && (ho >= hs) && (ho < he);
                 pending_row = store ? ho : -1;
                 if (store) {
                     unsigned char* otile = smem + Cfg::OT_OFF + parity * Cfg::OT_BYTES;
@@ -867,11 +874,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
                     }
                 parity ^= 1;
             };
-            for (int p = hs - 1;;) {
-                step(p, xpre0, gpre0);
-                if (++p > he + 1) break;
-                step(p, xpre1, gpre1);
-                if (++p > he + 1) break;
+            // pairs of steps, one per register set, and a single exit (see dwconv_wgrad_mfma_kernel); both roles run
+            // the same number of steps, so their barriers match
+            for (int p = hs - 1; p <= he + 1; p += 2) {
+                step(p, xpre0, gpre0, true);
+                step(p + 1, xpre1, gpre1, p + 1 <= he + 1);
             }
             __syncthreads();  // the last tile is written, every wavefront is done with the staging buffers
             flush_row(parity ^ 1);
@@ -888,9 +895,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
 #pragma unroll
             for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-        auto step = [&](int p, half8_t& xpre, half8_t& gpre) {
+        bool lane_used = true;  // index 3 of the operands is never used: its g operand is masked to zero
+        auto step = [&](int p, half8_t& xpre, half8_t& gpre, bool live) {
             const int xq = p - 1;
-            const bool xin = (xq >= 0) && (xq < H) && (xq >= hs - 1) && (xq <= he);
+            const bool xin = live && (xq >= 0) && (xq < H) && (xq >= hs - 1) && (xq <= he);
             const unsigned char* xbuf = smem + Cfg::XOFF + parity * SLOT;
             stage(p, xpre, gpre);
             __syncthreads();
@@ -898,7 +906,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
             __builtin_amdgcn_sched_barrier(0);
             if (xin) {
                 const int gp = p - r2s;  // the lane's g plane; planes of other chunks are masked
-                const uint32_t gmask = (gp >= hs && gp < he) ? 0xffffffffu : 0u;
+                const uint32_t gmask = (gp >= hs && gp < he && lane_used) ? 0xffffffffu : 0u;
                 const int gso = (gp & 3) * GSLOT;
                 half4_t G[RO][2];
 #pragma unroll
@@ -936,6 +944,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
                 const int qq = bb % NQ, ss = bb / NQ;
                 const int cbs = half * 64 + qq * 4, pg = (gd * NSUB + ss) * 4;
                 r2s = min(ln % 4, 2);
+                lane_used = ln % 4 < 3;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     aoff[k] = lds_swizzle<PB>(ra * PDP + pg + r2s + k, cbs);
@@ -946,11 +955,9 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::CG == 8 ? 1 : 4) void dwconv_bwd_spli
             prefetch(hs - 1, xpre0, gpre0);
             prefetch(hs, xpre1, gpre1);
             __syncthreads();  // the zero fill is complete before staging writes anything
-            for (int p = hs - 1;;) {
-                step(p, xpre0, gpre0);
-                if (++p > he + 1) break;
-                step(p, xpre1, gpre1);
-                if (++p > he + 1) break;
+            for (int p = hs - 1; p <= he + 1; p += 2) {
+                step(p, xpre0, gpre0, true);
+                step(p + 1, xpre1, gpre1, p + 1 <= he + 1);
             }
             __syncthreads();  // (the other role: the last tile is written); the staging buffers are free
         }
