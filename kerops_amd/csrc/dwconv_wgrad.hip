@@ -453,12 +453,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
         // volume load the plane's first chunk and write it to the dump slot
         uint32_t xgo[NLDX], ggo[NLDG];
         int xls[NLDX], gls[NLDG];
+        typedef HaloOrder<Cfg::TW, TD, CG> Order;  // chunks shared with neighbouring patches first, interior last
     #pragma unroll
         for (int j = 0; j < NLDX; ++j) {
             const int ch = t + j * NT;
-            const int wq = ch / ((TD + 2) * CG);
-            const int rem = ch - wq * ((TD + 2) * CG);
-            const int dq = rem / CG, cq = rem - dq * CG;
+            int wq, dq, cq;
+            Order::decode(ch, wq, dq, cq);
             const int w = w0 - 1 + wq, d = d0 - 1 + dq;
             const bool ok = (ch < Cfg::NXCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
             xgo[j] = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
@@ -485,7 +485,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
             const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
             const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(hp + 1, hs), he - 1) * plane_stride);
     #pragma unroll
-            for (int j = 0; j < NLDX; ++j) xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
+            for (int j = 0; j < NLDX; ++j) {
+                if (SC > 8 && Order::interior_only(j * NT))  // nobody else reads these chunks: they need not stay in the L2
+                    xpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(xplane + xgo[j]));
+                else
+                    xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
+            }
     #pragma unroll
             for (int j = 0; j < NLDG; ++j)
                 gpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(gplane + ggo[j]));
