@@ -52,3 +52,8 @@ def from_bits(arr):
 @pytest.fixture(scope='session')
 def golden():
     return np.load(os.path.join(ROOT, 'tests', 'golden', 'hotpath_small.npz'))
+
+
+@pytest.fixture(scope='session')
+def golden_config1():
+    return np.load(os.path.join(ROOT, 'tests', 'golden', 'config1_dwconv.npz'))

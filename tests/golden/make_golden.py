@@ -1,5 +1,6 @@
-"""Writes tests/golden/hotpath_small.npz: inputs and expected outputs for every op of the
-hot path on one small odd-sized case, computed with the torch CPU routines that the
+"""Writes tests/golden/hotpath_small.npz (inputs and expected outputs for every op of the
+hot path on one small odd-sized case) and tests/golden/config1_dwconv.npz (the CPU-runnable
+DWConv configuration, x (1,8,64,64,32)), computed with the torch CPU routines that the
 reference's own tests use as ground truth (tests/ops/test_conv.py:25,62-72,
 test_stats.py:13-16, test_bn_relu.py:18-30, test_avgpool.py:12-16 of the reference).
 
@@ -73,6 +74,27 @@ def main():
 
     np.savez_compressed(os.path.join(HERE, 'hotpath_small.npz'), **out)
     print('wrote', os.path.join(HERE, 'hotpath_small.npz'))
+    config1()
+
+
+def config1():
+    """x fp16 channels_last_3d (1,8,64,64,32) ~ N(0,1), depthwise weight (8,1,3,3,3) ~ N(0,1/27), padding 1,
+    stride 1, no bias: conv3d(groups=C) in fp32 on the CPU, output cast to fp16.  The weight gradient is taken by
+    fp64 autograd against the upstream gradient grad = x flipped along H, W and D (N(0,1) as well, and derivable
+    from x, which keeps the file to x, the weight and the two results)."""
+    g = torch.Generator('cpu').manual_seed(322)
+    n, c, h, w, d = 1, 8, 64, 64, 32
+    x = torch.randn(n, c, h, w, d, generator=g).half()
+    wt = (torch.randn(c, 1, 3, 3, 3, generator=g) / math.sqrt(27)).half()
+    out = {'x': bits(x), 'weight_c13x3x3': bits(wt)}
+    y32 = F.conv3d(x.float(), wt.float(), None, stride=1, padding=1, groups=c)
+    out['dwconv_y'] = bits(y32.half())
+    grad = torch.flip(x, dims=(2, 3, 4))
+    w64 = wt.double().clone().requires_grad_(True)
+    F.conv3d(x.double(), w64, None, stride=1, padding=1, groups=c).backward(grad.double())
+    out['dwconv_wgrad_f64'] = w64.grad[:, 0].permute(1, 2, 3, 0).contiguous().numpy()
+    np.savez_compressed(os.path.join(HERE, 'config1_dwconv.npz'), **out)
+    print('wrote', os.path.join(HERE, 'config1_dwconv.npz'))
 
 
 if __name__ == '__main__':

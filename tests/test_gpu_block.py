@@ -168,9 +168,18 @@ def test_lin_brelu_lin_backward_matches_oracle(c, spatial):
     rdx, rup, rdn, rdb = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
     assert dx.shape == x.shape and dx.stride() == x.stride()
     assert dup.shape == (c, 2 * c) and ddn.shape == (2 * c, c) and db.shape == (2 * c,)
-    # fp32 MFMA sums vs the oracle's fp64: an intermediate fp16 value may round (or its ReLU mask flip at a
-    # linup within one rounding of zero) differently once in a while
-    assert (dx.float() - rdx.float()).abs().max() <= 2.0 ** -7 * max(1.0, rdx.abs().max().item())
+    # fp32 MFMA sums vs the oracle's fp64: an intermediate fp16 value may round differently once in a while, and where
+    # a hidden pre-activation lies within a rounding of zero its ReLU mask may flip.  The reference's test rechecks
+    # such voxels by hand (tests/ops/test_linear.py:203-219); here the error a flip can cause is bounded per voxel:
+    # sum over the hidden units next to zero of |Wdown g|_j * |Wup[ci, j]|.
+    x2, g2 = (t_.permute(0, 2, 3, 4, 1).reshape(-1, c).double() for t_ in (x, grad))
+    linup = x2 @ Wup.double() + bias.double()
+    near = (linup.abs() < 4e-3).double()
+    flip_bound = ((near * (g2 @ Wdown.double().t()).abs()) @ Wup.double().abs().t()).float()
+    flip_bound = flip_bound.reshape(n, h, w, d, c).permute(0, 4, 1, 2, 3)
+    err = (dx.float() - rdx.float()).abs()
+    assert (err <= 2.0 ** -7 * max(1.0, rdx.abs().max().item()) + 1.01 * flip_bound).all()
+    kink = (near.sum(dim=1) > 0).reshape(n, 1, h, w, d).expand_as(dx)
     same = (dx.contiguous().view(torch.int16) == rdx.contiguous().view(torch.int16)).float().mean().item()
     assert same > 0.97, same
     for got, ref in ((dup, rup), (ddn, rdn), (db, rdb)):
@@ -180,7 +189,8 @@ def test_lin_brelu_lin_backward_matches_oracle(c, spatial):
     assert weight_grad_similarity(rdn.float(), ddn, rtol_cos=1e-4, atol_cos=1e-4, rtol_len=1e-3, atol_len=1e-3)
     assert weight_grad_similarity(rup.float(), dup, rtol_cos=1e-4, atol_cos=1e-4, rtol_len=2e-3, atol_len=1e-3)
     assert weight_grad_similarity(rdb.float(), db, rtol_cos=1e-3, atol_cos=1e-3, rtol_len=2e-3, atol_len=1e-3)
-    assert allclose_two_stage(rdx.contiguous(), dx.contiguous(), rtol_strict=1e-4, atol_strict=1e-3,
+    keep = (~kink).to(dx.dtype)  # voxels away from every kink: the reference's criterion without its manual recheck
+    assert allclose_two_stage((rdx * keep).contiguous(), (dx * keep).contiguous(), rtol_strict=1e-4, atol_strict=1e-3,
                               rtol_narrow=1e-3, atol_narrow=4e-3)
 
 
@@ -241,7 +251,12 @@ def _spatial_sample(n, seed, max_voxels=200_000):
     return out
 
 
-@pytest.mark.parametrize('spatial', _spatial_sample(12, seed=322))
+# batch 4 with the largest extents of the reference's grid, listed because a bounded random sample rarely holds them
+FORCED_SPATIAL = [(4, 111, 128, 2), (4, 128, 111, 3), (4, 2, 111, 128), (4, 3, 128, 111), (4, 128, 2, 111),
+                  (4, 128, 128, 2)]
+
+
+@pytest.mark.parametrize('spatial', _spatial_sample(50, seed=322) + FORCED_SPATIAL)
 @pytest.mark.parametrize('cout', [16, 32])
 def test_linear_family_on_reference_fixture_grid_sample(cout, spatial):
     # the reference's parameters: 32 input channels, channels_out in {16, 32} (tests/ops/test_linear.py:11-78) and

@@ -81,6 +81,23 @@ def test_oracle_against_golden(golden):
     assert torch.allclose(ps, torch.from_numpy(golden['avgpool_sqmean_f64']), rtol=1e-6, atol=1e-7)
 
 
+def test_oracle_against_config1_fixture(golden_config1):
+    """The CPU-runnable DWConv configuration, x (1,8,64,64,32): the oracle against the committed torch results."""
+    x = from_bits(golden_config1['x']).to(memory_format=torch.channels_last_3d)
+    wk = from_bits(golden_config1['weight_c13x3x3'])[:, 0].permute(1, 2, 3, 0).contiguous()
+    gold = from_bits(golden_config1['dwconv_y'])
+    for wide in (True, False):
+        y16 = oracle.dwconv_fwd(x, wk, wide=wide)
+        assert torch.allclose(y16.float(), gold.float(), rtol=1e-2, atol=1e-2)  # the configuration's tolerance
+        # torch rounded an fp32 sum, the oracle an fp64 (wide) or fp32 one: equal but for sums next to an fp16 tie
+        same = (y16.contiguous().view(torch.int16) == gold.view(torch.int16)).float().mean().item()
+        assert same >= 0.999, same
+        assert (y16.float() - gold.float()).abs().max() <= 2.0 ** -10 * max(1.0, gold.abs().max().item())
+    grad = torch.flip(x, dims=(2, 3, 4)).contiguous(memory_format=torch.channels_last_3d)
+    gw = oracle.dwconv_wgrad(x, grad)
+    assert torch.allclose(gw, torch.from_numpy(golden_config1['dwconv_wgrad_f64']), rtol=1e-11, atol=1e-11)
+
+
 # ------------------------------------------------------------------ DWConv forward
 @pytest.mark.parametrize('shape', SHAPES)
 def test_dwconv_fwd_vs_torch(shape):
