@@ -195,7 +195,7 @@ struct PoolDefault {
 };
 constexpr PoolDefault kDefPoolFwd{256, 4, 2};
 constexpr PoolDefault kDefPoolFwdBnRelu{512, 4, 1};
-constexpr PoolDefault kDefPoolBwd{256, 4, 2};
+constexpr PoolDefault kDefPoolBwd{256, 4, 1};
 constexpr int kMaxDefaultBlocks = 4096;  // workspace queries with blocks = 0 size for this many partials
 
 static int pool_plan(const char* op, const PoolDefault& def, int N, int H, int W, int D, int C, int blocks, int waves,

@@ -63,16 +63,18 @@ __device__ __forceinline__ void split_operands3(const uint32_t (&r)[3], half4_t&
 }
 
 constexpr int kWave = 64;
+constexpr int64_t kStreamInteriorMinBytes = 384ll << 20;
 
 // Order in which the 16-byte chunks of a staged plane (a TW x TD patch with its one-voxel halo, CG chunks per
 // position) are shared out to the threads: first the chunks that a neighbouring patch reads as well (the halo
 // ring around the patch and the patch's own border ring), then the interior, which only this workgroup reads.
 // A load instruction whose chunks are all interior carries the streaming hint, so these lines do not push the
 // shared ones out of the L2 before the neighbour has read them (forward kernel at 64 channels: x fetched from
-// memory 1.148 -> 1.108 times, 2.5 % less time; 3 % at 16 channels).  The kernels leave the hint off for 8-channel
-// slabs: the whole (1,8,350,350,128) tensor fits the 256 MB memory-side cache, which streaming loads do not use
-// (34 % more time there).  Runs stay whole lines: full rows of TD + 2 positions, pairs of positions at the sides,
-// TD - 2 positions inside.
+// memory 1.148 -> 1.108 times, 2.5 % less time; 3 % at 16 channels).  Streaming loads do not use the 256 MB
+// memory-side cache either, so the hint is for tensors that cannot stay there anyway: the launchers switch it on
+// above kStreamInteriorMinBytes (with the whole 251 MB (1,8,350,350,128) tensor cached between calls the hint cost
+// 34 %, with the 268 MB input of the fused block 7 %).  Runs stay whole lines: full rows of TD + 2 positions, pairs
+// of positions at the sides, TD - 2 positions inside.
 template <int TW, int TD, int CG>
 struct HaloOrder {
     static constexpr int ROWCH = (TD + 2) * CG;                  // chunks of one staged row

@@ -63,6 +63,7 @@ struct FwdArgs {
     // balanced split (matrix-core kernel, modes 0 and 1): bal_group > 0 switches it on
     uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
     uint32_t n_tiles;                  // tiles in the tensor
+    int stream_interior;               // host side only: selects the kernels built with the streaming hint (NTI)
 };
 
 // Packed weights of one thread: for every weight row kh and every channel j of the lane,
@@ -463,7 +464,7 @@ struct FmCfg {
 // transposed as in pointwise_kernel, a wavefront owns 32 positions x 32 output channels; pw^T sits in LDS), the
 // [positions][COUT] result is bounced through LDS and stored as 16-byte chunks with the running max|y| fused in.
 // One segment of a workgroup's work: the march over the rows [hs, he) of one tile (patch x slab x sample).
-template <class Cfg, int MODE, int COUT>
+template <class Cfg, int MODE, int COUT, bool NTI>
 __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsigned char* smem, float* amax_red,
                                                         uint32_t wg_slot, uint32_t tile, int hs, int he,
                                                         float (&ssum)[2], float (&ssq)[2])
@@ -627,7 +628,8 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
         const char* xplane = reinterpret_cast<const char*>(xn + min(max(hp, 0), H - 1) * plane_stride);
 #pragma unroll
         for (int j = 0; j < NLDX; ++j) {
-            if (SC > 8 && Order::interior_only(j * NT))  // nobody else reads these chunks: they need not stay in the L2
+            // nobody else reads the interior chunks: with the hint they do not push shared lines out of the L2
+            if (NTI && Order::interior_only(j * NT))
                 xpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(xplane + xgo[j]));
             else
                 xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
@@ -797,7 +799,9 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     }
 }
 
-template <class Cfg, int MODE, int COUT = 0>
+// NTI: loads of chunks no other workgroup reads carry the streaming hint (a compile-time choice: a run-time branch
+// next to the loads would make the compiler wait for every load in flight)
+template <class Cfg, int MODE, int COUT = 0, bool NTI = false>
 __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mfma_kernel(const FwdArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
@@ -844,10 +848,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     const uint32_t per_sample = (uint32_t)(a.n_slab * a.n_dt * a.n_wt);
     if constexpr (SEGMENTS) {
         while (segment_walk_next(walk, wg_slot, a.H, a.n_tiles, per_sample, a.n_hc, a.h_chunk, tile, hs, he))
-            dwconv_fwd_mfma_segment<Cfg, MODE, COUT>(a, smem, amax_red, wg_slot, tile, hs, he, ssum, ssq);
+            dwconv_fwd_mfma_segment<Cfg, MODE, COUT, NTI>(a, smem, amax_red, wg_slot, tile, hs, he, ssum, ssq);
     } else {
         segment_walk_next(walk, wg_slot, a.H, a.n_tiles, per_sample, a.n_hc, a.h_chunk, tile, hs, he);
-        dwconv_fwd_mfma_segment<Cfg, MODE, COUT>(a, smem, amax_red, wg_slot, tile, hs, he, ssum, ssq);
+        dwconv_fwd_mfma_segment<Cfg, MODE, COUT, NTI>(a, smem, amax_red, wg_slot, tile, hs, he, ssum, ssq);
     }
     if constexpr (STATS) {
         const int t = threadIdx.x;
@@ -942,6 +946,9 @@ static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t 
     if (a.scale) {
         hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 1>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
                            a);
+    } else if (a.stream_interior) {
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0, 0, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+                           stream, a);
     } else {
         hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
                            a);
@@ -1061,6 +1068,7 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
     a.W = W;
     a.D = D;
     a.C = C;
+    a.stream_interior = (int64_t)N * H * W * D * C * 2 >= kStreamInteriorMinBytes;
     hipStream_t s = (hipStream_t)stream;
     const int cg = C >= 64 ? 8 : C / 8;
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
@@ -1138,6 +1146,7 @@ int dwsep_fused_run(const void* x, const void* wt, const float* scale, const flo
     a.W = W;
     a.D = D;
     a.C = 64;
+    a.stream_interior = (int64_t)N * H * W * D * 64 * 2 >= kStreamInteriorMinBytes;
     int rc = plan_fwd_mfma<8, 8, 8, 512>(a, N, 0);
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
@@ -1210,12 +1219,17 @@ extern "C" int kerops_dwconv_stats_f16(const void* x, const void* wt, void* y, f
     a.W = W;
     a.D = D;
     a.C = C;
+    a.stream_interior = (int64_t)N * H * W * D * C * 2 >= kStreamInteriorMinBytes;
     hipStream_t s = (hipStream_t)stream;
     int rc = with_stats_shape(C, [&](auto cg, auto tw, auto td, auto nt) {
         using Cfg = FmCfg<cg(), tw(), td(), nt()>;
         int r = plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0, true, true);
         if (r != KEROPS_OK) return r;
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+        if (a.stream_interior)
+            hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3, 0, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+                               s, a);
+        else
+            hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
         return check_launch("dwconv_stats");
     });
     if (rc != KEROPS_OK) return rc;

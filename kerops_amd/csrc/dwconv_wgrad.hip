@@ -53,6 +53,7 @@ struct WgArgs {
     // balanced split (matrix-core weight-gradient kernel): bal_group > 0 switches it on, see pick_balanced
     uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
     uint32_t n_tiles;                  // tiles in the tensor
+    int stream_interior;               // host side only: selects the kernels built with the streaming hint (NTI)
 };
 
 __device__ __forceinline__ half2_t pack_lo(uint32_t a, uint32_t b)
@@ -344,7 +345,9 @@ struct WmCfg {
     __device__ static constexpr int swz(int p, int cb) { return lds_swizzle<PB>(p, cb); }
 };
 
-template <class Cfg>
+// NTI: loads of x chunks no other workgroup reads carry the streaming hint (a compile-time choice: a run-time branch
+// next to the loads would make the compiler wait for every load in flight)
+template <class Cfg, bool NTI>
 __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_mfma_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
@@ -486,7 +489,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
             const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(hp + 1, hs), he - 1) * plane_stride);
     #pragma unroll
             for (int j = 0; j < NLDX; ++j) {
-                if (SC > 8 && Order::interior_only(j * NT))  // nobody else reads these chunks: they need not stay in the L2
+                // nobody else reads the interior chunks: with the hint they do not push shared lines out of the L2
+                if (NTI && Order::interior_only(j * NT))
                     xpre[j] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(xplane + xgo[j]));
                 else
                     xpre[j] = *reinterpret_cast<const half8_t*>(xplane + xgo[j]);
@@ -1171,7 +1175,8 @@ template <int CG, int TW, int TD, int NT>
 static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
 {
     using Cfg = WmCfg<CG, TW, TD, NT>;
-    return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg>, base, p, gw, stream);
+    if (base.stream_interior) return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg, true>, base, p, gw, stream);
+    return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg, false>, base, p, gw, stream);
 }
 
 // fused backward: one patch shape per channel count, two workgroups of 512 threads per CU
@@ -1277,6 +1282,7 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
     a.W = W;
     a.D = D;
     a.C = C;
+    a.stream_interior = (int64_t)N * H * W * D * C * 2 >= kStreamInteriorMinBytes;
     hipStream_t s = (hipStream_t)stream;
     WgArgs b = a;
     b.n_wt = p.n_wt;
@@ -1342,6 +1348,7 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     a.W = W;
     a.D = D;
     a.C = C;
+    a.stream_interior = (int64_t)N * H * W * D * C * 2 >= kStreamInteriorMinBytes;
     hipStream_t s = (hipStream_t)stream;
     // (channel groups of 8, patch W, patch D, threads)
 #define KEROPS_WG_CASE(CGv, TWv, TDv, NTv)                                 \

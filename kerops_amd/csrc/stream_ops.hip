@@ -447,7 +447,7 @@ namespace {
 struct StreamDefault {
     int blocks, waves, segment;
 };
-constexpr StreamDefault kDefStats{512, 4, 4};
+constexpr StreamDefault kDefStats{256, 4, 8};
 constexpr StreamDefault kDefAddStats{256, 4, 1};
 constexpr StreamDefault kDefStatsBwd{4096, 16, 4};
 constexpr StreamDefault kDefAddStatsBwd{512, 4, 4};
