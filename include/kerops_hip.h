@@ -29,7 +29,7 @@
  *    workgroup count, the wavefronts per workgroup (4, 8 or 16) and the walk: segment
  *    1 = a workgroup's 16-byte chunks are interleaved with the other workgroups',
  *    4 or 8 = every step of a workgroup covers one contiguous run of that many chunks
- *    per thread; the pooling kernels count output chunks and take 1 or 2);
+ *    per thread (with C < 8 a request for 8 runs as 4); the pooling kernels count output chunks and take 1 or 2);
  *    0 selects the built-in choice for gfx950, an unbuilt combination
  *    returns KEROPS_E_BADARG.
  *    For kerops_dwconv_fwd_f16 and kerops_dwconv_wgrad_f16 with the matrix-core

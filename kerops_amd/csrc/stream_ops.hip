@@ -440,7 +440,7 @@ using namespace kerops;
 //   blocks   workgroups of the persistent loop
 //   waves    wavefronts per workgroup: 4, 8 or 16
 //   segment  1 = interleaved walk, 4 or 8 = each workgroup step covers one contiguous run of that many
-//            chunks per thread (8 needs C >= 8)
+//            chunks per thread (with C < 8 a request for 8 runs as 4)
 // Built-in choices: measured on MI355X at (1,64,350,350,128) with `python -m kerops_amd.tune --streams`.
 namespace {
 
@@ -463,13 +463,14 @@ int resolve_shape(const char* op, const StreamDefault& def, int64_t work_items, 
                   int segment, StreamShape* out)
 {
     if (waves == 0) waves = def.waves;
-    if (segment == 0) segment = (def.segment == 8 && !wide8) ? 4 : def.segment;
+    if (segment == 0) segment = def.segment;
+    if (segment == 8 && !wide8) segment = 4;  // narrow chunks (C < 8) are built with four per thread only
     if (!(waves == 4 || waves == 8 || waves == 16)) {
         set_error("%s: waves must be 4, 8 or 16 wavefronts per workgroup (got %d)", op, waves);
         return KEROPS_E_BADARG;
     }
-    if (!(segment == 1 || segment == 4 || (segment == 8 && wide8))) {
-        set_error("%s: segment must be 1 (interleaved), 4 or 8 (8 only with 16-byte chunks; got %d)", op, segment);
+    if (!(segment == 1 || segment == 4 || segment == 8)) {
+        set_error("%s: segment must be 1 (interleaved), 4 or 8 (got %d)", op, segment);
         return KEROPS_E_BADARG;
     }
     out->threads = waves * kWave;

@@ -238,6 +238,46 @@ def test_avgpool_golden(golden):
     assert torch.allclose(sq.cpu().double(), torch.from_numpy(golden['avgpool_sqmean_f64']), atol=1e-6)
 
 
+@pytest.mark.parametrize('shape', [(1, 2, 5, 7, 3), (2, 4, 3, 9, 11), (1, 8, 6, 5, 9), (1, 64, 9, 20, 33)])
+@pytest.mark.parametrize('warps,segment', [(4, 1), (4, 4), (4, 8), (8, 4), (16, 1), (16, 4), (16, 8)])
+def test_every_stream_launch_shape(shape, warps, segment):
+    """Every (wavefronts per workgroup, walk) the stream kernels are built with, at channel counts with narrow
+    (C < 8) and with 16-byte chunks, few and many workgroups: same bits as the oracle whatever the shape."""
+    g = cpu_gen(sum(shape) + warps + segment)
+    c = shape[1]
+    x, y = rand_cl3d(g, *shape), rand_cl3d(g, *shape)
+    xd, yd = x.to(DEV), y.to(DEV)
+    w, b = torch.rand(c, generator=g) + 0.5, torch.randn(c, generator=g) * 0.3
+    mg, sg = torch.randn(c, generator=g) / 3, torch.randn(c, generator=g) / 3
+    for blocks in (1, 5, 300):
+        kw = dict(blocks=blocks, num_warps=warps, segment=segment)
+        mean, sq = Stats(xd, **kw)
+        rm, rs = oracle.stats(x)
+        assert close64(mean, rm) and close64(sq, rs)
+        z, m2, q2 = AddStats(xd, yd, **kw)
+        rz, rm2, rq2 = oracle.add_stats(x, y)
+        assert bits_equal(z, rz) and close64(m2, rm2) and close64(q2, rq2)
+        assert bits_equal(ApplyBNReLU(xd, w.to(DEV), b.to(DEV), **kw), oracle.bnrelu_fwd(x, w, b))
+        dx, dW, dB = ApplyBNReLUBackward(xd, w.to(DEV), b.to(DEV), yd, **kw)
+        rdx, rdW, rdB = oracle.bnrelu_bwd(x, w, b, y)
+        assert bits_equal(dx, rdx) and close64(dW.flatten(), rdW, 1e-5) and close64(dB.flatten(), rdB, 1e-5)
+        assert bits_equal(StatsBackward(xd, mg.to(DEV), sg.to(DEV), **kw), oracle.stats_bwd(x, mg, sg))
+        assert bits_equal(AddStatsBackward(yd, mg.to(DEV), sg.to(DEV), xd, **kw), oracle.add_stats_bwd(y, mg, sg, x))
+        q = QuantUint8Window(xd, 2.5, **kw)
+        assert torch.equal(q.cpu(), oracle.quant_u8_window(x, 2.5))
+        assert bits_equal(DequantUint8Window(q, torch.float16, 2.5, **kw), oracle.dequant_u8_window(q.cpu(), torch.float16, 2.5))
+        qi, _ = QuantInt8Sym(xd, torch.tensor([3.3], device=DEV), **kw)
+        assert torch.equal(qi.cpu(), oracle.quant_i8_sym(x, 3.3))
+    for seg in (1, 2):
+        kw = dict(blocks=7, num_warps=warps, segment=seg)
+        pooled, pm, pq = AvgPoolCeilStats(xd, **kw)
+        rp, rpm, rpq = oracle.avgpool_ceil_stats(x)
+        assert bits_equal(pooled, rp) and close64(pm, rpm) and close64(pq, rpq)
+        gp = rand_cl3d(g, *rp.shape)
+        assert bits_equal(AvgPoolCeilStatsBackward(gp.to(DEV), mg.to(DEV), sg.to(DEV), pooled, list(x.shape), **kw),
+                          oracle.avgpool_ceil_stats_bwd(gp, mg, sg, rp, list(x.shape)))
+
+
 @pytest.mark.parametrize('blocks', [1, 3, 64])
 def test_explicit_block_counts_and_determinism(blocks):
     g = cpu_gen(4)
