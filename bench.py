@@ -37,14 +37,62 @@ HBM_PEAK_GBPS = 8000.0
 H, W, D = 350, 350, 128
 V = H * W * D
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs) at
-# (1,64,350,350,128), each counter scaled by what it reads for a 2 007 040 000-byte device copy
-# (FETCH_SIZE reads 0.5000 of the copied bytes, WRITE_SIZE 1.0000):
-# profiles/dwconv_fwd_wgrad_c64_readme_shape.md.
-MEASURED_TRAFFIC_BYTES = {
-    ('dwconv_fwd', 64): 4339515866,    # 2.332 GB read + 2.007 GB written (1.081 x algorithmic)
-    ('dwconv_wgrad', 64): 4376702479,  # 4.373 GB read + 0.004 GB written (1.090 x algorithmic)
-}
+TRAFFIC_TABLE = os.path.join(ROOT, 'profiles', 'dwconv_hbm_traffic_by_channels.md')
+
+
+def load_traffic_table(path=TRAFFIC_TABLE):
+    """HBM bytes per launch of the two convolution kernels, per channel count, from the committed rocprofv3 summary
+    (rows `| C | kernel | FETCH_SIZE KiB | WRITE_SIZE KiB | HBM bytes | ...`, measured at the commit the file
+    names).  Returns ({(kernel, C): bytes}, commit or None); an unreadable file gives an empty table."""
+    import re
+    table, commit = {}, None
+    try:
+        text = open(path).read()
+    except OSError:
+        return table, commit
+    m = re.search(r'measured at commit `?([0-9a-f]{7,40})`?', text)
+    commit = m.group(1) if m else None
+    for row in re.findall(r'^\|\s*(\d+)\s*\|\s*`?(dwconv_\w+)`?\s*\|[^|]*\|[^|]*\|\s*(\d+)\s*\|', text, flags=re.M):
+        table[(row[1], int(row[0]))] = int(row[2])
+    return table, commit
+
+
+def clock_under_load(torch, ops, seconds=1.2):
+    """Core clock (MHz) that rocm-smi reports while one op runs back to back for `seconds`: the matrix-core
+    convolution kernels draw enough power for the clock to come down from its 2.4 GHz ceiling, the pure stream
+    kernels do not, and the convolution kernels' time follows the clock.  A reported side figure; None when
+    rocm-smi is not there."""
+    import re
+    import subprocess
+    import threading
+    out = {}
+    for name, fn in ops.items():
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                try:
+                    r = subprocess.run(['rocm-smi', '--showclocks', '--json'], capture_output=True, text=True, timeout=5)
+                    m = re.search(r'"sclk clock speed:":\s*"\((\d+)Mhz\)"', r.stdout)
+                    if m:
+                        samples.append(int(m.group(1)))
+                except Exception:
+                    return
+        th = threading.Thread(target=sampler, daemon=True)
+        t0 = time.perf_counter()
+        n = 0
+        th.start()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(40):
+                fn()
+            torch.cuda.synchronize()
+            n += 40
+        ms = (time.perf_counter() - t0) * 1e3 / n
+        stop.set()
+        th.join(timeout=6)
+        body = samples[1:] if len(samples) > 2 else samples  # the first sample may predate the load
+        out[name] = {'sclk_mhz': median(body) if body else None, 'samples': len(samples), 'ms_back_to_back': round(ms, 4)}
+    return out
 
 
 def parse():
@@ -55,6 +103,7 @@ def parse():
     ap.add_argument('--channels', type=int, default=64, help='C of the timed step (README table: 8..128)')
     ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the CPU legs (used under rocprofv3)')
     ap.add_argument('--no-extra-ops', action='store_true', help='time only the DWConv step')
+    ap.add_argument('--no-clock-probe', action='store_true', help='skip the core-clock-under-load side figure')
     return ap.parse_args()
 
 
@@ -206,13 +255,17 @@ def main():
     wg = figures(median(wg_ts), nbytes, clone_gbps)
     wg['ms_avg'], wg['ms_min'] = round(wg_avg, 4), round(min(wg_ts), 4)
 
+    traffic_table, traffic_commit = load_traffic_table()
+    traffic_note = (f'HBM bytes per launch from profiles/dwconv_hbm_traffic_by_channels.md (rocprofv3 FETCH_SIZE + '
+                    f'WRITE_SIZE, measured at commit {traffic_commit})' if traffic_table else
+                    'null: profiles/dwconv_hbm_traffic_by_channels.md is missing or holds no row for this channel count')
     dom_name, dom_avg = ('dwconv_wgrad', wg_avg) if wg_avg >= fwd_avg else ('dwconv_fwd', fwd_avg)
     achieved = nbytes / dom_avg / 1e6
     roofline = {
         'kernel': 'kerops::' + dom_name + '_mfma_kernel',
         'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-        'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': MEASURED_TRAFFIC_BYTES.get((dom_name, C)),
-        'algorithmic_bytes': nbytes, 'avg_launch_ms': round(dom_avg, 4),
+        'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': traffic_table.get((dom_name, C)),
+        'traffic_source': traffic_note, 'algorithmic_bytes': nbytes, 'avg_launch_ms': round(dom_avg, 4),
         'note': 'avg over the timed steps of HIP events around the op on the launch stream; for wgrad the '
                 'launch includes its partial-sum reduce kernel (~1% of the time)',
     }
@@ -221,7 +274,7 @@ def main():
     roofline_other = {
         'kernel': 'kerops::' + other + '_mfma_kernel', 'bound': 'hbm', 'achieved': round(nbytes / other_avg / 1e6, 1),
         'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(nbytes / other_avg / 1e6 / HBM_PEAK_GBPS, 4),
-        'traffic': MEASURED_TRAFFIC_BYTES.get((other, C)), 'algorithmic_bytes': nbytes,
+        'traffic': traffic_table.get((other, C)), 'algorithmic_bytes': nbytes,
         'avg_launch_ms': round(other_avg, 4),
     }
 
@@ -354,6 +407,15 @@ def main():
                                '1x1x1 GEMM with fused max|y|; the 64-channel intermediate never reaches memory')
         ops['readme_table_note'] = 'C=8 (251 MB) fits the 256 MB Infinity Cache: its rows are not pure HBM numbers'
 
+    clocks = None
+    if not args.no_clock_probe:
+        xs, gs, wks = make(C)
+        from kerops_amd.ops.bnrelu import ApplyBNReLU as _bn
+        ones, zeros = torch.ones(C, device=dev), torch.zeros(C, device=dev)
+        clocks = clock_under_load(torch, {'DWConv': lambda: DWConv(xs, wks), 'DWConvWGRAD': lambda: DWConvWGRAD(xs, gs),
+                                          'ApplyBNReLU': lambda: _bn(xs, ones, zeros)})
+        del xs, gs
+
     cpu, cpu_torch = (None, None)
     if not args.no_cpu_baseline:
         cpu, cpu_torch = cpu_baseline(torch, C)
@@ -373,6 +435,7 @@ def main():
         'targets': {'fwd_frac_of_clone>=0.75': fwd['frac_of_clone'] >= 0.75,
                     'wgrad_frac_of_clone>=0.50': wg['frac_of_clone'] >= 0.50},
         'roofline': roofline, 'roofline_other': roofline_other,
+        'core_clock_under_load': clocks,
         'cpu_baseline': cpu, 'cpu_torch_conv3d': cpu_torch, 'ops': ops,
         'device': torch.cuda.get_device_name(0),
     }
