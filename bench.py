@@ -412,8 +412,20 @@ def main():
         xs, gs, wks = make(C)
         from kerops_amd.ops.bnrelu import ApplyBNReLU as _bn
         ones, zeros = torch.ones(C, device=dev), torch.zeros(C, device=dev)
-        clocks = clock_under_load(torch, {'DWConv': lambda: DWConv(xs, wks), 'DWConvWGRAD': lambda: DWConvWGRAD(xs, gs),
-                                          'ApplyBNReLU': lambda: _bn(xs, ones, zeros)})
+        probes = {'DWConv': lambda: DWConv(xs, wks), 'DWConvWGRAD': lambda: DWConvWGRAD(xs, gs),
+                  'ApplyBNReLU': lambda: _bn(xs, ones, zeros)}
+        if not args.no_extra_ops:
+            from kerops_amd.ops.conv import DWConvBackward as _bwd, DWConvStats as _cs
+            from kerops_amd.ops.fused import DWSepBlock as _blk, PointwiseLinear as _pw
+            probes['DWConvStats'] = lambda: _cs(xs, wks)
+            probes['DWConvBackward'] = lambda: _bwd(xs, gs, wks)
+            if C == 64:
+                Wp = (torch.randn(64, 128, device=dev, generator=gen) / 8.0).half()
+                probes['DWSepBlock_64_128'] = lambda: _blk(xs, wks, ones, zeros, Wp)
+                probes['PointwiseLinear_64_128'] = lambda: _pw(xs, Wp)
+        clocks = clock_under_load(torch, probes)
+        clocks['note'] = ('rocm-smi sclk sampled while the op runs back to back on the (1,C,350,350,128) tensor; '
+                          'ceiling 2400 MHz')
         del xs, gs
 
     cpu, cpu_torch = (None, None)
