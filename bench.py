@@ -113,10 +113,17 @@ def median(xs):
 
 
 def time_op(torch, fn, iters, warm):
-    """Median / min of per-launch HIP-event times on torch's current stream."""
+    """Median / min of per-launch HIP-event times on torch's current stream.  Warm-up: at least `warm` launches and
+    at least 30 ms of back-to-back launches, the time the core clock takes to settle after an idle gap (allocations
+    and host work between two ops are such gaps; a 0.15 ms kernel would otherwise be timed on the ramp)."""
+    t0 = time.perf_counter()
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
+    while time.perf_counter() - t0 < 0.03:
+        for _ in range(max(warm, 5)):
+            fn()
+        torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
     for a, b in evs:
         a.record()
