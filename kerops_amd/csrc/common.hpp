@@ -12,6 +12,7 @@
 #include <stdint.h>
 
 #include <cmath>
+#include <type_traits>
 
 #include "../../include/kerops_hip.h"
 
@@ -60,6 +61,16 @@ __device__ __forceinline__ void split_operands3(const uint32_t (&r)[3], half4_t&
     const u32x2_t o = {__builtin_amdgcn_perm(r[1], r[0], 0x07060302u), __builtin_amdgcn_perm(0u, r[2], 0x0c0c0302u)};
     even = __builtin_bit_cast(half4_t, e);
     odd = __builtin_bit_cast(half4_t, o);
+}
+
+// every lane takes the value of the previous lane of its quad (lane 0 that of lane 3): one DPP move per dword
+__device__ __forceinline__ half4_t quad_rotate_up(half4_t v)
+{
+    u32x2_t w = __builtin_bit_cast(u32x2_t, v);
+    // (every lane has a source, so the "old" operand is never kept: passing the source itself lets the move run in place)
+    w[0] = (uint32_t)__builtin_amdgcn_update_dpp((int)w[0], (int)w[0], 0x93, 0xf, 0xf, false);  // quad_perm:[3,0,1,2]
+    w[1] = (uint32_t)__builtin_amdgcn_update_dpp((int)w[1], (int)w[1], 0x93, 0xf, 0xf, false);
+    return __builtin_bit_cast(half4_t, w);
 }
 
 constexpr int kWave = 64;

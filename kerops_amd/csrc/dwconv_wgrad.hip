@@ -613,34 +613,41 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
 // Run separately the two products read g twice (8.8 GB at C=64 with the halos); here a workgroup stages
 // every g plane of its patch once, with halo, into a ring of four LDS slots and uses it twice: as the
 // scattered operand of the forward scheme (weights flipped, accumulator registers = the dx planes
-// p+1, p, p-1 of g plane p) and, through the interior of the slots of the planes p, p-1, p-2, as the
-// lane-indexed operand of the weight-gradient scheme against x plane p-1.  The g planes next to the chunk
-// are real data for dx but belong to other chunks for gw: the lanes that read them there are masked.
+// p+1, p, p-1 of g plane p) and as the window operand of the weight-gradient scheme.  The weight gradient is
+// summed over the x positions of the patch, gw[kh,kw,kd] = sum x[h+kh-1,w,d] * g[h,w-kw+1,d-kd+1] (the same sum
+// with the shifts along W and D moved to g; positions of g outside the volume contribute nothing), so x is read
+// without a halo along W and D: one tensor with halo instead of two.  x planes live in a ring of four patch-sized
+// slots; g plane P is multiplied with the x planes P-1, P, P+1 (lane j takes the slot of plane P+j-1) once plane
+// P+1 of x has arrived.  The g planes next to the chunk are real data for dx but belong to other chunks for gw:
+// those steps are skipped by the weight-gradient role.
 //
 // The two products run on different wavefronts: all 8 wavefronts of a workgroup stage the planes of x and g
-// (with halo) into LDS, then wavefronts 0-3 run the input-gradient scheme (and store dx) while wavefronts 4-7
+// into LDS, then wavefronts 0-3 run the input-gradient scheme (and store dx) while wavefronts 4-7
 // run the weight-gradient scheme on the same LDS data, each role in its own loop with the same sequence of
 // workgroup barriers.  A role keeps only its own accumulators: 123-128 registers and 42-62 KB of LDS, so two
 // workgroups (16 wavefronts) are resident per CU, where running both schemes in every wavefront needs ~190
-// registers and holds 8 wavefronts (that version took 1.55 ms at (1,64,350,350,128), this one 1.42 ms; the
-// two separate kernels 1.54-1.58 ms).  An 8x8 patch with 16 wavefronts re-reads less halo but leaves one
-// workgroup per CU, whose per-plane barriers are then fully exposed: 1.50 ms.
+// registers and holds 8 wavefronts.  An 8x8 patch with 16 wavefronts re-reads less halo but leaves one
+// workgroup per CU, whose per-plane barriers are then fully exposed.
 template <int CG_, int TW_, int TD_, int NT_>
 struct BsCfg {
     static constexpr int CG = CG_, TW = TW_, TD = TD_, NT = NT_, RWAVES = NT_ / 128;  // wavefronts per role
     static constexpr int SC = CG * 8, PB = SC * 2;
     static constexpr int NQ = SC >= 32 ? 16 : SC / 2, NSUB = 16 / NQ, NHALF = SC / (2 * NQ);
     static constexpr int NPART = RWAVES / NHALF, GD = TD / (4 * NSUB), RSPLIT = NPART / GD, RO = TW / RSPLIT;
-    static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, SLOT = R * PDP * PB;
-    static constexpr int GSLOT = SLOT + (SC == 8 ? 16 : 32);  // lanes j read different slots: shift their banks apart
+    static constexpr int R = TW + 2, PDP = (TD + 3 + 3) / 4 * 4, GSLOT = R * PDP * PB;  // a g plane with its halo
+    static constexpr int NPOS = TW * TD;
+    // an x plane of the patch alone; lanes j of the weight-gradient role read different slots: shift their banks apart
+    static constexpr int XSLOT = NPOS * PB + (SC == 8 ? 16 : 32);
     static constexpr int XOFF = 4 * GSLOT;
     // dx leaves through two LDS output tiles as 16-byte chunks (whole lines, one store per thread and plane)
-    static constexpr int NPOS = TW * TD, OT_BYTES = NPOS * PB, OT_OFF = XOFF + 2 * SLOT;
+    static constexpr int OT_BYTES = NPOS * PB, OT_OFF = XOFF + 4 * XSLOT;
     static constexpr int DUMP = OT_OFF + 2 * OT_BYTES, STAGE_BYTES = DUMP + 16;
-    static constexpr int NCH = R * (TD + 2) * CG;  // 16-byte chunks of a staged plane: one per thread, t < NCH
+    static constexpr int NCH = R * (TD + 2) * CG;  // 16-byte chunks of a staged g plane: one per thread, t < NCH
+    static constexpr int NXCH = NPOS * CG;         // ... of a staged x plane: t < NXCH
     static constexpr int RED_BYTES = NPART * 27 * SC * 4;
     static constexpr int LDS_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
-    static_assert(NCH <= NT && RO == 4 && TD % (4 * NSUB) == 0 && NPART % GD == 0 && TW % RSPLIT == 0, "even split");
+    static_assert(NCH <= NT && NXCH <= NT && RO == 4 && TD % (4 * NSUB) == 0 && NPART % GD == 0 && TW % RSPLIT == 0,
+                  "even split");
     static_assert(NPOS * CG == RWAVES * 64, "the dx role stores the tile: one 16-byte chunk per thread");
     static_assert(STAGE_BYTES % 16 == 0, "16-byte chunks");
 };
@@ -649,7 +656,7 @@ template <class Cfg>
 __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
-    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, SLOT = Cfg::SLOT, GSLOT = Cfg::GSLOT;
+    constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, GSLOT = Cfg::GSLOT, XSLOT = Cfg::XSLOT;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
     const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
@@ -692,8 +699,9 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
     const half_t* xn = a.x;
     const half_t* gn_ptr = a.g;
     half_t* dxn = a.dx;
-    uint32_t go = 0;  // staging: thread t owns chunk t of the patch with halo (x and g alike); threads without a
-    int ls = -1;      // chunk inside the volume load the plane's first chunk and write it to the dump slot
+    uint32_t go = 0, xgo = 0;  // staging: thread t owns chunk t of the g patch with halo and chunk t of the x patch;
+    int ls = -1, xls = -1;     // threads without a chunk inside the volume load the plane's first chunk and write
+                               // it to the dump slot
     auto next_segment = [&]() -> bool {  // workgroup-uniform
         uint32_t L;
         for (;;) {
@@ -749,42 +757,55 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
         const bool ok = (ts < Cfg::NCH) && (w >= 0) && (w < W) && (d >= 0) && (d < D);
         go = ok ? (uint32_t)(((w * D + d) * C + cslab + cq * 8) * 2) : 0u;
         ls = ok ? lds_swizzle<PB>(wq * PDP + dq, cq * 16) : -1;
+        // x: the patch alone (the weight gradient is summed over the x positions of the patch against the g
+        // positions around them, so that only one of the two tensors is read with a halo)
+        const int xwq = ts / (TD * CG);
+        const int xrem = ts - xwq * (TD * CG);
+        const int xdq = xrem / CG, xcq = xrem - xdq * CG;
+        const bool xok = (ts < Cfg::NXCH) && (w0 + xwq < W) && (d0 + xdq < D);
+        xgo = xok ? (uint32_t)((((w0 + xwq) * D + d0 + xdq) * C + cslab + xcq * 8) * 2) : 0u;
+        xls = xok ? lds_swizzle<PB>(xwq * TD + xdq, xcq * 16) : -1;
         return true;
     };
 
     // loads run two steps ahead in two register sets; unconditional (clamped plane indices)
     half8_t xpre0, xpre1, gpre0, gpre1;
-    auto prefetch = [&](int p, half8_t& xpre, half8_t& gpre) {  // x plane p-1, g plane p
-        const char* xplane = reinterpret_cast<const char*>(xn + min(max(p - 1, 0), H - 1) * plane_stride);
-        const char* gplane = reinterpret_cast<const char*>(gn_ptr + min(max(p, 0), H - 1) * plane_stride);
-        xpre = *reinterpret_cast<const half8_t*>(xplane + go);
-        gpre = *reinterpret_cast<const half8_t*>(gplane + go);
+    auto prefetch = [&](int p, half8_t& xpre, half8_t& gpre) {  // planes p of x and g
+        const int64_t poff = min(max(p, 0), H - 1) * plane_stride;
+        xpre = *reinterpret_cast<const half8_t*>(reinterpret_cast<const char*>(xn + poff) + xgo);
+        gpre = *reinterpret_cast<const half8_t*>(reinterpret_cast<const char*>(gn_ptr + poff) + go);
     };
-    int parity = 0;
+    int parity = 0;  // output tile in use (input-gradient role)
+    // Planes outside the volume or beyond the chunk arrive as copies of a clamped plane and are staged as they
+    // are: the input-gradient role skips the step of such a g plane, the weight-gradient role never takes a g
+    // plane outside its chunk and zeroes the operand of a lane whose x plane lies outside the volume.
     auto stage = [&](int p, const half8_t& xpre, const half8_t& gpre) {
-        const bool gin = (p >= 0) && (p < H) && (p <= he);  // g plane p exists and is needed (dx)
-        unsigned char* xbuf = smem + Cfg::XOFF + parity * SLOT;
+        unsigned char* xslot = smem + Cfg::XOFF + (p & 3) * XSLOT;
         unsigned char* gslot = smem + (p & 3) * GSLOT;
-        unsigned char* xd = ls >= 0 ? xbuf + ls : smem + Cfg::DUMP;
+        unsigned char* xd = xls >= 0 ? xslot + xls : smem + Cfg::DUMP;
         unsigned char* gdst = ls >= 0 ? gslot + ls : smem + Cfg::DUMP;
         *reinterpret_cast<half8_t*>(xd) = xpre;
-        *reinterpret_cast<half8_t*>(gdst) = gin ? gpre : z8;
+        *reinterpret_cast<half8_t*>(gdst) = gpre;
     };
 
     if (role == 0) {
-        // ---- input gradient: flipped weight operands, lane rr = kh' holds (kd' = 0, 1, 2, -) ----
+        // ---- input gradient: flipped weight operands, (kd' = 0, 1, 2, -) of one kh' per lane.  The four registers
+        // of an accumulator tile form a ring: dx plane h lives in register (h - hs + 1) % 4 for the three steps
+        // that add to it, so nothing is moved between steps.  At step s (g plane p = hs - 1 + s) register i takes
+        // kh' = (s + 1 - i) % 4 (3 = none: zero weights), i.e. every step each lane hands its weights to the next
+        // lane of its quad; a march of 4n steps leaves them where they started. ----
         half4_t wA[3][2];
         {
-            const int rr = lane % 4, c0 = cslab + half * 32 + 2 * ((lane / 4) % NQ);
+            const int r0 = (1 - lane % 4) & 3, c0 = cslab + half * 32 + 2 * ((lane / 4) % NQ);
 #pragma unroll
             for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
                     half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
-                    if (rr < 3) {
+                    if (r0 < 3) {
 #pragma unroll
                         for (int kd = 0; kd < 3; ++kd)
-                            v[kd] = a.wt[(((2 - rr) * 3 + (2 - kw)) * 3 + (2 - kd)) * C + c0 + e];
+                            v[kd] = a.wt[(((2 - r0) * 3 + (2 - kw)) * 3 + (2 - kd)) * C + c0 + e];
                     }
                     wA[kw][e] = v;
                 }
@@ -827,13 +848,14 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
                             o8, reinterpret_cast<half8_t*>(reinterpret_cast<char*>(dxn + pending_row * plane_stride) + ogo));
                 }
             };
-            float4_t T[RO][2];  // dx tiles: registers 0, 1, 2 = planes p+1, p, p-1
+            float4_t T[RO][2];  // dx tiles, four planes in a ring of registers
     #pragma unroll
             for (int o = 0; o < RO; ++o)
     #pragma unroll
                 for (int e = 0; e < 2; ++e) T[o][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-            auto step = [&](int p, half8_t& xpre, half8_t& gpre, bool live) {
+            auto step = [&](auto ring, int p, half8_t& xpre, half8_t& gpre, bool live) {
+                constexpr int DONE = (decltype(ring)::value + 3) & 3;  // register of dx plane p-1, complete after this step
                 const bool gin = live && (p >= 0) && (p < H) && (p <= he);
                 unsigned char* gslot = smem + (p & 3) * GSLOT;
                 stage(p, xpre, gpre);
@@ -860,7 +882,7 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
                         }
                     }
                 }
-                const int ho = p - 1;  // dx plane p-1 is complete
+                const int ho = p - 1;
                 const bool store = live && (ho >= hs) && (ho < he);
                 pending_row = store ? ho : -1;
                 if (store) {
@@ -869,25 +891,29 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
                     for (int o = 0; o < RO; ++o) {
                         half2_t v;
     #pragma unroll
-                        for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][2];
+                        for (int e = 0; e < 2; ++e) v[e] = (half_t)T[o][e][DONE];
                         *reinterpret_cast<half2_t*>(otile + owr[o]) = v;
                     }
                 }
+                // the finished register rests for one step (its lane has zero weights then) and starts its next
+                // plane from zero; the weights move on by one lane
     #pragma unroll
                 for (int o = 0; o < RO; ++o)
     #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        T[o][e][2] = T[o][e][1];
-                        T[o][e][1] = T[o][e][0];
-                        T[o][e][0] = 0.0f;
-                    }
+                    for (int e = 0; e < 2; ++e) T[o][e][DONE] = 0.0f;
+    #pragma unroll
+                for (int kw = 0; kw < 3; ++kw)
+    #pragma unroll
+                    for (int e = 0; e < 2; ++e) wA[kw][e] = quad_rotate_up(wA[kw][e]);
                 parity ^= 1;
             };
-            // pairs of steps, one per register set, and a single exit (see dwconv_wgrad_mfma_kernel); both roles run
-            // the same number of steps, so their barriers match
-            for (int p = hs - 1; p <= he + 1; p += 2) {
-                step(p, xpre0, gpre0, true);
-                step(p + 1, xpre1, gpre1, p + 1 <= he + 1);
+            // groups of four steps (the ring's period), register sets alternating, and a single exit (see
+            // dwconv_wgrad_mfma_kernel); both roles run the same number of steps, so their barriers match
+            for (int p = hs - 1; p <= he + 1; p += 4) {
+                step(std::integral_constant<int, 0>{}, p, xpre0, gpre0, true);
+                step(std::integral_constant<int, 1>{}, p + 1, xpre1, gpre1, p + 1 <= he + 1);
+                step(std::integral_constant<int, 2>{}, p + 2, xpre0, gpre0, p + 2 <= he + 1);
+                step(std::integral_constant<int, 3>{}, p + 3, xpre1, gpre1, p + 3 <= he + 1);
             }
             __syncthreads();  // the last tile is written, every wavefront is done with the staging buffers
             flush_row(parity ^ 1);
@@ -895,8 +921,11 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
         __syncthreads();  // (the other role: staging buffers are dead)
         __syncthreads();  // (the other role: partial sums are in LDS)
     } else {
-        // ---- weight gradient: x windows (patch row ra + xr, positions pgrp + r2 + k) against the interior of
-        // the g slots (patch row ra + 1 + gr, positions pgrp + 1 + k), lane j reads the slot of plane p - j ----
+        // ---- weight gradient, summed over the x positions of the patch: gw[kh][kw][kd] = sum x[P+kh-1][w][d] *
+        // g[P][w-kw+1][d-kd+1].  Operand A (lane i = kd): the window of g plane P, halo row ra + t, that starts kd
+        // positions to the left; operand B (lane j = kh): four positions of x row ra + o in the slot of plane
+        // P + j - 1.  Planes of x next to the chunk are real data, g planes next to it belong to other chunks: the
+        // step with such a P is skipped as a whole. ----
         int aoff[4], boff[4], r2s = 0;  // set per segment (see the other role)
         float4_t acc[3][2];  // one tile per kw: D[i = kd][j = kh]
 #pragma unroll
@@ -904,45 +933,47 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
 #pragma unroll
             for (int e = 0; e < 2; ++e) acc[kw][e] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-        bool lane_used = true;  // index 3 of the operands is never used: its g operand is masked to zero
+        // byte selectors that split a dword pair into the even / odd channel's operand; all-zero operands
+        // (selector 0x0c0c0c0c) for index 3, which no result uses, and for a lane whose x plane is outside the volume
+        uint32_t sel_e = 0x05040100u, sel_o = 0x07060302u;
         auto step = [&](int p, half8_t& xpre, half8_t& gpre, bool live) {
-            const int xq = p - 1;
-            const bool xin = live && (xq >= 0) && (xq < H) && (xq >= hs - 1) && (xq <= he);
-            const unsigned char* xbuf = smem + Cfg::XOFF + parity * SLOT;
+            const int P = p - 1;  // g plane P meets the x planes P-1, P, P+1 = p, the newest one staged
+            const bool on = live && (P >= hs) && (P < he);
             stage(p, xpre, gpre);
             __syncthreads();
             prefetch(p + 2, xpre, gpre);
             __builtin_amdgcn_sched_barrier(0);
-            if (xin) {
-                const int gp = p - r2s;  // the lane's g plane; planes of other chunks are masked
-                const uint32_t gmask = (gp >= hs && gp < he && lane_used) ? 0xffffffffu : 0u;
-                const int gso = (gp & 3) * GSLOT;
-                half4_t G[RO][2];
+            if (on) {
+                const unsigned char* gsl = smem + (P & 3) * GSLOT;
+                const int xp = P - 1 + r2s;  // the lane's x plane
+                const unsigned char* xsl = smem + Cfg::XOFF + (xp & 3) * XSLOT;
+                const bool xv = (unsigned)xp < (unsigned)H;
+                const uint32_t se = xv ? sel_e : 0x0c0c0c0cu, so = xv ? sel_o : 0x0c0c0c0cu;
+                half4_t X[RO][2];
 #pragma unroll
-                for (int xr = 0; xr < RO + 2; ++xr) {
-                    if (xr < RO) {
-                        uint32_t r[4];
-#pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                            r[k] = *reinterpret_cast<const uint32_t*>(smem + gso + boff[k] + xr * PDP * PB) & gmask;
-                        split_operands(r, G[xr][0], G[xr][1]);
-                    }
+                for (int o = 0; o < RO; ++o) {
                     uint32_t r[4];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) r[k] = *reinterpret_cast<const uint32_t*>(xbuf + aoff[k] + xr * PDP * PB);
+                    for (int k = 0; k < 4; ++k) r[k] = *reinterpret_cast<const uint32_t*>(xsl + boff[k] + o * TD * PB);
+                    split_operands_sel(r, se, so, X[o][0], X[o][1]);
+                }
+#pragma unroll
+                for (int tr = 0; tr < RO + 2; ++tr) {
+                    uint32_t r[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) r[k] = *reinterpret_cast<const uint32_t*>(gsl + aoff[k] + tr * PDP * PB);
                     half4_t A[2];
                     split_operands(r, A[0], A[1]);
 #pragma unroll
                     for (int kw = 0; kw < 3; ++kw) {
-                        if (xr - kw >= 0 && xr - kw < RO) {
+                        if (tr + kw - 2 >= 0 && tr + kw - 2 < RO) {
 #pragma unroll
                             for (int e = 0; e < 2; ++e)
-                                acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], G[xr - kw][e], acc[kw][e], 0, 0, 0);
+                                acc[kw][e] = __builtin_amdgcn_mfma_f32_4x4x4f16(A[e], X[tr + kw - 2][e], acc[kw][e], 0, 0, 0);
                         }
                     }
                 }
             }
-            parity ^= 1;
         };
         while (next_segment()) {
             {
@@ -953,20 +984,23 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
                 const int qq = bb % NQ, ss = bb / NQ;
                 const int cbs = half * 64 + qq * 4, pg = (gd * NSUB + ss) * 4;
                 r2s = min(ln % 4, 2);
-                lane_used = ln % 4 < 3;
+                sel_e = ln % 4 < 3 ? 0x05040100u : 0x0c0c0c0cu;
+                sel_o = ln % 4 < 3 ? 0x07060302u : 0x0c0c0c0cu;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    aoff[k] = lds_swizzle<PB>(ra * PDP + pg + r2s + k, cbs);
-                    boff[k] = lds_swizzle<PB>((ra + 1) * PDP + pg + 1 + k, cbs);
+                    aoff[k] = lds_swizzle<PB>(ra * PDP + pg + 2 - r2s + k, cbs);
+                    boff[k] = lds_swizzle<PB>(ra * TD + pg + k, cbs);
                 }
             }
             parity = 0;
             prefetch(hs - 1, xpre0, gpre0);
             prefetch(hs, xpre1, gpre1);
             __syncthreads();  // the zero fill is complete before staging writes anything
-            for (int p = hs - 1; p <= he + 1; p += 2) {
+            for (int p = hs - 1; p <= he + 1; p += 4) {  // four steps per round, as in the other role
                 step(p, xpre0, gpre0, true);
                 step(p + 1, xpre1, gpre1, p + 1 <= he + 1);
+                step(p + 2, xpre0, gpre0, p + 2 <= he + 1);
+                step(p + 3, xpre1, gpre1, p + 3 <= he + 1);
             }
             __syncthreads();  // (the other role: the last tile is written); the staging buffers are free
         }
