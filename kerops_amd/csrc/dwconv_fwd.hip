@@ -537,19 +537,26 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     const int c0 = cslab + half * 32 + 2 * q;  // its first channel
     const int pgrp = (gd * NSUB + sub) * 4;    // first output position of the lane's group inside the patch row
 
-    // weight operands: lane rr = kh holds (kd = 0, 1, 2, -) of tap row (kh, kw) for the even / odd channel
+    // weight operands: (kd = 0, 1, 2, -) of tap row (kh, kw) for the even / odd channel, one kh per lane of a quad.
+    // The four registers of an accumulator tile form a ring: output plane h lives in register (h - hs + 1) % 4 for
+    // the three steps that add to it, so no register is moved between steps.  At step s (x plane hp = hs - 1 + s)
+    // register i takes kh = (s + 1 - i) % 4 (3 = none: zero weights), i.e. every step each lane hands its weights
+    // to the next lane of its quad (one DPP move per dword); a march of 4n steps leaves them where they started.
     half4_t wA[3][2];
+    {
+        const int r0 = (1 - rr) & 3;
 #pragma unroll
-    for (int kw = 0; kw < 3; ++kw)
+        for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
-            if (rr < 3) {
+            for (int e = 0; e < 2; ++e) {
+                half4_t v = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+                if (r0 < 3) {
 #pragma unroll
-                for (int kd = 0; kd < 3; ++kd) v[kd] = a.wt[((rr * 3 + kw) * 3 + kd) * C + c0 + e];
+                    for (int kd = 0; kd < 3; ++kd) v[kd] = a.wt[((r0 * 3 + kw) * 3 + kd) * C + c0 + e];
+                }
+                wA[kw][e] = v;
             }
-            wA[kw][e] = v;
-        }
+    }
     float esc[2] = {1.0f, 1.0f}, esh[2] = {0.0f, 0.0f};
     if (EPI) {
 #pragma unroll
@@ -637,7 +644,8 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     };
 
     int parity = 0;
-    auto step = [&](int hp, half8_t(&xpre)[NLDX], bool live) {
+    auto step = [&](auto ring, int hp, half8_t(&xpre)[NLDX], bool live) {
+        constexpr int DONE = (decltype(ring)::value + 3) & 3;  // register of output plane hp-1, complete after this step
         const bool xin = live && (hp >= 0) && (hp < H);  // wavefront-uniform
         unsigned char* xbuf = smem + parity * XSLOT;
 #pragma unroll
@@ -669,7 +677,7 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
                 }
             }
         }
-        // register 2 of every tile is the finished output plane hp-1
+        // register DONE of every tile is the finished output plane hp-1
         const int ho = hp - 1;
         const bool finished = live && (ho >= hs);
         pending_row = finished ? ho : -1;
@@ -682,7 +690,7 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
                 half2_t v;
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    float f = T[o][e][2];
+                    float f = T[o][e][DONE];
                     if (EPI) f = fmaxf(__builtin_fmaf(f, esc[e], esh[e]), 0.0f);
                     v[e] = (half_t)f;
                 }
@@ -754,30 +762,41 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
                 }
             }
         }
+        // the finished register rests for one step (its lane has zero weights then) and starts its next plane
+        // from zero; the weights move on by one lane
 #pragma unroll
         for (int o = 0; o < RO; ++o)
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                T[o][e][2] = T[o][e][1];
-                T[o][e][1] = T[o][e][0];
-                T[o][e][0] = 0.0f;
-            }
+            for (int e = 0; e < 2; ++e) T[o][e][DONE] = 0.0f;
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) wA[kw][e] = quad_rotate_up(wA[kw][e]);
         parity ^= 1;
     };
 
     prefetch(hs - 1, xpre0);
     if (AHEAD >= 2) prefetch(hs, xpre1);
     __syncthreads();  // the one-off zero fill is complete before staging writes anything
-    // The steps hp = hs-1 .. he run in groups of AHEAD, one per register set, in a loop whose only exit is at its end:
-    // an exit between two steps would give the loop a second way into its first step, on which the newest set is
-    // the oldest, and the compiler's wait before that step's staging writes would cover every load in flight.  A
-    // count that does not divide ends with steps that stage planes nobody reads, compute and store nothing.
+    // The steps hp = hs-1 .. he run in groups of four (the period of the accumulator ring; the register sets
+    // alternate inside a group), in a loop whose only exit is at its end: an exit between two steps would give the
+    // loop a second way into its first step, on which the newest set is the oldest, and the compiler's wait before
+    // that step's staging writes would cover every load in flight.  A count that does not divide ends with steps
+    // that stage planes nobody reads, compute and store nothing.
+    using std::integral_constant;
     if constexpr (AHEAD == 1) {
-        for (int hp = hs - 1; hp <= he; ++hp) step(hp, xpre0, true);
+        for (int hp = hs - 1; hp <= he; hp += 4) {
+            step(integral_constant<int, 0>{}, hp, xpre0, true);
+            step(integral_constant<int, 1>{}, hp + 1, xpre0, hp + 1 <= he);
+            step(integral_constant<int, 2>{}, hp + 2, xpre0, hp + 2 <= he);
+            step(integral_constant<int, 3>{}, hp + 3, xpre0, hp + 3 <= he);
+        }
     } else {
-        for (int hp = hs - 1; hp <= he; hp += 2) {
-            step(hp, xpre0, true);
-            step(hp + 1, xpre1, hp + 1 <= he);
+        for (int hp = hs - 1; hp <= he; hp += 4) {
+            step(integral_constant<int, 0>{}, hp, xpre0, true);
+            step(integral_constant<int, 1>{}, hp + 1, xpre1, hp + 1 <= he);
+            step(integral_constant<int, 2>{}, hp + 2, xpre0, hp + 2 <= he);
+            step(integral_constant<int, 3>{}, hp + 3, xpre1, hp + 3 <= he);
         }
     }
     if constexpr (BOUNCE) {
