@@ -353,3 +353,30 @@ def test_fused_backward_matches_oracle_and_separate_ops(c, shape_hc):
     # determinism
     dx3, gw3 = DWConvBackward(xd, gd, wd, H_chunk=hc, out_dtype=torch.float32)
     assert torch.equal(dx, dx3) and torch.equal(gw, gw3)
+
+
+@pytest.mark.parametrize('c', [8, 64])
+@pytest.mark.parametrize('h', [4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize('hc', [0, 3, 4, 5])
+def test_march_period_of_four_every_step_count(c, h, hc):
+    """The marching kernels run their plane steps in groups of four (the accumulator registers of a tile are a
+    ring of four planes): every residue of the step count mod 4, with chunk borders inside the volume (hc rows per
+    chunk) and without (0: balanced split), for the forward kernel, the statistics mode and the fused backward."""
+    from kerops_amd.ops.conv import DWConvBackward
+    g = cpu_gen(17 * c + 5 * h + hc)
+    x, grad = rand_cl3d(g, 1, c, h, 9, 12), rand_cl3d(g, 1, c, h, 9, 12)
+    _, wk = rand_dw_weight(g, c)
+    xd, gd, wd = x.to(DEV), grad.to(DEV), wk.to(DEV)
+    y = DWConv(xd, wd, H_chunk=hc)
+    check_fwd(x, wk, y)
+    assert torch.equal(y, DWConv(xd, wd))
+    ys, mean, sqmean = DWConvStats(xd, wd)
+    assert torch.equal(ys, y)
+    yf = y.float()
+    assert torch.allclose(mean.cpu(), yf.mean(dim=(0, 2, 3, 4)).cpu(), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(sqmean.cpu(), (yf * yf).mean(dim=(0, 2, 3, 4)).cpu(), rtol=1e-5, atol=1e-6)
+    dx, gw = DWConvBackward(xd, gd, wd, H_chunk=hc, out_dtype=torch.float32)
+    wflip = torch.flip(wk, dims=(0, 1, 2)).contiguous()
+    check_fwd(grad, wflip, dx)
+    ref_gw = oracle.dwconv_wgrad(x, grad)
+    assert ((gw.cpu().double() - ref_gw).norm() / ref_gw.norm()).item() < 2e-6
