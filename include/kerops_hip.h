@@ -59,6 +59,13 @@ extern "C" {
 #define KEROPS_DTYPE_F32 1
 #define KEROPS_DTYPE_BF16 2
 
+/* Version of this interface: bumped whenever an entry point is added or a signature changes, so a
+ * caller built against an older header can detect the mismatch before passing arguments
+ * (kerops_hip_version() of the loaded library must equal the KEROPS_HIP_VERSION it was compiled
+ * against).  100: first interface; 200: launch-shape knobs (waves, segment) on the stream entry points,
+ * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16. */
+#define KEROPS_HIP_VERSION 200
+
 int kerops_hip_version(void);
 const char* kerops_last_error_string(void);
 

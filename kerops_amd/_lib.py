@@ -17,6 +17,9 @@ KEROPS_E_UNSUPPORTED_C = -2
 KEROPS_E_WORKSPACE = -3
 KEROPS_E_LAUNCH = -4
 
+# KEROPS_HIP_VERSION of include/kerops_hip.h that SIGNATURES below mirrors
+HEADER_VERSION = 200
+
 DTYPE_TAGS = {torch.float16: 0, torch.float32: 1, torch.bfloat16: 2}
 
 _p = ctypes.c_void_p
@@ -92,6 +95,12 @@ def load():
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
+        built = lib.kerops_hip_version()
+        if built != HEADER_VERSION:
+            raise RuntimeError(
+                f'{LIB_PATH} reports interface version {built}, this binding was written for {HEADER_VERSION}: '
+                'rebuild the library (python -m kerops_amd.build)'
+            )
         _lib = lib
     return _lib
 

@@ -28,7 +28,7 @@ int check_launch(const char* what)
 
 }  // namespace kerops
 
-extern "C" int kerops_hip_version(void) { return 100; }
+extern "C" int kerops_hip_version(void) { return KEROPS_HIP_VERSION; }
 
 extern "C" const char* kerops_last_error_string(void) { return kerops::g_err; }
 

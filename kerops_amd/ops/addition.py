@@ -8,7 +8,7 @@ import torch
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
 from ..settings.stream_table import stream_knob
-from ._common import next_power_of_2, numel_no_channels, require_cuda
+from ._common import next_power_of_2, numel_no_channels, require_cuda, stream_waves
 
 
 @configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AddStats', 'num_warps'),
@@ -18,9 +18,9 @@ def AddStats(
     segment: ConfigurableArg
 ):
     """Returns (x + y as fp16, mean, sqmean); with inplace=True the sum overwrites x.
-    Launch knobs: `num_warps` = wavefronts per workgroup (4, 8, 16), `blocks` = workgroups, `segment` = walk of the
-    stream (1 interleaved, 4 / 8 contiguous chunks per thread); 0 = the library's choice.  `l1_cache_bytes` is
-    accepted and not used."""
+    Launch knobs: `num_warps` = wavefronts per workgroup (built: 4, 8, 16; any other positive value runs on the
+    nearest built count), `blocks` = workgroups, `segment` = walk of the stream (1 interleaved, 4 / 8 contiguous
+    chunks per thread); 0 = the library's choice.  `l1_cache_bytes` is accepted and not used."""
     num_channels = x.shape[1]
     assert x.shape == y.shape
     assert x.ndim == y.ndim == 5
@@ -37,8 +37,8 @@ def AddStats(
     mean = torch.empty(num_channels, dtype=torch.float32, device=x.device)
     sqmean = torch.empty(num_channels, dtype=torch.float32, device=x.device)
     _lib.call('kerops_add_stats_f16', x.data_ptr(), y.data_ptr(), output.data_ptr(), mean.data_ptr(),
-              sqmean.data_ptr(), m, num_channels, ws.data_ptr(), ws_bytes, int(blocks), int(num_warps), int(segment),
-              _lib.stream_of(x))
+              sqmean.data_ptr(), m, num_channels, ws.data_ptr(), ws_bytes, int(blocks), stream_waves(num_warps),
+              int(segment), _lib.stream_of(x))
     return output, mean, sqmean
 
 
@@ -71,5 +71,5 @@ def AddStatsBackward(
     output_grad = torch.empty_like(add_grad)
     _lib.call('kerops_add_stats_bwd_f16', add_grad.data_ptr(), mean_grad.data_ptr(), sqmean_grad.data_ptr(),
               add_result.data_ptr(), output_grad.data_ptr(), numel_no_channels(add_grad), num_channels, int(blocks),
-              int(num_warps), int(segment), _lib.stream_of(add_grad))
+              stream_waves(num_warps), int(segment), _lib.stream_of(add_grad))
     return output_grad

@@ -11,7 +11,7 @@ import torch
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
 from ..settings.stream_table import stream_knob
-from ._common import next_power_of_2, require_cuda
+from ._common import next_power_of_2, require_cuda, stream_waves
 
 
 @configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AvgPoolCeilStats', 'num_warps'),
@@ -20,8 +20,9 @@ def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: Configura
                      segment: ConfigurableArg):
     """Returns (pooled fp16 (N,C,ceil(H/2),ceil(W/2),ceil(D/2)) channels_last_3d, mean, sqmean).
 
-    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (4, 8 or 16), `blocks` = workgroups, `segment` =
-    pooled chunks per thread and step (1 or 2); 0 = the library's choice.  `l1_cache_bytes` only feeds the
+    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (built: 4, 8, 16; any other positive value, such
+    as the reference's own 2, runs on the nearest built count), `blocks` = workgroups, `segment` = pooled chunks
+    per thread and step (1 or 2); 0 = the library's choice.  `l1_cache_bytes` only feeds the
     reference's row-size assert below."""
     num_channels = x.shape[1]
     input_d = x.shape[-1]
@@ -44,7 +45,7 @@ def AvgPoolCeilStats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: Configura
     ws_bytes = _lib.query('kerops_avgpool_ceil_stats_workspace_bytes', n, h, w, d, num_channels, int(blocks))
     ws = _lib.workspace(ws_bytes, x.device)
     _lib.call('kerops_avgpool_ceil_stats_f16', x.data_ptr(), output.data_ptr(), mean.data_ptr(), sqmean.data_ptr(),
-              n, h, w, d, num_channels, ws.data_ptr(), ws_bytes, int(blocks), int(num_warps), int(segment),
+              n, h, w, d, num_channels, ws.data_ptr(), ws_bytes, int(blocks), stream_waves(num_warps), int(segment),
               _lib.stream_of(x))
     return output, mean, sqmean
 
@@ -76,7 +77,7 @@ def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg, num
     ws = _lib.workspace(ws_bytes, x.device)
     _lib.call('kerops_bnrelu_avgpool_ceil_stats_f16', x.data_ptr(), weight.data_ptr(), bias.data_ptr(),
               output.data_ptr(), mean.data_ptr(), sqmean.data_ptr(), n, h, w, d, num_channels, ws.data_ptr(),
-              ws_bytes, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
+              ws_bytes, int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(x))
     return output, mean, sqmean
 
 
@@ -121,5 +122,5 @@ def AvgPoolCeilStatsBackward(
     sqmeangrad = sqmeangrad.contiguous()
     _lib.call('kerops_avgpool_ceil_stats_bwd_f16', inpgrad.data_ptr(), meangrad.data_ptr(), sqmeangrad.data_ptr(),
               output.data_ptr(), outgrad.data_ptr(), bsize, h_outgrad, w_outgrad, d_outgrad, num_channels,
-              int(blocks), int(num_warps), int(segment), _lib.stream_of(inpgrad))
+              int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(inpgrad))
     return outgrad

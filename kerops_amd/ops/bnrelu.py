@@ -10,7 +10,7 @@ import torch
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
 from ..settings.stream_table import stream_knob
-from ._common import next_power_of_2, numel_no_channels, require_cuda
+from ._common import next_power_of_2, numel_no_channels, require_cuda, stream_waves
 
 
 @configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('ApplyBNReLU', 'num_warps'),
@@ -21,8 +21,9 @@ def ApplyBNReLU(
 ):
     """y = fp16(max(x * weight[c] + bias[c], 0)).
 
-    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (4, 8 or 16), `blocks` = workgroups, `segment` =
-    walk of the stream (1 interleaved, 4 / 8 contiguous chunks per thread); 0 = the library's choice.
+    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (built: 4, 8, 16; any other positive value runs
+    on the nearest built count), `blocks` = workgroups, `segment` = walk of the stream (1 interleaved, 4 / 8
+    contiguous chunks per thread); 0 = the library's choice.
     `l1_cache_bytes` is accepted for compatibility and not used: the reference sized its blocks with it."""
     num_channels = x.shape[1]
     assert x.ndim == 5
@@ -36,7 +37,7 @@ def ApplyBNReLU(
     bias = bias.to(torch.float32).contiguous()
     output = torch.empty_like(x)
     _lib.call('kerops_bnrelu_fwd_f16', x.data_ptr(), weight.data_ptr(), bias.data_ptr(), output.data_ptr(),
-              numel_no_channels(x), num_channels, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
+              numel_no_channels(x), num_channels, int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(x))
     return output
 
 
@@ -69,5 +70,5 @@ def ApplyBNReLUBackward(
     ws = _lib.workspace(ws_bytes, x.device)
     _lib.call('kerops_bnrelu_bwd_f16', x.data_ptr(), wflat.data_ptr(), bflat.data_ptr(), grad.data_ptr(),
               outgrad.data_ptr(), weight_grad.data_ptr(), bias_grad.data_ptr(), m, num_channels, ws.data_ptr(),
-              ws_bytes, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
+              ws_bytes, int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(x))
     return outgrad, weight_grad, bias_grad

@@ -7,7 +7,8 @@ import torch
 
 from ... import _lib
 from ...settings import ConfigurableArg, confexc, configure
-from .._common import cl3d, next_power_of_2, require_cuda
+from .._common import cl3d, nearest_conv_shape, next_power_of_2, require_cuda
+from .variants import FWD_VARIANTS
 
 # gfx950 launch table, keyed by channel count like the reference's `warps` / `dblock`
 # (kerops/ops/conv/dwconv.py:10-17): (wavefronts per workgroup, tile extent along D,
@@ -60,15 +61,15 @@ def DWConv(
 ):
     """y = conv3d(x, weight, padding=1, stride=1, groups=C) with weight laid out [3,3,3,C].
 
-    ACCTYPE / num_warps / D_block keep the reference's names: accumulation is always
-    fp32 ('float16' is accepted and computed in fp32), num_warps is the number of
-    64-wide wavefronts per workgroup (fixed per patch shape in the library: 4, or 8 for the
-    8x8 patch) and D_block the tile
-    extent along D.  W_block (tile extent along W), H_chunk (> 0: rows one workgroup marches
-    over; 0: the balanced split, in which groups of workgroups share out the rows of all
-    patches evenly; -g: that split with groups of g workgroups) and lane_channels (16 =
-    matrix-core kernels, the default; 2 or 4 = vector kernels with that many channels per
-    lane) are additional gfx950 knobs.
+    ACCTYPE / num_warps / D_block keep the reference's names and accept every value the reference accepts
+    (kerops/ops/conv/dwconv.py:10-17,33): accumulation is always fp32 ('float16' is accepted and computed in
+    fp32); num_warps (any positive count) is accepted and not used, because the library fixes the wavefronts per
+    workgroup with the patch shape (4, or 8 for 512-thread patches); D_block (any power of two) is the tile
+    extent along D, and a (W_block, D_block) pair the library is not built with runs on the nearest built patch
+    shape of the same kernel family.  W_block (tile extent along W), H_chunk (> 0: rows one workgroup marches
+    over; 0: the balanced split, in which groups of workgroups share out the rows of all patches evenly; -g:
+    that split with groups of g workgroups) and lane_channels (16 = matrix-core kernels, the default; 2 or 4 =
+    vector kernels with that many channels per lane) are additional gfx950 knobs.
     """
     channels = x.shape[1]
 
@@ -79,7 +80,7 @@ def DWConv(
     assert list(weight.shape) == [3, 3, 3, channels]
     assert D_block == next_power_of_2(D_block)
     {'float32': None, 'float16': None}[ACCTYPE]
-    assert num_warps in (4, 8), 'the gfx950 kernels are built with 4 or 8 wavefronts per workgroup'
+    assert int(num_warps) > 0
     require_cuda(x, weight)
 
     bsize, _, H, W, D = x.shape
@@ -87,8 +88,9 @@ def DWConv(
     output = torch.empty_like(x)
     assert cl3d(output)
 
+    w_block, d_block, lane_c = nearest_conv_shape(FWD_VARIANTS, channels, W_block, D_block, lane_channels)
     _lib.call(
         'kerops_dwconv_fwd_f16', x.data_ptr(), weight.data_ptr(), output.data_ptr(), bsize, H, W, D, channels,
-        int(W_block), int(D_block), int(H_chunk), int(lane_channels), _lib.stream_of(x),
+        w_block, d_block, int(H_chunk), lane_c, _lib.stream_of(x),
     )
     return output

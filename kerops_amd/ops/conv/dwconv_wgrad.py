@@ -9,7 +9,8 @@ import torch
 
 from ... import _lib
 from ...settings import ConfigurableArg, confexc, configure
-from .._common import next_power_of_2, require_cuda
+from .._common import nearest_conv_shape, next_power_of_2, require_cuda
+from .variants import WGRAD_VARIANTS
 
 _WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
 _TILE_D = {8: 32, 16: 16, 32: 16, 64: 8, 128: 8}
@@ -63,6 +64,11 @@ def DWConvWGRAD(
 ):
     """grad_w[kh,kw,kd,c] = sum_{n,h,w,d} grad[n,c,h,w,d] * x[n,c,h+kh-1,w+kw-1,d+kd-1].
 
+    ACCTYPE, num_warps, D_block and ILP accept every value the reference accepts
+    (kerops/ops/conv/dwconv_wgrad.py:10-22,42): accumulation is always fp32; num_warps and ILP (any positive
+    count) are accepted and not used (the library fixes the wavefronts per workgroup with the patch shape, and
+    a workgroup marches over rows of H instead of 2*ILP of them); a (W_block, D_block) pair the library is not
+    built with runs on the nearest built patch shape of the same kernel family.
     H_chunk > 0: rows one workgroup marches over; 0: the balanced split (groups of workgroups share out the
     rows of all patches evenly); -g: that split with groups of g workgroups.  The split fixes the order of the
     fp32 additions: the same call always returns the same bits, different splits differ in the last bits.
@@ -77,11 +83,12 @@ def DWConvWGRAD(
     assert channels == next_power_of_2(channels)
     assert D_block == next_power_of_2(D_block)
     {'float32': None, 'float16': None}[ACCTYPE]
-    assert num_warps in (4, 8), 'the gfx950 kernels are built for 4 or 8 wavefronts per workgroup'
+    assert int(num_warps) > 0 and int(ILP) > 0
     require_cuda(x, grad)
 
     bsize, _, H, W, D = x.shape
-    cfg = (int(W_block), int(D_block), int(H_chunk), int(lane_channels))
+    w_block, d_block, lane_c = nearest_conv_shape(WGRAD_VARIANTS, channels, W_block, D_block, lane_channels)
+    cfg = (w_block, d_block, int(H_chunk), lane_c)
     ws_bytes = _lib.query('kerops_dwconv_wgrad_workspace_bytes', bsize, H, W, D, channels, *cfg)
     ws = _lib.workspace(ws_bytes, x.device)
     grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=torch.float32)

@@ -58,7 +58,10 @@ def ReLULinearBackward(
     assert x.is_contiguous(memory_format=torch.channels_last_3d)
     assert grad.is_contiguous(memory_format=torch.channels_last_3d)
     assert out_channels in _BUILT, 'the MFMA kernel is built for 16, 32, 64 or 128 output channels'
-    assert num_warps == 4 and D_block == 64, 'the gfx950 kernel runs 4 wavefronts on tiles of 64 voxels'
+    # num_warps, D_block and ILP are accepted with any positive value, as in the reference
+    # (kerops/ops/linear/relu_linear_backward.py:20-24), and not used: the gfx950 kernel always runs 4
+    # wavefronts on tiles of 64 voxels
+    assert int(num_warps) > 0 and int(D_block) > 0 and int(ILP) > 0
     require_cuda(x, grad, weight)
 
     weight = weight.contiguous()

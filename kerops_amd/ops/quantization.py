@@ -13,7 +13,7 @@ import torch
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
 from ..settings.stream_table import stream_knob
-from ._common import require_cuda
+from ._common import require_cuda, stream_waves
 
 
 def _dense(x):
@@ -29,15 +29,15 @@ def QuantUint8Window(x, window, *, num_warps: ConfigurableArg, l1_cache_bytes: C
                      blocks: ConfigurableArg, segment: ConfigurableArg):
     """u8 = trunc((clip(x, -window, window) + window) / (2*window) * 255), fp32 arithmetic; x fp16, bf16 or fp32.
 
-    Launch knobs: `num_warps` = wavefronts per workgroup (4, 8, 16), `blocks` = workgroups, `segment` = walk of the
-    stream (1 interleaved, 4 / 8 contiguous pieces per thread); 0 = the library's choice.  `l1_cache_bytes` is
-    accepted and not used."""
+    Launch knobs: `num_warps` = wavefronts per workgroup (built: 4, 8, 16; any other positive value runs on the
+    nearest built count), `blocks` = workgroups, `segment` = walk of the stream (1 interleaved, 4 / 8 contiguous
+    pieces per thread); 0 = the library's choice.  `l1_cache_bytes` is accepted and not used."""
     require_cuda(x)
     assert x.dtype in _lib.DTYPE_TAGS, 'fp16, bf16 or fp32 input'
     assert _dense(x)
     output = torch.empty_like(x, dtype=torch.uint8)
     _lib.call('kerops_quant_u8_window', x.data_ptr(), _lib.DTYPE_TAGS[x.dtype], output.data_ptr(), x.numel(),
-              float(window), int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
+              float(window), int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(x))
     return output
 
 
@@ -53,7 +53,7 @@ def DequantUint8Window(x, init_dtype, window, *, num_warps: ConfigurableArg, l1_
     assert _dense(x)
     output = torch.empty_like(x, dtype=init_dtype)
     _lib.call('kerops_dequant_u8_window', x.data_ptr(), output.data_ptr(), _lib.DTYPE_TAGS[init_dtype], x.numel(),
-              float(window), int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
+              float(window), int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(x))
     return output
 
 
@@ -87,5 +87,5 @@ def QuantInt8Sym(y, absmax=None, *, blocks: ConfigurableArg, num_warps: Configur
     assert absmax.dtype == torch.float32 and absmax.numel() == 1 and absmax.is_cuda
     q = torch.empty_like(y, dtype=torch.int8)
     _lib.call('kerops_quant_i8_sym_f16', y.data_ptr(), absmax.data_ptr(), q.data_ptr(), y.numel(), int(blocks),
-              int(num_warps), int(segment), _lib.stream_of(y))
+              stream_waves(num_warps), int(segment), _lib.stream_of(y))
     return q, absmax / 127.0

@@ -8,7 +8,7 @@ import torch
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
 from ..settings.stream_table import stream_knob
-from ._common import next_power_of_2, numel_no_channels, require_cuda
+from ._common import next_power_of_2, numel_no_channels, require_cuda, stream_waves
 
 
 @configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('Stats', 'num_warps'),
@@ -17,8 +17,9 @@ def Stats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blo
           segment: ConfigurableArg):
     """Returns (mean, sqmean), fp32 [C], over every axis but channels.
 
-    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (4, 8 or 16), `blocks` = workgroups of the
-    persistent loop, `segment` = walk of the stream (1 interleaved, 4 / 8 contiguous chunks per thread);
+    Launch knobs: `num_warps` = 64-wide wavefronts per workgroup (built: 4, 8, 16; any other positive value runs
+    on the nearest built count), `blocks` = workgroups of the persistent loop, `segment` = walk of the stream
+    (1 interleaved, 4 / 8 contiguous chunks per thread);
     0 = the library's choice.  `l1_cache_bytes` keeps the reference's name, is accepted and not used.
     """
     num_channels = x.shape[1]
@@ -34,7 +35,7 @@ def Stats(x, *, l1_cache_bytes: ConfigurableArg, num_warps: ConfigurableArg, blo
     mean = torch.empty(num_channels, dtype=torch.float32, device=x.device)
     sqmean = torch.empty(num_channels, dtype=torch.float32, device=x.device)
     _lib.call('kerops_stats_f16', x.data_ptr(), mean.data_ptr(), sqmean.data_ptr(), m, num_channels, ws.data_ptr(),
-              ws_bytes, int(blocks), int(num_warps), int(segment), _lib.stream_of(x))
+              ws_bytes, int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(x))
     return mean, sqmean
 
 
@@ -57,6 +58,6 @@ def StatsBackward(
     sqmean_grad = sqmean_grad.to(torch.float32).contiguous()
     output_grad = torch.empty_like(x)
     _lib.call('kerops_stats_bwd_f16', x.data_ptr(), mean_grad.data_ptr(), sqmean_grad.data_ptr(),
-              output_grad.data_ptr(), numel_no_channels(x), num_channels, int(blocks), int(num_warps), int(segment),
-              _lib.stream_of(x))
+              output_grad.data_ptr(), numel_no_channels(x), num_channels, int(blocks), stream_waves(num_warps),
+              int(segment), _lib.stream_of(x))
     return output_grad

@@ -22,6 +22,10 @@ def declared_symbols():
     return sorted(set(re.findall(r'\b(kerops_[a-z0-9_]+)\s*\(', text)))
 
 
+def header_version():
+    return int(re.search(r'#define\s+KEROPS_HIP_VERSION\s+(\d+)', open(HEADER).read()).group(1))
+
+
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = declared_symbols()
@@ -30,7 +34,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f'{name} is declared in include/kerops_hip.h but not exported'
     # and the ctypes table binds exactly the declared set
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.kerops_hip_version() >= 100
+    assert lib.kerops_hip_version() == _lib.HEADER_VERSION == header_version()
 
 
 def test_argument_validation_needs_no_device():

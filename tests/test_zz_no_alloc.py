@@ -36,12 +36,18 @@ def test_noalloc_wgrad_matches_workspace_entry_point_twice(c):
     tensors = [(rand_cl3d(gen, *s).to(DEV), rand_cl3d(gen, *s).to(DEV)) for s in shapes]
     outs = [torch.full((3, 3, 3, c), float('nan'), dtype=torch.float32, device=DEV) for _ in shapes]
     refs = [wgrad_workspace(x, g) for x, g in tensors]
+    # one call first: the entry point looks up its device array on its first call on a device
+    wgrad_noalloc(*tensors[1], outs[1])
+    torch.cuda.synchronize()
+    outs[1].fill_(float('nan'))
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]  # the driver's view: would also see a hipMalloc inside the library
     for (x, g), out in zip(tensors, outs):  # back to back on one stream, no allocation in between
         wgrad_noalloc(x, g, out)
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     for (x, g), out, ref in zip(tensors, outs, refs):
         assert torch.equal(out.view(torch.int32), ref.view(torch.int32))  # same kernels, same order: same bits
         gw64 = oracle.dwconv_wgrad(x.cpu(), g.cpu())
