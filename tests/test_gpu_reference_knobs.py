@@ -101,7 +101,7 @@ def test_stream_ops_with_reference_defaults(c):
         b_ = b_ if isinstance(b_, tuple) else (b_,)
         for u, v in zip(a, b_):
             if u.dtype == torch.float32 and not exact_float:
-                assert torch.allclose(u, v, rtol=2e-6, atol=2e-6)
+                assert torch.allclose(u, v, rtol=1e-5, atol=1e-5)  # sums: the addition order follows the launch shape
             else:
                 assert torch.equal(bits(u), bits(v))
 
