@@ -17,6 +17,7 @@
 // one partial [27][slab] to the workspace.  A second kernel adds the partials in a
 // fixed order, so the result is deterministic (no atomics).
 #include "common.hpp"
+#include "dwconv_wgrad.hpp"
 
 namespace kerops {
 
@@ -41,20 +42,6 @@ struct WgCfg {
     static_assert((TD & (TD - 1)) == 0 && TD >= 2, "TD power of two");
 };
 
-struct WgArgs {
-    const half_t* x;
-    const half_t* g;
-    float* ws;
-    const half_t* wt;  // fused backward only: the forward weight [3][3][3][C]
-    half_t* dx;        // fused backward only: the input gradient
-    int H, W, D, C;
-    int n_wt, n_dt, n_hc, n_slab, h_chunk;
-    uint32_t nblocks;
-    // balanced split (matrix-core weight-gradient kernel): bal_group > 0 switches it on, see pick_balanced
-    uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
-    uint32_t n_tiles;                  // tiles in the tensor
-    int stream_interior;               // host side only: selects the kernels built with the streaming hint (NTI)
-};
 
 __device__ __forceinline__ half2_t pack_lo(uint32_t a, uint32_t b)
 {
@@ -1098,14 +1085,15 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     }
     p->cg = C >= 64 ? 8 : C / 8;
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
-        // measured best on MI355X at (1, C, 350, 350, 128): the matrix-core kernels
+        // measured best on MI355X at (1, C, 350, 350, 128): the matrix-core kernels with LDS-direct staging,
+        // 512-thread workgroups on patches of 512 16-byte chunks
         switch (p->cg) {
-            case 1: tile_w = 8; tile_d = 32; break;
-            case 2: tile_w = 8; tile_d = 16; break;
-            case 4: tile_w = 4; tile_d = 16; break;
+            case 1: tile_w = 8; tile_d = 64; break;
+            case 2: tile_w = 8; tile_d = 32; break;
+            case 4: tile_w = 8; tile_d = 16; break;
             default: tile_w = 8; tile_d = 8; break;
         }
-        lane_channels = 16;
+        lane_channels = 32;
     }
     // only the all-zero triple selects the built-in shape; anything else must name a positive patch
     // (checked before the extents are divided by it) and is matched against the built kernels at launch
@@ -1122,12 +1110,13 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     p->n_dt = ceil_div(D, tile_d);
     // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each; every workgroup also leaves one partial
     const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-    const bool big_wg = p->cg == 8 && (tile_w * tile_d >= 64);
+    // matrix-core kernels run 512 threads on patches of 512 or more 16-byte chunks
+    const bool big_wg = lane_channels >= 16 ? tile_w * tile_d * p->cg >= 512 : (p->cg == 8 && tile_w * tile_d >= 64);
     const int slots = big_wg ? 512 : 1024;
     p->bal_group = 0;
     // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups; matrix-core
     // kernels only); > 0: uniform chunks of that many rows
-    if (lane_channels == 16 && h_chunk <= 0) {
+    if (lane_channels >= 16 && h_chunk <= 0) {
         if (h_chunk < 0 && (-h_chunk) % p->n_slab != 0) {
             set_error("dwconv_wgrad: the group size of the balanced split must be a multiple of the slab count %d",
                       p->n_slab);
@@ -1412,6 +1401,26 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
     KEROPS_WM_CASE(8, 8, 8, 512)
     KEROPS_WM_CASE(8, 4, 16, 512)
 #undef KEROPS_WM_CASE
+    // LDS-direct matrix-core kernels: lane_channels 32 (built-in planes ahead), 33 / 34 / 35 = (1,1) / (2,2) / (1,2)
+    if (p.cl >= 32 && p.cl <= 35) {
+        WgArgs b = a;
+        b.n_wt = p.n_wt;
+        b.n_dt = p.n_dt;
+        b.n_hc = p.n_hc;
+        b.n_slab = p.n_slab;
+        b.h_chunk = p.h_chunk;
+        b.nblocks = (uint32_t)p.nblocks;
+        b.bal_group = p.bal_group;
+        b.bal_q = p.bal_q;
+        b.bal_r = p.bal_r;
+        b.n_tiles = p.n_tiles;
+        const int depth = p.cl == 32 ? 0 : p.cl == 33 ? 11 : p.cl == 34 ? 22 : 12;
+        if (launch_wgrad_dma(b, p.cg, p.tile_w, p.tile_d, depth, s) == 0) {
+            rc = check_launch("dwconv_wgrad");
+            if (rc != KEROPS_OK) return rc;
+            return reduce_partials(b.ws, p, p.cg * 8, b.C, gw, s);
+        }
+    }
     set_error("dwconv_wgrad: no kernel built for C=%d tile_w=%d tile_d=%d lane_channels=%d", C, p.tile_w, p.tile_d,
               p.cl);
     return KEROPS_E_BADARG;

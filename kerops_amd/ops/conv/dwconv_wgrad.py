@@ -12,9 +12,13 @@ from ...settings import ConfigurableArg, confexc, configure
 from .._common import nearest_conv_shape, next_power_of_2, require_cuda
 from .variants import WGRAD_VARIANTS
 
-_WAVES = {8: 4, 16: 4, 32: 4, 64: 8, 128: 8}
-_TILE_D = {8: 32, 16: 16, 32: 16, 64: 8, 128: 8}
-_TILE_W = {8: 8, 16: 8, 32: 4, 64: 8, 128: 8}
+# gfx950 launch table, keyed by channel count like the reference's (kerops/ops/conv/dwconv_wgrad.py:10-22):
+# wavefronts per workgroup, tile extents along D and W, kernel family (32 = matrix-core kernel with LDS-direct
+# staging, 16 = matrix-core kernel staged through registers, 2 = vector kernel)
+_WAVES = {8: 8, 16: 8, 32: 8, 64: 8, 128: 8}
+_TILE_D = {8: 64, 16: 32, 32: 16, 64: 8, 128: 8}
+_TILE_W = {8: 8, 16: 8, 32: 8, 64: 8, 128: 8}
+_LANE_C = {8: 32, 16: 32, 32: 32, 64: 32, 128: 32}
 
 
 @confexc(KeyError)
@@ -33,6 +37,11 @@ def wtile(channels):
 
 
 @confexc(KeyError)
+def lanec(channels):
+    return _LANE_C[channels]
+
+
+@confexc(KeyError)
 def ilp(channels):
     # the reference's ILP (2*ILP rows of H per program, kerops/ops/conv/dwconv_wgrad.py:20-22)
     # has no separate meaning here: a workgroup marches over H_chunk rows
@@ -46,7 +55,7 @@ def ilp(channels):
     ILP=lambda x: ilp(x.shape[1]),
     W_block=lambda x: wtile(x.shape[1]),
     H_chunk=0,
-    lane_channels=16,
+    lane_channels=lambda x: lanec(x.shape[1]),
     out_dtype=torch.float16,
 )
 def DWConvWGRAD(

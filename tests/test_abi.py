@@ -142,7 +142,7 @@ def test_split_of_the_h_march():
         assert blocks(1, 350, 350, 128, 64) == 512   # 8 groups of 64 (weight gradient: 4 rows of 16 patches)
         assert blocks(1, 350, 350, 128, 128) == 512  # the same patches in 2 slabs
         assert blocks(1, 128, 128, 128, 64) == 512
-    assert wgrad_blocks(1, 350, 350, 128, 8) in range(960, 1025)
+    assert wgrad_blocks(1, 350, 350, 128, 8) in range(480, 513)  # 512-thread workgroups at every channel count
     assert wgrad_blocks(1, 1, 8, 8, 8) == 1 and stats_blocks(1, 1, 8, 8, 64) == 1 and bwd_blocks(1, 1, 8, 8, 64) == 2
     assert wgrad_blocks(1, 350, 350, 128, 64, 175) == 1408 and bwd_blocks(1, 350, 350, 128, 64, 175) == 2816
     assert wgrad_blocks(1, 350, 350, 128, 64, -32) == 512 and bwd_blocks(1, 350, 350, 128, 64, -32) == 512
