@@ -74,6 +74,52 @@ __device__ __forceinline__ half4_t quad_rotate_up(half4_t v)
 }
 
 constexpr int kWave = 64;
+
+// ---- LDS-direct loads (global_load_lds_dwordx4) with hand-placed waits ------------------------------------
+// The compiler neither sees these memory instructions nor counts them: a kernel that uses them issues the same
+// number of them in every wavefront and step (an instruction whose mask is empty still counts) and waits with
+// wait_loads_in_flight<n>, which returns when all but the newest n vector memory instructions of the wavefront
+// have completed (loads and stores retire in issue order).  M0 is used by nothing else in these kernels.
+// one LDS-direct load of a wavefront: lane l brings the 16 bytes at sbase + voff to LDS address lds_addr + 16*l;
+// lanes outside `mask` do nothing.  sbase, lds_addr and mask are wavefront-uniform (scalar registers).
+template <bool STREAM>
+__device__ __forceinline__ void lds_direct_load16(const void* sbase, uint32_t voff, uint32_t lds_addr, uint64_t mask)
+{
+    uint64_t saved;
+    if (STREAM)
+        asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %2, %1 nt\n\ts_mov_b64 exec, %0"
+                     : "=&s"(saved)
+                     : "s"(sbase), "v"(voff), "s"(lds_addr), "s"(mask)
+                     : "memory");
+    else
+        asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %2, %1\n\ts_mov_b64 exec, %0"
+                     : "=&s"(saved)
+                     : "s"(sbase), "v"(voff), "s"(lds_addr), "s"(mask)
+                     : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_in_flight()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ const char* uniform_ptr(const char* p)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+}
+
+// 16-byte streaming store of the lanes in `mask` to sbase + voff, counted like the loads above
+__device__ __forceinline__ void masked_store16_stream(void* sbase, uint32_t voff, u32x4_t data, uint64_t mask)
+{
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\tglobal_store_dwordx4 %2, %3, %1 nt\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "s"(sbase), "v"(voff), "v"(data), "s"(mask)
+                 : "memory");
+}
 constexpr int64_t kStreamInteriorMinBytes = 384ll << 20;
 
 // Order in which the 16-byte chunks of a staged plane (a TW x TD patch with its one-voxel halo, CG chunks per

@@ -70,37 +70,6 @@ struct WdCfg {
     __device__ static constexpr int rot(int dq) { return PB == 128 ? 64 * ((dq >> 1) & 1) : 0; }
 };
 
-// one LDS-direct load of a wavefront: lane l brings the 16 bytes at sbase + voff to LDS address lds_addr + 16*l;
-// lanes outside `mask` do nothing.  sbase, lds_addr and mask are wavefront-uniform (scalar registers).
-template <bool STREAM>
-__device__ __forceinline__ void lds_direct_load16(const void* sbase, uint32_t voff, uint32_t lds_addr, uint64_t mask)
-{
-    uint64_t saved;
-    if (STREAM)
-        asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
-                     "global_load_lds_dwordx4 %2, %1 nt\n\ts_mov_b64 exec, %0"
-                     : "=&s"(saved)
-                     : "s"(sbase), "v"(voff), "s"(lds_addr), "s"(mask)
-                     : "memory");
-    else
-        asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
-                     "global_load_lds_dwordx4 %2, %1\n\ts_mov_b64 exec, %0"
-                     : "=&s"(saved)
-                     : "s"(sbase), "v"(voff), "s"(lds_addr), "s"(mask)
-                     : "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_loads_in_flight()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ const char* uniform_ptr(const char* p)
-{
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
-}
-
 // NTI: the x chunks that no other workgroup reads (the patch without its border ring) are loaded by instructions
 // of their own that carry the streaming hint, so that they do not push the shared halo lines out of the L2; a
 // compile-time choice made on the host by tensor size (streaming loads bypass the memory-side cache as well)

@@ -36,8 +36,10 @@ def check_fwd(x, wk, y):
     # fp32 accumulation: never more than one fp16 rounding away from the exact sum
     err = (y.float() - ref32).abs()
     assert (err <= 2.0 ** -11 * ref32.abs().clamp(min=2.0 ** -14) * 1.01 + 1e-6).all()
+    # ... and almost always the same fp16 value as the rounded wide sum: the two differ where the fp32 sum's own
+    # error (a few 2^-24 of the largest term) crosses a rounding boundary of fp16, about 0.15 % of the outputs
     same = (y.contiguous().view(torch.int16) == ref16.contiguous().view(torch.int16)).float().mean().item()
-    assert same >= 0.998, same
+    assert same >= 0.998 - 3.0 * math.sqrt(0.002 / y.numel()), same
 
 
 @pytest.mark.parametrize('shape', SHAPES)
@@ -121,7 +123,7 @@ FORCED_GRID = [(4, 64, 111, 128, 2), (4, 128, 128, 111, 3), (4, 64, 2, 111, 128)
                (3, 64, 7, 128, 111), (4, 128, 2, 128, 128)]
 
 
-@pytest.mark.parametrize('shape', fixture_grid_sample(100, [8, 16, 32, 64, 128], 150_000, seed=322) + FORCED_GRID)
+@pytest.mark.parametrize('shape', fixture_grid_sample(500, [8, 16, 32, 64, 128], 150_000, seed=322) + FORCED_GRID)
 def test_reference_fixture_grid_sample(shape):
     g = cpu_gen(sum(shape))
     x, grad = rand_cl3d(g, *shape), rand_cl3d(g, *shape)

@@ -111,7 +111,7 @@ FORCED_GRID = [(4, 32, 111, 128, 2), (4, 16, 128, 111, 3), (4, 8, 2, 111, 128), 
                (4, 4, 128, 128, 13), (3, 64, 111, 111, 3)]
 
 
-@pytest.mark.parametrize('shape', _grid_sample(100, seed=322) + FORCED_GRID)
+@pytest.mark.parametrize('shape', _grid_sample(500, seed=322) + FORCED_GRID)
 def test_stream_ops_on_reference_fixture_grid_sample(shape):
     g = cpu_gen(sum(shape))
     c = shape[1]
