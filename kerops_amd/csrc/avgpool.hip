@@ -240,7 +240,10 @@ static int pool_plan(const char* op, const PoolDefault& def, int N, int H, int W
     *nchunks = (int64_t)N * p->Ho * p->Wo * p->Do * p->CG;
     sh->threads = waves * kWave;
     sh->segment = segment;
-    if (blocks <= 0) blocks = def.blocks;
+    // the built-in workgroup counts were measured on 256 compute units: scale them to the device at hand
+    // (never beyond what a workspace query with blocks = 0 sizes for)
+    if (blocks <= 0)
+        blocks = std::min(kMaxDefaultBlocks, std::max(1, (int)((int64_t)def.blocks * device_geometry().cus / 256)));
     sh->blocks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(*nchunks, (int64_t)sh->threads * segment), blocks));
     return KEROPS_OK;
 }

@@ -166,6 +166,18 @@ struct HaloOrder {
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 
+// ---- device geometry (host) -------------------------------------------------
+// Compute units and accelerator dies (XCDs, each with its own L2) of the current device, read once per device
+// with hipDeviceGetAttribute (core.hip); without a usable device (a workspace query on a machine without a GPU)
+// the MI355X's 256 / 8.  The H-marching kernels size their launch to the workgroups the device holds at once
+// and walk every die's share of the tiles contiguously.
+struct DeviceGeometry {
+    int cus, xcds;
+    // workgroups resident at once: 16 wavefronts per compute unit at the register budget of these kernels
+    int resident_workgroups(int threads) const { return cus * (threads >= 512 ? 2 : 4); }
+};
+DeviceGeometry device_geometry();
+
 // ---- cross-file launchers (defined in dwconv_fwd.hip / pointwise.hip) ----------------
 int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, const float* shift, int32_t N,
                    int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
@@ -248,17 +260,18 @@ static inline BalancedSplit make_balanced(int H, int64_t tiles, int slots, int g
     b.ngroups = (uint32_t)std::min<int64_t>(std::max(1, slots / group), std::max<int64_t>(1, b.units / 2));
     return b;
 }
-static inline double balanced_cost(const BalancedSplit& b, int H, int row_len, int slots, int setup)
+static inline double balanced_cost(const BalancedSplit& b, int H, int row_len, int slots, int setup, int xcds)
 {
     const double share = (double)((b.units + b.ngroups - 1) / b.ngroups);
     const double crossings = share / H;  // expected bundle boundaries inside a share
     const double rows = (double)b.group / row_len;
     // a group larger than the workgroups one XCD holds is spread over several L2s (measured: 2-3 % slower)
-    const double spread = (int)b.group > slots / 8 ? 1.04 : 1.0;
+    const double spread = (int)b.group > slots / xcds ? 1.04 : 1.0;
     return (share + 2 + setup + crossings * 5.0) * (1.0 + 0.1 / rows) * (1.0 + 0.004 * H / share) * spread;
 }
 // slab_mult: the group size must be a multiple of it (kernels that keep per-slab state across bundles)
-static inline BalancedSplit pick_balanced(int H, int64_t tiles, int row_len, int slots, int setup, int slab_mult)
+static inline BalancedSplit pick_balanced(int H, int64_t tiles, int row_len, int slots, int setup, int slab_mult,
+                                          int xcds)
 {
     BalancedSplit best = make_balanced(H, tiles, slots, slab_mult);
     double best_cost = 1e300;
@@ -266,7 +279,7 @@ static inline BalancedSplit pick_balanced(int H, int64_t tiles, int row_len, int
         if (g < 1 || g > slots || g % slab_mult != 0) return;
         if (g >= tiles + row_len && g > slab_mult) return;  // more than a row of idle members
         const BalancedSplit b = make_balanced(H, tiles, slots, (int)g);
-        const double c = balanced_cost(b, H, row_len, slots, setup);
+        const double c = balanced_cost(b, H, row_len, slots, setup, xcds);
         if (c < best_cost) {
             best_cost = c;
             best = b;
@@ -333,22 +346,21 @@ __device__ __forceinline__ bool segment_walk_next(SegmentWalk& s, uint32_t wg, i
     return true;
 }
 
-// The 8 XCDs of the chip receive workgroups round-robin (workgroup b runs on XCD
-// b % 8) and each XCD has a private L2.  remap_xcd turns the hardware workgroup
+// The XCDs of the chip (8 on MI355X; the launchers pass the device's count) receive workgroups round-robin
+// (workgroup b runs on XCD b % n) and each XCD has a private L2.  remap_xcd turns the hardware workgroup
 // index into a logical tile index such that each XCD walks one contiguous range of
 // logical tiles: neighbouring tiles (which share halo voxels) then meet in the same
 // L2 instead of being fetched once per XCD.
-__device__ __forceinline__ uint32_t remap_xcd(uint32_t b, uint32_t nblocks)
+__device__ __forceinline__ uint32_t remap_xcd(uint32_t b, uint32_t nblocks, uint32_t n_xcd)
 {
-    constexpr uint32_t kXcd = 8;
-    uint32_t per = (nblocks + kXcd - 1) / kXcd;  // logical tiles per XCD (last range may be short)
-    uint32_t xcd = b % kXcd;
-    uint32_t idx = b / kXcd;
+    uint32_t per = (nblocks + n_xcd - 1) / n_xcd;  // logical tiles per XCD (last range may be short)
+    uint32_t xcd = b % n_xcd;
+    uint32_t idx = b / n_xcd;
     // ranges [xcd*per, (xcd+1)*per); the tail ranges can exceed nblocks, so the
-    // grid is launched with per*kXcd workgroups and the caller drops ids >= nblocks.
+    // grid is launched with per*n_xcd workgroups and the caller drops ids >= nblocks.
     return xcd * per + idx;
 }
-static inline uint32_t xcd_padded_grid(uint32_t nblocks) { return ((nblocks + 7u) / 8u) * 8u; }
+static inline uint32_t xcd_padded_grid(uint32_t nblocks, uint32_t n_xcd) { return ((nblocks + n_xcd - 1) / n_xcd) * n_xcd; }
 
 // ---- 16-byte chunk access ---------------------------------------------------
 __device__ __forceinline__ half8_t load_c8(const half_t* p) { return *reinterpret_cast<const half8_t*>(p); }

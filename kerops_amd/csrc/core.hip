@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "common.hpp"
 
 namespace kerops {
@@ -24,6 +26,32 @@ int check_launch(const char* what)
         return KEROPS_E_LAUNCH;
     }
     return KEROPS_OK;
+}
+
+DeviceGeometry device_geometry()
+{
+    static std::mutex mutex;
+    static DeviceGeometry known[64];  // cus == 0: not looked up yet
+    const DeviceGeometry fallback{256, 8};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();  // a query without a device must not leave an error behind for the next launch check
+        return fallback;
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (known[dev].cus == 0) {
+        int cus = 0, xcds = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            (void)hipGetLastError();
+            return fallback;
+        }
+        if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, dev) != hipSuccess || xcds <= 0) {
+            (void)hipGetLastError();
+            xcds = cus >= 64 ? cus / 32 : 1;  // a runtime without the attribute: 32 compute units per die
+        }
+        known[dev] = DeviceGeometry{cus, xcds};
+    }
+    return known[dev];
 }
 
 }  // namespace kerops

@@ -63,6 +63,7 @@ struct FwdArgs {
     // balanced split (matrix-core kernel, modes 0 and 1): bal_group > 0 switches it on
     uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
     uint32_t n_tiles;                  // tiles in the tensor
+    uint32_t n_xcd;                    // accelerator dies of the device: the logical workgroup order follows them
     int stream_interior;               // host side only: selects the kernels built with the streaming hint (NTI)
 };
 
@@ -393,7 +394,7 @@ template <class Cfg, bool EPI>
 __global__ __launch_bounds__(Cfg::NT, Cfg::WPE) void dwconv_fwd_kernel(const FwdArgs a)
 {
     __shared__ half8_t lds[2][Cfg::NCH + 1];  // +1: write-only dump slot for lanes with nothing to stage
-    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
+    uint32_t L = remap_xcd(blockIdx.x, a.nblocks, a.n_xcd);
     if (L >= a.nblocks) return;
     // logical order, fastest first: slab, d-tile, w-tile, h-chunk, n
     const int slab = L % a.n_slab;
@@ -844,7 +845,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_fwd_mf
     __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
     __shared__ float amax_red[Cfg::NWAVE];
 
-    const uint32_t wg_slot = remap_xcd(blockIdx.x, a.nblocks);
+    const uint32_t wg_slot = remap_xcd(blockIdx.x, a.nblocks, a.n_xcd);
     if (wg_slot >= a.nblocks) return;
     // mode 3: sums over the lane's channel pair, carried over every segment (all tiles of a workgroup belong to
     // the same slab: the group size of the balanced split is a multiple of the slab count)
@@ -915,14 +916,16 @@ static int plan_fwd_mfma(FwdArgs& a, int N, int h_chunk, bool balanced_ok = fals
     a.n_wt = ceil_div(a.W, TW);
     a.n_dt = ceil_div(a.D, TD);
     a.bal_group = 0;
-    const int slots = NT >= 512 ? 512 : 1024;  // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each
+    const DeviceGeometry geo = device_geometry();
+    a.n_xcd = (uint32_t)geo.xcds;
+    const int slots = geo.resident_workgroups(NT);  // 2 workgroups of 512 threads or 4 of 256 per compute unit
     // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups) for the kernels
     // that support it; > 0: uniform chunks of that many rows
     if (h_chunk < 0 || (h_chunk == 0 && balanced_ok)) {
         const int64_t tiles = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
         const BalancedSplit b = h_chunk < 0 ? make_balanced(a.H, tiles, slots, -h_chunk)
                                             : pick_balanced(a.H, tiles, a.n_dt * a.n_slab, slots, 6,
-                                                            per_slab_state ? a.n_slab : 1);
+                                                            per_slab_state ? a.n_slab : 1, geo.xcds);
         const bool fits = b.units < (1LL << 31) && tiles + b.group < (1LL << 31);  // 32-bit counters in the kernel
         if (!fits && h_chunk < 0) {
             set_error("dwconv_fwd: too many plane steps for the balanced split");
@@ -963,13 +966,13 @@ static int launch_fwd_mfma(const FwdArgs& base, int N, int h_chunk, hipStream_t 
     int rc = plan_fwd_mfma<CG, TW, TD, NT>(a, N, h_chunk, true);
     if (rc != KEROPS_OK) return rc;
     if (a.scale) {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 1>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 1>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, stream,
                            a);
     } else if (a.stream_interior) {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0, 0, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0, 0, true>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0,
                            stream, a);
     } else {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 0>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, stream,
                            a);
     }
     return check_launch("dwconv_fwd");
@@ -1021,11 +1024,13 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
     a.n_slab = a.C / (CG * 8);
     a.n_wt = ceil_div(a.W, TW);
     a.n_dt = ceil_div(a.D, TD);
+    const DeviceGeometry geo = device_geometry();
+    a.n_xcd = (uint32_t)geo.xcds;
     if (h_chunk <= 0) {
-        // enough workgroups to fill 256 CUs several times over, but rows per chunk
+        // enough workgroups to fill the compute units several times over (11 each), but rows per chunk
         // large enough that the two halo planes of a chunk stay a small overhead
         const int64_t per_plane = (int64_t)N * a.n_wt * a.n_dt * a.n_slab;
-        const int want_chunks = (int)std::max<int64_t>(1, ceil_div64(2816, per_plane));
+        const int want_chunks = (int)std::max<int64_t>(1, ceil_div64(11 * geo.cus, per_plane));
         h_chunk = std::max(ceil_div(a.H, want_chunks), std::min(a.H, 24));
     }
     h_chunk = std::min(h_chunk, a.H);
@@ -1039,14 +1044,14 @@ static int launch_fwd(const FwdArgs& base, int N, int h_chunk, hipStream_t strea
     a.nblocks = (uint32_t)nb;
     if (a.scale) {
         if constexpr (CG == 8 && TW == 8 && TD == 8 && CL == 2 && NT == 512) {
-            hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+            hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, true>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0,
                                stream, a);
         } else {
             set_error("dwconv_fwd: the fused affine+ReLU epilogue is built for the 64-channel 8x8 patch only");
             return KEROPS_E_BADARG;
         }
     } else {
-        hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, false>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream,
+        hipLaunchKernelGGL((dwconv_fwd_kernel<Cfg, false>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, stream,
                            a);
     }
     return check_launch("dwconv_fwd");
@@ -1170,9 +1175,9 @@ int dwsep_fused_run(const void* x, const void* wt, const float* scale, const flo
     if (rc != KEROPS_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
     if (Cout == 128) {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 2, 128>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 2, 128>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, s, a);
     } else if (Cout == 64) {
-        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 2, 64>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+        hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 2, 64>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, s, a);
     } else {
         set_error("dwsep_block: the fused kernel is built for Cout in {64,128}");
         return KEROPS_E_UNSUPPORTED_C;
@@ -1245,10 +1250,10 @@ extern "C" int kerops_dwconv_stats_f16(const void* x, const void* wt, void* y, f
         int r = plan_fwd_mfma<cg(), tw(), td(), nt()>(a, N, 0, true, true);
         if (r != KEROPS_OK) return r;
         if (a.stream_interior)
-            hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3, 0, true>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0,
+            hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3, 0, true>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0,
                                s, a);
         else
-            hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3>), dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, s, a);
+            hipLaunchKernelGGL((dwconv_fwd_mfma_kernel<Cfg, 3>), dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, s, a);
         return check_launch("dwconv_stats");
     });
     if (rc != KEROPS_OK) return rc;

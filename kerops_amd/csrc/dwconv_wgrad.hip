@@ -60,7 +60,7 @@ __global__ __launch_bounds__(Cfg::NT, (Cfg::NT >= 512 || Cfg::STRAIGHT) ? 4 : 3)
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
     half8_t* stage = reinterpret_cast<half8_t*>(smem);
 
-    uint32_t L = remap_xcd(blockIdx.x, a.nblocks);
+    uint32_t L = remap_xcd(blockIdx.x, a.nblocks, a.n_xcd);
     if (L >= a.nblocks) return;
     const uint32_t ws_slot = L;
     const int slab = L % a.n_slab;
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 3) void dwconv_wgrad_
     constexpr int NLDX = Cfg::NLDX, NLDG = Cfg::NLDG;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
-    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
+    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks, a.n_xcd);
     if (ws_slot >= a.nblocks) return;
     const int H = a.H, W = a.W, D = a.D, C = a.C;
 
@@ -646,7 +646,7 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RO = Cfg::RO, GSLOT = Cfg::GSLOT, XSLOT = Cfg::XSLOT;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
 
-    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
+    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks, a.n_xcd);
     if (ws_slot >= a.nblocks) return;
     const int t = threadIdx.x;
     const int H = a.H, W = a.W, D = a.D, C = a.C;
@@ -1063,7 +1063,7 @@ __global__ __launch_bounds__(1024) void wgrad_reduce_kernel(const float* __restr
 }
 
 struct WgPlan {
-    int cg, tile_w, tile_d, cl, h_chunk, n_wt, n_dt, n_hc, n_slab;
+    int cg, tile_w, tile_d, cl, h_chunk, n_wt, n_dt, n_hc, n_slab, n_xcd = 8;
     int64_t nblocks;
     uint32_t bal_group = 0, bal_q = 0, bal_r = 0, n_tiles = 0;  // balanced split (bal_group > 0), see pick_balanced
 };
@@ -1112,7 +1112,9 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
     // matrix-core kernels run 512 threads on patches of 512 or more 16-byte chunks
     const bool big_wg = lane_channels >= 16 ? tile_w * tile_d * p->cg >= 512 : (p->cg == 8 && tile_w * tile_d >= 64);
-    const int slots = big_wg ? 512 : 1024;
+    const DeviceGeometry geo = device_geometry();
+    p->n_xcd = geo.xcds;
+    const int slots = geo.resident_workgroups(big_wg ? 512 : 256);
     p->bal_group = 0;
     // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups; matrix-core
     // kernels only); > 0: uniform chunks of that many rows
@@ -1123,7 +1125,8 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
             return KEROPS_E_BADARG;
         }
         const BalancedSplit b = h_chunk < 0 ? make_balanced(H, per_plane, slots, -h_chunk)
-                                            : pick_balanced(H, per_plane, p->n_dt * p->n_slab, slots, 8, p->n_slab);
+                                            : pick_balanced(H, per_plane, p->n_dt * p->n_slab, slots, 8, p->n_slab,
+                                                            geo.xcds);
         const bool fits = b.units < (1LL << 31) && per_plane + b.group < (1LL << 31);  // 32-bit counters in the kernel
         if (!fits && h_chunk < 0) {
             set_error("dwconv_wgrad: too many plane steps for the balanced split");
@@ -1181,7 +1184,8 @@ static int launch_wgrad_cfg(KernelT kernel, const WgArgs& base, const WgPlan& p,
     a.bal_q = p.bal_q;
     a.bal_r = p.bal_r;
     a.n_tiles = p.n_tiles;
-    hipLaunchKernelGGL(kernel, dim3(xcd_padded_grid(a.nblocks)), dim3(Cfg::NT), 0, stream, a);
+    a.n_xcd = (uint32_t)p.n_xcd;
+    hipLaunchKernelGGL(kernel, dim3(xcd_padded_grid(a.nblocks, a.n_xcd)), dim3(Cfg::NT), 0, stream, a);
     int rc = check_launch("dwconv_wgrad");
     if (rc != KEROPS_OK) return rc;
     return reduce_partials(a.ws, p, Cfg::SC, a.C, gw, stream);
@@ -1225,7 +1229,9 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
     p->n_wt = ceil_div(W, p->tile_w);
     p->n_dt = ceil_div(D, p->tile_d);
     const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-    const int slots = 512;  // two workgroups of 512 threads per CU
+    const DeviceGeometry geo = device_geometry();
+    p->n_xcd = geo.xcds;
+    const int slots = geo.resident_workgroups(512);  // two workgroups of 512 threads per compute unit
     p->bal_group = 0;
     // h_chunk 0: balanced split with the group size of the cost model (-g: groups of g workgroups); > 0: uniform
     // chunks of that many rows
@@ -1236,7 +1242,8 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
             return KEROPS_E_BADARG;
         }
         const BalancedSplit b = h_chunk < 0 ? make_balanced(H, per_plane, slots, -h_chunk)
-                                            : pick_balanced(H, per_plane, p->n_dt * p->n_slab, slots, 8, p->n_slab);
+                                            : pick_balanced(H, per_plane, p->n_dt * p->n_slab, slots, 8, p->n_slab,
+                                                            geo.xcds);
         const bool fits = b.units < (1LL << 31) && per_plane + b.group < (1LL << 31);  // 32-bit counters in the kernel
         if (!fits && h_chunk < 0) {
             set_error("dwconv_bwd: too many plane steps for the balanced split");
@@ -1318,10 +1325,11 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
     b.bal_q = p.bal_q;
     b.bal_r = p.bal_r;
     b.n_tiles = p.n_tiles;
+    b.n_xcd = (uint32_t)p.n_xcd;
 #define KEROPS_BS_GO(CGv, TWv, TDv)                                                                                  \
     {                                                                                                                \
         using Cfg = BsCfg<CGv, TWv, TDv, 512>;                                                                       \
-        hipLaunchKernelGGL(dwconv_bwd_split_kernel<Cfg>, dim3(xcd_padded_grid(b.nblocks)), dim3(Cfg::NT), 0, s, b); \
+        hipLaunchKernelGGL(dwconv_bwd_split_kernel<Cfg>, dim3(xcd_padded_grid(b.nblocks, b.n_xcd)), dim3(Cfg::NT), 0, s, b); \
     }
     switch (p.cg) {
         case 1: KEROPS_BS_GO(1, 8, 32) break;
@@ -1414,6 +1422,8 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
         b.bal_q = p.bal_q;
         b.bal_r = p.bal_r;
         b.n_tiles = p.n_tiles;
+        b.n_xcd = (uint32_t)p.n_xcd;
+    b.n_xcd = (uint32_t)p.n_xcd;
         const int depth = p.cl == 32 ? 0 : p.cl == 33 ? 11 : p.cl == 34 ? 22 : 12;
         if (launch_wgrad_dma(b, p.cg, p.tile_w, p.tile_d, depth, s) == 0) {
             rc = check_launch("dwconv_wgrad");

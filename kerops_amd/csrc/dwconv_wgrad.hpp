@@ -17,6 +17,7 @@ struct WgArgs {
     // balanced split (matrix-core weight-gradient kernel): bal_group > 0 switches it on, see pick_balanced
     uint32_t bal_group, bal_q, bal_r;  // workgroups per group; bundles * H plane steps = groups * bal_q + bal_r
     uint32_t n_tiles;                  // tiles in the tensor
+    uint32_t n_xcd;                    // accelerator dies of the device: the logical workgroup order follows them
     int stream_interior;               // host side only: selects the kernels built with the streaming hint (NTI)
 };
 

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 4) void dwconv_wgrad_
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(void __attribute__((address_space(3)))*)smem;
 
-    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks);
+    const uint32_t ws_slot = remap_xcd(blockIdx.x, a.nblocks, a.n_xcd);
     if (ws_slot >= a.nblocks) return;
     const int H = a.H, W = a.W, D = a.D, C = a.C;
 
@@ -322,7 +322,7 @@ template <int CG, int TW, int TD, int NT, int AX, int AG>
 void launch_shape(const WgArgs& a, hipStream_t stream)
 {
     using Cfg = WdCfg<CG, TW, TD, NT, AX, AG>;
-    const dim3 grid(xcd_padded_grid(a.nblocks)), block(Cfg::NT);
+    const dim3 grid(xcd_padded_grid(a.nblocks, a.n_xcd)), block(Cfg::NT);
     if (a.stream_interior)
         hipLaunchKernelGGL((dwconv_wgrad_dma_kernel<Cfg, true>), grid, block, 0, stream, a);
     else

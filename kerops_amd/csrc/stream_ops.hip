@@ -479,7 +479,10 @@ int resolve_shape(const char* op, const StreamDefault& def, int64_t work_items, 
         set_error("%s: blocks must be <= %d", op, kMaxStreamBlocks);
         return KEROPS_E_BADARG;
     }
-    if (blocks <= 0) blocks = def.blocks;
+    // the built-in workgroup counts were measured on 256 compute units: scale them to the device at hand
+    // (never beyond what a workspace query with blocks = 0 sizes for)
+    if (blocks <= 0)
+        blocks = std::min(kMaxDefaultBlocks, std::max(1, (int)((int64_t)def.blocks * device_geometry().cus / 256)));
     // never more workgroups than steps of work (small tensors)
     const int64_t per_step = (int64_t)out->threads * out->unroll();
     out->blocks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(work_items, per_step), blocks));

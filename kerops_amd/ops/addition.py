@@ -42,8 +42,9 @@ def AddStats(
     return output, mean, sqmean
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AddStatsBackward', 'num_warps'),
-           blocks=stream_knob('AddStatsBackward', 'blocks'), segment=stream_knob('AddStatsBackward', 'segment'))
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AddStatsBackward', 'num_warps', 'add_grad'),
+           blocks=stream_knob('AddStatsBackward', 'blocks', 'add_grad'),
+           segment=stream_knob('AddStatsBackward', 'segment', 'add_grad'))
 def AddStatsBackward(
     add_grad,
     mean_grad,

@@ -81,9 +81,9 @@ def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg, num
     return output, mean, sqmean
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AvgPoolCeilStatsBackward', 'num_warps'),
-           blocks=stream_knob('AvgPoolCeilStatsBackward', 'blocks'),
-           segment=stream_knob('AvgPoolCeilStatsBackward', 'segment'))
+@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AvgPoolCeilStatsBackward', 'num_warps', 'inpgrad'),
+           blocks=stream_knob('AvgPoolCeilStatsBackward', 'blocks', 'inpgrad'),
+           segment=stream_knob('AvgPoolCeilStatsBackward', 'segment', 'inpgrad'))
 def AvgPoolCeilStatsBackward(
     inpgrad,
     meangrad,

@@ -71,8 +71,8 @@ def AbsMax(y, *, blocks: ConfigurableArg):
     return out
 
 
-@configure(blocks=stream_knob('QuantInt8Sym', 'blocks'), num_warps=stream_knob('QuantInt8Sym', 'num_warps'),
-           segment=stream_knob('QuantInt8Sym', 'segment'))
+@configure(blocks=stream_knob('QuantInt8Sym', 'blocks', 'y'), num_warps=stream_knob('QuantInt8Sym', 'num_warps', 'y'),
+           segment=stream_knob('QuantInt8Sym', 'segment', 'y'))
 def QuantInt8Sym(y, absmax=None, *, blocks: ConfigurableArg, num_warps: ConfigurableArg, segment: ConfigurableArg):
     """Symmetric per-tensor int8: scale = absmax/127, q = clamp(rint(y/scale), -127, 127).
 

@@ -8,12 +8,14 @@ kerops/ops/conv/dwconv_wgrad.py:10-22); the tables in kerops_amd/ops/conv were m
     python -m kerops_amd.tune --channels 32 64 --apply          # and reconfigure the ops of this process
 
     python -m kerops_amd.tune --streams                         # the flat stream ops: (blocks, num_warps, segment)
-    python -m kerops_amd.tune --streams --write                 # ... and rewrite settings/stream_shapes.json
+    python -m kerops_amd.tune --streams --all --write           # every channel count of the README table and the
+                                                                # small-tensor class; rewrites settings/stream_shapes.json
 
 `tune(...)` returns {op: {C: (W_block, D_block, lane_channels, H_chunk, ms)}}; `apply(result)` installs the
 choices through the ops' `reconfigure`, the same mechanism a user of the reference has for overriding its tables.
-`tune_streams(...)` returns {op: (blocks, num_warps, segment, ms)}; `apply_streams(result)` puts them into the live
-table of `kerops_amd.settings.stream_table`, which the stream ops read on every call.
+`tune_streams(...)` returns {op: (blocks, num_warps, segment, ms)}; `apply_streams(result, key)` puts them into the
+live table of `kerops_amd.settings.stream_table` under a key (a channel count, "small" or "default"), which the
+stream ops read on every call.
 """
 import argparse
 import math
@@ -162,12 +164,18 @@ def tune_streams(shape=(1, 64, 350, 350, 128), ops=None, iters=12, warmup=3, rou
     return result
 
 
-def apply_streams(result, write=False, note=''):
+def apply_streams(result, write=False, note='', key='default'):
     from .settings import stream_table
     for op, (blocks, warps, segment, _) in result.items():
-        stream_table.set_stream_shape(op, blocks=blocks, num_warps=warps, segment=segment)
+        stream_table.set_stream_shape(op, blocks=blocks, num_warps=warps, segment=segment, key=key)
     if write:
         stream_table.save(note=note)
+
+
+# `--streams --all`: the tensors behind each key of the stream table.  "default" (channel counts without an entry)
+# repeats the 64-channel measurement.
+STREAM_CLASSES = (('8', (1, 8, 350, 350, 128)), ('16', (1, 16, 350, 350, 128)), ('32', (1, 32, 350, 350, 128)),
+                  ('64', (1, 64, 350, 350, 128)), ('128', (1, 128, 350, 350, 128)), ('small', (2, 16, 64, 64, 64)))
 
 
 def main():
@@ -175,18 +183,28 @@ def main():
     ap.add_argument('--streams', action='store_true', help='tune the flat stream ops instead of the convolution pair')
     ap.add_argument('--write', action='store_true', help='with --streams: rewrite settings/stream_shapes.json')
     ap.add_argument('--ops', nargs='*', default=None, help='with --streams: only these ops')
+    ap.add_argument('--all', action='store_true', help='with --streams: every class of the stream table')
+    ap.add_argument('--key', default=None, help='with --streams: table key to file the result under (default: the '
+                                                'channel count of --shape)')
     ap.add_argument('--shape', type=int, nargs=5, default=[1, 64, 350, 350, 128], metavar=('N', 'C', 'H', 'W', 'D'))
     ap.add_argument('--channels', type=int, nargs='*', default=None)
     ap.add_argument('--h-chunks', type=int, nargs='*', default=[0])
     ap.add_argument('--apply', action='store_true')
     args = ap.parse_args()
     if args.streams:
-        res = tune_streams(tuple(args.shape), ops=args.ops, verbose=True)
-        for op, (blocks, warps, segment, ms) in res.items():
-            print(f'best {op:20s}: blocks={blocks} num_warps={warps} segment={segment}  {ms:.4f} ms')
-        shape = ','.join(str(v) for v in args.shape)
-        apply_streams(res, write=args.write, note=f'measured by kerops_amd.tune --streams at ({shape}) on '
-                                                  f'{torch.cuda.get_device_name(0)}')
+        classes = STREAM_CLASSES if args.all else ((args.key or str(args.shape[1]), tuple(args.shape)),)
+        for key, shape in classes:
+            res = tune_streams(shape, ops=args.ops, verbose=not args.all)
+            for op, (blocks, warps, segment, ms) in res.items():
+                print(f'best {key:>7s} {op:28s}: blocks={blocks} num_warps={warps} segment={segment}  {ms:.4f} ms',
+                      flush=True)
+            apply_streams(res, key=key)
+            if key == '64':
+                apply_streams(res, key='default')
+        if args.write:
+            from .settings import stream_table
+            stream_table.save(note='measured by kerops_amd.tune --streams on ' + torch.cuda.get_device_name(0) + ': keys '
+                              + ', '.join(f'{k} at {sh}' for k, sh in classes) + '; "default" repeats 64')
         return
     res = tune(tuple(args.shape), args.channels, tuple(args.h_chunks), verbose=True)
     for op, table in res.items():

@@ -140,36 +140,59 @@ def test_tuner_apply_installs_and_falls_back():
 
 
 def test_stream_table_feeds_the_stream_ops_live():
-    """The launch shapes of the stream ops come from settings/stream_shapes.json through zero-argument
-    configurators: the ops see a changed table on their next call, an op missing from the table gets zeros
-    (the library's built-in choice)."""
+    """The launch shapes of the stream ops come from settings/stream_shapes.json, keyed by op and channel count like
+    the reference's tables (kerops/ops/conv/dwconv.py:10-17), through configurators that receive the op's tensor:
+    the ops see a changed table on their next call; a channel count without an entry gets the op's default, small
+    tensors their own class, an op missing from the table zeros (the library's built-in choice)."""
+    from kerops_amd.ops.addition import AddStatsBackward
     from kerops_amd.ops.bnrelu import ApplyBNReLU
     from kerops_amd.settings import stream_table
 
     table = stream_table.load()
-    assert set(table['ApplyBNReLU']) == {'blocks', 'num_warps', 'segment'}
+    assert 'default' in table['ApplyBNReLU']
     for op, entry in table.items():
-        assert entry['num_warps'] in (0, 4, 8, 16) and entry['segment'] in (0, 1, 2, 4, 8) and 0 <= entry['blocks'] <= 65536
+        for key, shape in entry.items():
+            assert key in ('default', 'small') or int(key) in (2, 4, 8, 16, 32, 64, 128, 256), (op, key)
+            assert set(shape) == {'blocks', 'num_warps', 'segment'}
+            assert shape['num_warps'] in (0, 4, 8, 16) and shape['segment'] in (0, 1, 2, 4, 8)
+            assert 0 <= shape['blocks'] <= 65536
+    import torch
+    big = torch.empty((1, 64, 350, 350, 128), dtype=torch.float16, device='meta')
+    other = torch.empty((1, 256, 350, 350, 16), dtype=torch.float16, device='meta')
+    small = torch.empty((1, 64, 16, 16, 16), dtype=torch.float16, device='meta')
     knob = ApplyBNReLU.configurators['num_warps']
-    assert callable(knob) and knob() == table['ApplyBNReLU']['num_warps']
-    saved = stream_table.stream_shape('ApplyBNReLU')
+    assert callable(knob) and knob(big) == stream_table.stream_shape('ApplyBNReLU', 64, big.numel() * 2)['num_warps']
+    assert AddStatsBackward.configurators['blocks'](add_grad=big) == \
+        stream_table.stream_shape('AddStatsBackward', 64, big.numel() * 2)['blocks']
+    saved = {op: {k: dict(v) for k, v in e.items()} for op, e in table.items()}
     try:
-        stream_table.set_stream_shape('ApplyBNReLU', blocks=7, num_warps=4, segment=1)
-        assert ApplyBNReLU.configurators['blocks']() == 7 and ApplyBNReLU.configurators['segment']() == 1
+        stream_table.set_stream_shape('ApplyBNReLU', blocks=7, num_warps=4, segment=1, key=64)
+        stream_table.set_stream_shape('ApplyBNReLU', blocks=9, num_warps=8, segment=4, key='default')
+        stream_table.set_stream_shape('ApplyBNReLU', blocks=3, num_warps=4, segment=1, key='small')
+        conf = ApplyBNReLU.configurators
+        assert (conf['blocks'](big), conf['num_warps'](big), conf['segment'](big)) == (7, 4, 1)
+        assert (conf['blocks'](other), conf['num_warps'](other), conf['segment'](other)) == (9, 8, 4)
+        assert (conf['blocks'](small), conf['num_warps'](small), conf['segment'](small)) == (3, 4, 1)
+        assert ApplyBNReLU.can_be_configured(x=big)
     finally:
-        stream_table.set_stream_shape('ApplyBNReLU', **saved)
+        stream_table._table.clear()
+        stream_table._table.update(saved)
     assert stream_table.stream_shape('NoSuchOp') == {'blocks': 0, 'num_warps': 0, 'segment': 0}
-    assert stream_table.stream_knob('NoSuchOp', 'blocks')() == 0
+    assert stream_table.stream_knob('NoSuchOp', 'blocks')(big) == 0
 
 
 def test_stream_table_round_trips_through_its_file(tmp_path):
     from kerops_amd.settings import stream_table
 
-    before = {op: dict(e) for op, e in stream_table.load().items()}
+    before = {op: {k: dict(v) for k, v in e.items()} for op, e in stream_table.load().items()}
     path = str(tmp_path / 'shapes.json')
     try:
-        stream_table.set_stream_shape('Stats', blocks=123, num_warps=16, segment=8)
+        stream_table.set_stream_shape('Stats', blocks=123, num_warps=16, segment=8, key=32)
         stream_table.save(path, note='test')
-        assert stream_table.load(path)['Stats'] == {'blocks': 123, 'num_warps': 16, 'segment': 8}
+        assert stream_table.load(path)['Stats']['32'] == {'blocks': 123, 'num_warps': 16, 'segment': 8}
+        # the one-shape-per-op form is read as the op's default
+        with open(path, 'w') as f:
+            f.write('{"shapes": {"Stats": {"blocks": 5, "num_warps": 4, "segment": 1}}}')
+        assert stream_table.load(path) == {'Stats': {'default': {'blocks': 5, 'num_warps': 4, 'segment': 1}}}
     finally:
         assert stream_table.load() == before
