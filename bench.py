@@ -15,9 +15,11 @@ channels_last_3d (the README-shape forward and weight-gradient target configurat
   ops                     the same figures for every other op of the path (statistics, BN-ReLU, pooling,
                           quantisers, their backward ops, the fused and the linear ops) and for every C of
                           the README table
-  cpu_baseline            the CPU oracle (oracle/kerops_oracle.c, OpenMP) on a bounded crop of the
-                          same workload, scaled by the voxel ratio; torch's CPU conv3d(groups=C),
-                          the reference tests' ground truth, is timed beside it
+  cpu_baseline            torch.nn.functional.conv3d(groups=C) in fp32 and its autograd weight gradient on the
+                          box's host cores (the CPU baseline the target names; the reference tests' ground
+                          truth), at the full shape when the host has the memory for it, else on a crop scaled
+                          by the voxel ratio; the CPU oracle (oracle/kerops_oracle.c, OpenMP) is timed beside
+                          it on a bounded crop (cpu_oracle_port)
 
 Inputs are synthetic: x, grad ~ N(0, 1) (mean, variance), depthwise weight ~ N(0, 1/27), drawn
 with a fixed seed.  Every GPU on this pool is a single-GPU box, so --gpus above 1 is refused.
@@ -38,6 +40,7 @@ H, W, D = 350, 350, 128
 V = H * W * D
 
 TRAFFIC_TABLE = os.path.join(ROOT, 'profiles', 'dwconv_hbm_traffic_by_channels.md')
+KERNEL_NAMES = {'dwconv_fwd': 'kerops::dwconv_fwd_mfma_kernel', 'dwconv_wgrad': 'kerops::dwconv_wgrad_dma_kernel'}
 
 
 def load_traffic_table(path=TRAFFIC_TABLE):
@@ -78,7 +81,7 @@ def clock_under_load(torch, ops, seconds=1.2):
                         samples.append(int(m.group(1)))
                 except Exception:
                     return
-        th = threading.Thread(target=sampler, daemon=True)
+        th = threading.Thread(target=sampler)
         t0 = time.perf_counter()
         n = 0
         th.start()
@@ -89,7 +92,7 @@ def clock_under_load(torch, ops, seconds=1.2):
             n += 40
         ms = (time.perf_counter() - t0) * 1e3 / n
         stop.set()
-        th.join(timeout=6)
+        th.join()  # the last rocm-smi call (bounded by its own timeout) returns before the run goes on
         body = samples[1:] if len(samples) > 2 else samples  # the first sample may predate the load
         out[name] = {'sclk_mhz': median(body) if body else None, 'samples': len(samples), 'ms_back_to_back': round(ms, 4)}
     return out
@@ -140,54 +143,90 @@ def figures(ms, nbytes, clone_gbps):
             'frac_of_clone': round(gbps / clone_gbps, 4) if clone_gbps else None, 'algorithmic_bytes': nbytes}
 
 
-def cpu_baseline(torch, C):
-    """Oracle (a scalar-per-voxel C port with OpenMP) and torch CPU conv3d on a crop."""
+def host_memory_gib():
+    """(total, available) host memory in GiB, from /proc/meminfo."""
+    info = {}
+    try:
+        for line in open('/proc/meminfo'):
+            k, v = line.split(':', 1)
+            info[k] = int(v.split()[0]) / 2 ** 20
+    except OSError:
+        return None, None
+    return info.get('MemTotal'), info.get('MemAvailable')
+
+
+def cpu_baseline(torch, C, x_dev, g_dev, wk_dev):
+    """The host baselines.  Returns (torch conv3d figures, oracle port figures)."""
     import oracle
     from torch.nn import functional as F
 
-    crop = (1, C, 176, 176, 128)
-    vox = crop[2] * crop[3] * crop[4]
-    g = torch.Generator('cpu').manual_seed(322)
-    x = torch.randn(*crop, generator=g).half().to(memory_format=torch.channels_last_3d)
-    gr = torch.randn(*crop, generator=g).half().to(memory_format=torch.channels_last_3d)
-    wt = (torch.randn(C, 1, 3, 3, 3, generator=g) / math.sqrt(27)).half()
-    wk = wt[:, 0].permute(1, 2, 3, 0).contiguous()
-    oracle.dwconv_fwd(x[:, :, :8], wk, wide=False)  # load the library, warm the thread pool
-
-    reps_f, reps_w = 12, 8  # about 10 s of CPU work on 16 cores
-    t0 = time.perf_counter()
-    for _ in range(reps_f):
-        oracle.dwconv_fwd(x, wk, wide=False)
-    t_f = (time.perf_counter() - t0) / reps_f
-    t0 = time.perf_counter()
-    for _ in range(reps_w):
-        oracle.dwconv_wgrad(x, gr)
-    t_w = (time.perf_counter() - t0) / reps_w
+    total_gib, avail_gib = host_memory_gib()
+    # fp32 x, grad, y and the weight-gradient pass's temporaries: about 16 bytes * 3 per element, with headroom
+    need_gib = 3 * 4 * V * C * 4 / 2 ** 30
+    full = avail_gib is not None and avail_gib >= need_gib
+    hh = H if full else 176
+    ww = W if full else 176
+    vox = hh * ww * D
     scale = V / vox
-    port = {
-        'value': round((t_f + t_w) * 1e3 * scale, 1), 'unit': 'ms', 'cores': oracle.num_threads(), 'kind': 'port',
-        'sample': f'oracle DWConv fwd (fp32, {reps_f} runs) + wgrad (fp64, {reps_w} runs) on the leading crop '
-                  f'(1,{C},176,176,128), time scaled by the voxel ratio {scale:.2f} to (1,{C},350,350,128)',
-        'fwd_ms_scaled': round(t_f * 1e3 * scale, 1), 'wgrad_ms_scaled': round(t_w * 1e3 * scale, 1),
-        'host_cpus': os.cpu_count(),
-    }
-    # the reference tests' ground truth on the same crop: conv3d(groups=C) in fp32 and its autograd
-    xf = x.float()
+    # the same synthetic tensors as the GPU step (leading crop when the host is short of memory)
+    x16 = x_dev[:, :, :hh, :ww].contiguous(memory_format=torch.channels_last_3d).cpu()
+    g16 = g_dev[:, :, :hh, :ww].contiguous(memory_format=torch.channels_last_3d).cpu()
+    wk = wk_dev.cpu()
+    wt = wk.permute(3, 0, 1, 2).unsqueeze(1).contiguous()  # (C,1,3,3,3), the layout torch wants
+
+    xf, gf = x16.float(), g16.float()
     w32 = wt.float().requires_grad_(True)
     ts_f, ts_w = [], []
-    for _ in range(3):
+    reps = 3
+    for _ in range(reps):
         t0 = time.perf_counter()
         y = F.conv3d(xf, w32, None, 1, 1, 1, C)
         ts_f.append(time.perf_counter() - t0)
         t0 = time.perf_counter()
-        (gw,) = torch.autograd.grad(y, w32, gr.float())
+        (gw,) = torch.autograd.grad(y, w32, gf)
         ts_w.append(time.perf_counter() - t0)
+        del y, gw
+    del xf, gf
+    t_f, t_w = median(ts_f), median(ts_w)
+    where = (f'full shape (1,{C},{H},{W},{D})' if full else
+             f'leading crop (1,{C},{hh},{ww},{D}), times scaled by the voxel ratio {scale:.2f} '
+             f'(host memory available {avail_gib} GiB < {need_gib:.0f} GiB wanted for the full shape)')
     torch_cpu = {
-        'fwd_ms_scaled': round(median(ts_f) * 1e3 * scale, 1), 'wgrad_ms_scaled': round(median(ts_w) * 1e3 * scale, 1),
-        'threads': torch.get_num_threads(), 'host_cpus': os.cpu_count(),
-        'sample': 'torch.nn.functional.conv3d(groups=C) fp32 and autograd wgrad on the same crop, median of 3, scaled',
+        'value': round((t_f + t_w) * 1e3 * scale, 1), 'unit': 'ms', 'cores': torch.get_num_threads(), 'kind': 'reference',
+        'kind_note': 'torch.nn.functional.conv3d(groups=C) on the host, the library routine the reference tests use as '
+                     'ground truth (tests/ops/test_conv.py:25,62-72) and the CPU baseline the target names; not a build '
+                     'of the reference (which is Python/Triton and has no CPU path)',
+        'sample': f'fp32 conv3d(groups={C}) forward + autograd weight gradient, median of {reps} runs, {where}',
+        'fwd_ms': round(t_f * 1e3 * scale, 1), 'wgrad_ms': round(t_w * 1e3 * scale, 1),
+        'torch_num_threads': torch.get_num_threads(), 'host_cpus': os.cpu_count(),
+        'host_memory_gib': {'total': round(total_gib, 1) if total_gib else None,
+                            'available': round(avail_gib, 1) if avail_gib else None},
+        'full_shape': full,
     }
-    return port, torch_cpu
+
+    # the oracle port on a bounded crop
+    crop = (176, 176)
+    xo = x16[:, :, :crop[0], :crop[1]].contiguous(memory_format=torch.channels_last_3d)
+    go = g16[:, :, :crop[0], :crop[1]].contiguous(memory_format=torch.channels_last_3d)
+    oscale = V / (crop[0] * crop[1] * D)
+    oracle.dwconv_fwd(xo[:, :, :8], wk, wide=False)  # load the library, warm the thread pool
+    reps_f, reps_w = 6, 4
+    t0 = time.perf_counter()
+    for _ in range(reps_f):
+        oracle.dwconv_fwd(xo, wk, wide=False)
+    o_f = (time.perf_counter() - t0) / reps_f
+    t0 = time.perf_counter()
+    for _ in range(reps_w):
+        oracle.dwconv_wgrad(xo, go)
+    o_w = (time.perf_counter() - t0) / reps_w
+    port = {
+        'value': round((o_f + o_w) * 1e3 * oscale, 1), 'unit': 'ms', 'cores': oracle.num_threads(), 'kind': 'port',
+        'sample': f'oracle DWConv fwd (fp32, {reps_f} runs) + wgrad (fp64, {reps_w} runs) on the leading crop '
+                  f'(1,{C},{crop[0]},{crop[1]},{D}), time scaled by the voxel ratio {oscale:.2f} to (1,{C},{H},{W},{D})',
+        'fwd_ms_scaled': round(o_f * 1e3 * oscale, 1), 'wgrad_ms_scaled': round(o_w * 1e3 * oscale, 1),
+        'host_cpus': os.cpu_count(),
+    }
+    return torch_cpu, port
 
 
 def main():
@@ -269,7 +308,7 @@ def main():
     dom_name, dom_avg = ('dwconv_wgrad', wg_avg) if wg_avg >= fwd_avg else ('dwconv_fwd', fwd_avg)
     achieved = nbytes / dom_avg / 1e6
     roofline = {
-        'kernel': 'kerops::' + dom_name + '_mfma_kernel',
+        'kernel': KERNEL_NAMES[dom_name],
         'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
         'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': traffic_table.get((dom_name, C)),
         'traffic_source': traffic_note, 'algorithmic_bytes': nbytes, 'avg_launch_ms': round(dom_avg, 4),
@@ -279,7 +318,7 @@ def main():
     other = 'dwconv_fwd' if dom_name == 'dwconv_wgrad' else 'dwconv_wgrad'
     other_avg = fwd_avg if other == 'dwconv_fwd' else wg_avg
     roofline_other = {
-        'kernel': 'kerops::' + other + '_mfma_kernel', 'bound': 'hbm', 'achieved': round(nbytes / other_avg / 1e6, 1),
+        'kernel': KERNEL_NAMES[other], 'bound': 'hbm', 'achieved': round(nbytes / other_avg / 1e6, 1),
         'peak': HBM_PEAK_GBPS, 'unit': 'GB/s', 'frac': round(nbytes / other_avg / 1e6 / HBM_PEAK_GBPS, 4),
         'traffic': traffic_table.get((other, C)), 'algorithmic_bytes': nbytes,
         'avg_launch_ms': round(other_avg, 4),
@@ -341,7 +380,40 @@ def main():
             del wt_t
         except Exception as e:  # a reported side figure only
             ops['gpu_torch_conv3d_groups'] = {'error': repr(e)[:200]}
-        table = {}
+        def stream_rows(xc, gc, c):
+            """Every stream op at (1,c,350,350,128): ms and fraction of the HBM peak of its algorithmic bytes."""
+            wv = torch.rand(c, device=dev, generator=gen) + 0.5
+            bv = torch.randn(c, device=dev, generator=gen) * 0.3
+            mgc = torch.randn(c, device=dev, generator=gen)
+            sgc = torch.randn(c, device=dev, generator=gen)
+            pooled_c = AvgPoolCeilStats(xc)[0]
+            gpc = torch.randn_like(pooled_c)
+            q8c = QuantUint8Window(xc, 3.0)
+            amax = torch.full((1,), 5.0, device=dev)
+            vc = V * c
+            cases = [
+                ('Stats', lambda: Stats(xc), 2 * vc), ('StatsBackward', lambda: StatsBackward(xc, mgc, sgc), 4 * vc),
+                ('AddStats', lambda: AddStats(xc, gc), 6 * vc),
+                ('AddStatsBackward', lambda: AddStatsBackward(gc, mgc, sgc, xc), 6 * vc),
+                ('ApplyBNReLU', lambda: ApplyBNReLU(xc, wv, bv), 4 * vc),
+                ('ApplyBNReLUBackward', lambda: ApplyBNReLUBackward(xc, wv, bv, gc), 6 * vc),
+                ('AvgPoolCeilStats', lambda: AvgPoolCeilStats(xc), 2 * vc + 2 * pooled_c.numel()),
+                ('ApplyBNReLU+AvgPoolCeilStats_fused', lambda: ApplyBNReLUAvgPoolCeilStats(xc, wv, bv),
+                 2 * vc + 2 * pooled_c.numel()),
+                ('AvgPoolCeilStatsBackward', lambda: AvgPoolCeilStatsBackward(gpc, mgc, sgc, pooled_c, tuple(xc.shape)),
+                 2 * vc + 4 * pooled_c.numel()),
+                ('QuantUint8Window', lambda: QuantUint8Window(xc, 3.0), 3 * vc),
+                ('DequantUint8Window', lambda: DequantUint8Window(q8c, torch.float16, 3.0), 3 * vc),
+                ('QuantInt8Sym', lambda: QuantInt8Sym(xc, amax), 3 * vc),
+            ]
+            rows = {}
+            for name, fn, nb in cases:
+                ms_ = time_op(torch, fn, it, wm)[0]
+                rows[name] = {'ms': round(ms_, 4), 'frac_hbm_peak': round(nb / ms_ / 1e6 / HBM_PEAK_GBPS, 4)}
+            return rows
+
+        from kerops_amd.ops.quantization import QuantInt8Sym
+        table, stream_table = {}, {str(C): stream_rows(x, g, C)}  # (x, g still hold the C-channel tensors here)
         for c in (8, 16, 32, 64, 128):
             if c == C:
                 table[str(c)] = {'clone_ms': round(clone_ms, 4), 'dwconv_ms': fwd['ms'], 'wgrad_ms': wg['ms'],
@@ -356,10 +428,19 @@ def main():
             cm = time_op(torch, lambda: x.clone(), it, wm)[0]
             fm = time_op(torch, lambda: DWConv(x, wkc), it, wm)[0]
             wgm = time_op(torch, lambda: DWConvWGRAD(x, g), it, wm)[0]
+            bwm = time_op(torch, lambda: DWConvBackward(x, g, wkc), it, wm)[0]
             table[str(c)] = {'clone_ms': round(cm, 4), 'dwconv_ms': round(fm, 4), 'wgrad_ms': round(wgm, 4),
                              'dwconv_frac_of_clone': round(cm / fm, 4), 'wgrad_frac_of_clone': round(cm / wgm, 4),
                              'dwconv_frac_hbm_peak': round(4 * V * c / fm / 1e6 / HBM_PEAK_GBPS, 4),
-                             'wgrad_frac_hbm_peak': round(4 * V * c / wgm / 1e6 / HBM_PEAK_GBPS, 4)}
+                             'wgrad_frac_hbm_peak': round(4 * V * c / wgm / 1e6 / HBM_PEAK_GBPS, 4),
+                             'backward_fused_ms': round(bwm, 4),
+                             'backward_fused_frac_hbm_peak': round(6 * V * c / bwm / 1e6 / HBM_PEAK_GBPS, 4)}
+            stream_table[str(c)] = stream_rows(x, g, c)
+        table[str(C)]['backward_fused_ms'] = ops['DWConvBackward_fused']['ms']
+        table[str(C)]['backward_fused_frac_hbm_peak'] = ops['DWConvBackward_fused']['frac_hbm_peak']
+        ops['stream_ops_by_channels'] = {str(c): stream_table[str(c)] for c in (8, 16, 32, 64, 128) if str(c) in stream_table}
+        ops['stream_ops_by_channels_note'] = ('every stream op at (1,C,350,350,128) with the launch shape of the table '
+                                              'entry for that C (kerops_amd/settings/stream_shapes.json)')
         ops['readme_table'] = table
         # target configuration 5: fused depthwise-separable block with int8 output at (1,64,128,128,128)
         del x, g
@@ -435,12 +516,14 @@ def main():
                           'ceiling 2400 MHz')
         del xs, gs
 
-    cpu, cpu_torch = (None, None)
+    cpu, cpu_port = (None, None)
     if not args.no_cpu_baseline:
-        cpu, cpu_torch = cpu_baseline(torch, C)
+        xs, gs, wks = make(C)
+        cpu, cpu_port = cpu_baseline(torch, C, xs, gs, wks)
+        del xs, gs
 
     out = {
-        'metric': 'DWConv fwd/wgrad ms + % HBM roofline, fp16 (1,64,350,350,128) NDHWC',
+        'metric': f'DWConv fwd/wgrad ms + % HBM roofline, fp16 (1,{C},350,350,128) NDHWC',
         'value': round(ms_per_step, 4), 'unit': 'ms', 'n_gpus': 1, 'steps': K, 'warmup': args.warmup,
         'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'f16 in/out, f32 accumulate', 'data': 'synthetic',
@@ -455,7 +538,7 @@ def main():
                     'wgrad_frac_of_clone>=0.50': wg['frac_of_clone'] >= 0.50},
         'roofline': roofline, 'roofline_other': roofline_other,
         'core_clock_under_load': clocks,
-        'cpu_baseline': cpu, 'cpu_torch_conv3d': cpu_torch, 'ops': ops,
+        'cpu_baseline': cpu, 'cpu_oracle_port': cpu_port, 'ops': ops,
         'device': torch.cuda.get_device_name(0),
     }
     print(json.dumps(out))

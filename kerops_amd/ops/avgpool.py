@@ -10,7 +10,7 @@ import torch
 
 from .. import _lib
 from ..settings import ConfigurableArg, configure, get_l1_cache
-from ..settings.stream_table import stream_knob
+from ..settings.stream_table import stream_knob, stream_shape
 from ._common import next_power_of_2, require_cuda, stream_waves
 
 
@@ -81,9 +81,21 @@ def ApplyBNReLUAvgPoolCeilStats(x, weight, bias, *, blocks: ConfigurableArg, num
     return output, mean, sqmean
 
 
-@configure(l1_cache_bytes=get_l1_cache, num_warps=stream_knob('AvgPoolCeilStatsBackward', 'num_warps', 'inpgrad'),
-           blocks=stream_knob('AvgPoolCeilStatsBackward', 'blocks', 'inpgrad'),
-           segment=stream_knob('AvgPoolCeilStatsBackward', 'segment', 'inpgrad'))
+def _backward_knob(key):
+    """Table value for the gradient tensor the op writes: its tensor arguments are all of the pooled size (an eighth),
+    so the class is taken from `outgrad_shape`."""
+    def knob(outgrad_shape):
+        voxels = 1
+        for extent in outgrad_shape:
+            voxels *= int(extent)
+        return stream_shape('AvgPoolCeilStatsBackward', int(outgrad_shape[1]), 2 * voxels)[key]
+
+    knob.__name__ = f'AvgPoolCeilStatsBackward_{key}'
+    return knob
+
+
+@configure(l1_cache_bytes=get_l1_cache, num_warps=_backward_knob('num_warps'), blocks=_backward_knob('blocks'),
+           segment=_backward_knob('segment'))
 def AvgPoolCeilStatsBackward(
     inpgrad,
     meangrad,
