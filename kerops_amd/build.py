@@ -34,6 +34,7 @@ COMMON_FLAGS = [
 # at a fraction of the rate of two ds_read_b64: the kernels that read their operands 8 bytes wide are built without it.
 PER_FILE_FLAGS = {
     'dwconv_wgrad_dma.hip': ['-Xclang', '-target-feature', '-Xclang', '-load-store-opt'],
+    'dwconv_bwd_dma.hip': ['-Xclang', '-target-feature', '-Xclang', '-load-store-opt'],
 }
 
 

@@ -16,6 +16,8 @@
 // combined with wavefront shuffles, wavefronts through LDS, and the workgroup writes
 // one partial [27][slab] to the workspace.  A second kernel adds the partials in a
 // fixed order, so the result is deterministic (no atomics).
+#include <cstdlib>
+
 #include "common.hpp"
 #include "dwconv_wgrad.hpp"
 
@@ -1207,6 +1209,17 @@ static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, float* gw, hip
 }
 
 // fused backward: one patch shape per channel count, two workgroups of 512 threads per CU
+// KEROPS_BWD_STAGING=registers selects the register-staged kernel (kept as a tested alternative) instead of the
+// LDS-direct one; the two use different patch shapes, so the choice is part of the plan
+static bool bwd_staged_in_registers()
+{
+    static const bool v = [] {
+        const char* e = getenv("KEROPS_BWD_STAGING");
+        return e && e[0] == 'r';
+    }();
+    return v;
+}
+
 static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
 {
     if (N <= 0 || H <= 0 || W <= 0 || D <= 0) {
@@ -1223,8 +1236,13 @@ static int plan_bwd(int N, int H, int W, int D, int C, int h_chunk, WgPlan* p)
     }
     p->cg = C >= 64 ? 8 : C / 8;
     p->cl = 16;
-    p->tile_w = p->cg == 8 ? 4 : 8;
-    p->tile_d = p->cg >= 4 ? 8 : p->cg == 2 ? 16 : 32;
+    if (bwd_staged_in_registers()) {
+        p->tile_w = p->cg == 8 ? 4 : 8;
+        p->tile_d = p->cg >= 4 ? 8 : p->cg == 2 ? 16 : 32;
+    } else {  // patches of 512 16-byte chunks: a wavefront of either role owns four rows
+        p->tile_w = 8;
+        p->tile_d = 64 / p->cg;
+    }
     p->n_slab = C / (p->cg * 8);
     p->n_wt = ceil_div(W, p->tile_w);
     p->n_dt = ceil_div(D, p->tile_d);
@@ -1326,6 +1344,11 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
     b.bal_r = p.bal_r;
     b.n_tiles = p.n_tiles;
     b.n_xcd = (uint32_t)p.n_xcd;
+    if (!bwd_staged_in_registers() && launch_bwd_dma(b, p.cg, p.tile_w, p.tile_d, s) == 0) {
+        rc = check_launch("dwconv_bwd");
+        if (rc != KEROPS_OK) return rc;
+        return reduce_partials(b.ws, p, p.cg * 8, b.C, gw, s);
+    }
 #define KEROPS_BS_GO(CGv, TWv, TDv)                                                                                  \
     {                                                                                                                \
         using Cfg = BsCfg<CGv, TWv, TDv, 512>;                                                                       \

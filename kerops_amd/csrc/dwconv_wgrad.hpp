@@ -26,4 +26,9 @@ struct WgArgs {
 // g planes ahead); the partials go to a.ws like those of the other kernels.  Returns 1 if no kernel has that shape.
 int launch_wgrad_dma(const WgArgs& a, int cg, int tile_w, int tile_d, int depth, hipStream_t stream);
 
+
+// dwconv_bwd_dma.hip: launches the LDS-direct fused backward kernel for (channel groups of 8 per slab, patch W, patch D)
+// if it is built with that shape; dx is written, the weight-gradient partials go to a.ws.  Returns 1 otherwise.
+int launch_bwd_dma(const WgArgs& a, int cg, int tile_w, int tile_d, hipStream_t stream);
+
 }  // namespace kerops

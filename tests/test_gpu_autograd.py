@@ -139,8 +139,8 @@ def test_linear_family_gradients_against_torch_autograd():
 
 
 def test_fused_forward_functions_have_the_gradients_of_their_compositions():
-    # the one-pass forward ops are bit-identical to the compositions they stand for; their backward runs the same
-    # backward ops
+    # the one-pass forward ops do the arithmetic of the compositions they stand for (the conv output bit for bit; the
+    # statistics are fp32 sums taken in another order); their backward runs the same backward ops
     g = cpu_gen(47)
     n, c, h, w, d = 2, 32, 6, 7, 9
     x = rand_cl3d(g, n, c, h, w, d)
@@ -167,13 +167,23 @@ def test_fused_forward_functions_have_the_gradients_of_their_compositions():
         else:
             out = ReLULinearAddFn.apply(ApplyBNReLUFn.apply(y, scale, shift), pd, rd)
         out.backward(go.to(DEV))
-        return [out.detach()] + [t.grad for t in leaves]
+        return [out.detach()] + [t.grad for t in leaves] + [y.detach(), mean.detach(), sq.detach()]
 
     a, b = run(True), run(False)
-    assert torch.equal(a[0], b[0])  # forward: bit for bit
+    assert torch.equal(a[7], b[7])  # the conv output: bit for bit
+    for u, v in ((a[8], b[8]), (a[9], b[9])):  # per-channel sums of 756 values in two orders
+        assert torch.allclose(u, v, rtol=1e-5, atol=1e-6)
+    # scale and shift then differ in their last fp32 bits, which can move an fp16 activation by one step before
+    # the pointwise layer and the output by one more
+    assert (a[0].float() - b[0].float()).abs().max().item() <= 2.0 ** -8 * max(1.0, b[0].float().abs().max().item())
+    # with the same scale and shift the fused second half is bit-identical to its composition
+    yd, pd, rd = a[7], pw.to(DEV), res.to(DEV)
+    sc, sh = (torch.rand(c, generator=g) + 0.5).to(DEV), (torch.randn(c, generator=g) * 0.3).to(DEV)
+    assert torch.equal(ApplyBNReLULinearAddFn.apply(yd, sc, sh, pd, rd),
+                       ReLULinearAddFn.apply(ApplyBNReLUFn.apply(yd, sc, sh), pd, rd))
     # backward: the same backward ops on the same tensors, except that the composition lets torch add the two fp16
     # gradients that reach y (one more rounding) where the fused Function adds them in fp32 inside AddStatsBackward
-    for i, (u, v) in enumerate(zip(a[1:], b[1:])):
+    for i, (u, v) in enumerate(zip(a[1:7], b[1:7])):
         assert u.dtype == v.dtype and u.shape == v.shape, i
         err = (u.float() - v.float()).abs().max().item()
         assert err <= 2.0 ** -8 * max(1.0, v.float().abs().max().item()), (i, err)
