@@ -1088,7 +1088,7 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     p->cg = C >= 64 ? 8 : C / 8;
     if (tile_w == 0 && tile_d == 0 && lane_channels == 0) {
         // measured best on MI355X at (1, C, 350, 350, 128): the matrix-core kernels with LDS-direct staging,
-        // 512-thread workgroups on patches of 512 16-byte chunks
+        // 256-thread workgroups on patches of 512 16-byte chunks
         switch (p->cg) {
             case 1: tile_w = 8; tile_d = 64; break;
             case 2: tile_w = 8; tile_d = 32; break;
@@ -1112,7 +1112,8 @@ static int plan_wgrad(int N, int H, int W, int D, int C, int tile_w, int tile_d,
     p->n_dt = ceil_div(D, tile_d);
     // 256 CUs hold 2 workgroups of 512 threads or 4 of 256 each; every workgroup also leaves one partial
     const int64_t per_plane = (int64_t)N * p->n_wt * p->n_dt * p->n_slab;
-    // matrix-core kernels run 512 threads on patches of 512 or more 16-byte chunks
+    // patches of 512 or more 16-byte chunks: two workgroups per compute unit (512 threads each when staged through
+    // registers; the LDS-direct kernels run 256 threads and are held to two by their staging rings)
     const bool big_wg = lane_channels >= 16 ? tile_w * tile_d * p->cg >= 512 : (p->cg == 8 && tile_w * tile_d >= 64);
     const DeviceGeometry geo = device_geometry();
     p->n_xcd = geo.xcds;

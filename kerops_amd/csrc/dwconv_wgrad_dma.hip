@@ -7,6 +7,9 @@
 #ifndef KEROPS_WD_COMPUTE
 #define KEROPS_WD_COMPUTE 1
 #endif
+#ifndef KEROPS_WD_LOADS
+#define KEROPS_WD_LOADS 1
+#endif
 
 namespace kerops {
 
@@ -74,7 +77,7 @@ struct WdCfg {
 // of their own that carry the streaming hint, so that they do not push the shared halo lines out of the L2; a
 // compile-time choice made on the host by tensor size (streaming loads bypass the memory-side cache as well)
 template <class Cfg, bool NTI>
-__global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 4) void dwconv_wgrad_dma_kernel(const WgArgs a)
+__global__ __launch_bounds__(Cfg::NT, 4) void dwconv_wgrad_dma_kernel(const WgArgs a)
 {
     constexpr int CG = Cfg::CG, TD = Cfg::TD, TW = Cfg::TW, NT = Cfg::NT, SC = Cfg::SC, PB = Cfg::PB, PDP = Cfg::PDP;
     constexpr int NQ = Cfg::NQ, NSUB = Cfg::NSUB, RG = Cfg::RG, XSLOT = Cfg::XSLOT, GSLOT = Cfg::GSLOT, CPL = Cfg::CPL;
@@ -244,10 +247,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::NT >= 512 ? 4 : 4) void dwconv_wgrad_
         // lane j reads the g slot of plane hp + 1 - j: its slot index runs one step behind lane j - 1's
         int gslot_lane = (1 + NGS - r2) % NGS;
         for (int hp = hs - 1; hp <= he; ++hp) {
-            wait_loads_in_flight<Cfg::template inflight<NTI>()>();
+            wait_loads_in_flight<KEROPS_WD_LOADS ? Cfg::template inflight<NTI>() : 0>();
             __syncthreads();
-            load_x(hp + AX, xs_load);
-            load_g(hp + 1 + AG, gs_load);
+            if (KEROPS_WD_LOADS) {
+                load_x(hp + AX, xs_load);
+                load_g(hp + 1 + AG, gs_load);
+            }
             xs_load = xs_load + 1 == NXS ? 0 : xs_load + 1;
             gs_load = gs_load + 1 == NGS ? 0 : gs_load + 1;
             if (KEROPS_WD_COMPUTE && hp >= 0 && hp < H) {  // wavefront-uniform
@@ -350,10 +355,13 @@ int launch_wgrad_dma(const WgArgs& a, int cg, int tile_w, int tile_d, int depth,
         launch_depth<CGv, TWv, TDv, NTv>(a, depth, stream);   \
         return 0;                                             \
     }
-    KEROPS_WD_CASE(8, 8, 8, 512)
-    KEROPS_WD_CASE(4, 8, 16, 512)
-    KEROPS_WD_CASE(2, 8, 32, 512)
-    KEROPS_WD_CASE(1, 8, 64, 512)
+    // 8-row patches on four wavefronts: each owns four g rows and gathers six x rows for them (ten operand
+    // gathers per 48 matrix instructions; eight wavefronts with two rows each need six per 24), measured 3-8 %
+    // faster at every channel count although half as many wavefronts are resident
+    KEROPS_WD_CASE(8, 8, 8, 256)
+    KEROPS_WD_CASE(4, 8, 16, 256)
+    KEROPS_WD_CASE(2, 8, 32, 256)
+    KEROPS_WD_CASE(1, 8, 64, 256)
     KEROPS_WD_CASE(8, 4, 8, 256)
     KEROPS_WD_CASE(4, 4, 16, 256)
     KEROPS_WD_CASE(2, 4, 32, 256)

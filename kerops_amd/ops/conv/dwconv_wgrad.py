@@ -15,7 +15,7 @@ from .variants import WGRAD_VARIANTS
 # gfx950 launch table, keyed by channel count like the reference's (kerops/ops/conv/dwconv_wgrad.py:10-22):
 # wavefronts per workgroup, tile extents along D and W, kernel family (32 = matrix-core kernel with LDS-direct
 # staging, 16 = matrix-core kernel staged through registers, 2 = vector kernel)
-_WAVES = {8: 8, 16: 8, 32: 8, 64: 8, 128: 8}
+_WAVES = {8: 4, 16: 4, 32: 4, 64: 4, 128: 4}
 _TILE_D = {8: 64, 16: 32, 32: 16, 64: 8, 128: 8}
 _TILE_W = {8: 8, 16: 8, 32: 8, 64: 8, 128: 8}
 _LANE_C = {8: 32, 16: 32, 32: 32, 64: 32, 128: 32}

@@ -24,6 +24,8 @@ WGRAD_VARIANTS = {
 
 def threads_per_workgroup(channels, w_block, d_block, lane_channels):
     """Workgroup size the library uses for a launch shape (fixed per shape inside the library)."""
+    if lane_channels >= 32:
+        return 256  # LDS-direct weight gradient: four wavefronts, each with four (8-row patches) or two g rows
     if lane_channels >= 16:
         slab = min(channels, 64)
         return 512 if w_block * d_block * slab // 8 >= 512 else 256
