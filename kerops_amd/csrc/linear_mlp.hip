@@ -787,6 +787,322 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
     for (int i = t; i < Cfg::RW; i += kMlpThreads) out[i] = red[i];
 }
 
+// ---------------------------------------------------------------------------------------------
+// C = 32 with transposing LDS reads.
+//
+// Same tiles, products and accumulators as lin_brelu_lin_bwd_wave_kernel; what differs is how the "channel per
+// lane" operands of the two weight-gradient products are made.  gfx950 reads LDS transposed: ds_read_b64_tr_b16
+// takes, in every block of 16 lanes, the 16 x 4 matrix M of 16-bit values that the lanes address (lane s supplies
+// the address of four consecutive values M[s][0..3]) and returns to lane i the values M[4 j + i/4][i%4], j = 0..3.
+// With lane s pointing at row s/4, columns 4 (s%4) .. 4 (s%4) + 3 of a row-major [voxel][channel] tile, lane i
+// receives channel i of four consecutive voxels: one instruction transposes a 4 x 16 patch, two of them make the
+// eight reduction values of a 32x32x16 operand.  So the x, g, hid and lg tiles of a wavefront are written to its own
+// LDS area as they sit in the registers (one 64-byte row per voxel) and read back transposed, instead of being
+// multiplied with an identity on the matrix cores and converted back to fp16: 12 of 32 matrix instructions and the
+// conversions of their results go.
+// LDS layout: measured on gfx950, reads see 64 banks of 4 bytes (32 lanes of an 8-byte read or 16 lanes of a 16-byte
+// read per clock), writes see 32 (16 lanes of an 8-byte write, 8 lanes of a 16-byte write per clock).  Chunk c of
+// row r sits in chunk slot c ^ ((r / 2) % 4): the eight rows of a write phase then cover the 128 bytes of write
+// banks once, and a read phase takes whole rows.
+// x and g are fetched as whole rows (one instruction = 16 voxels x 64 bytes = 1 KB of consecutive memory) into the
+// tiles; the lane's own row comes back from there as the operand of the per-voxel products.
+// The hidden channels of a tile row are stored in the order the accumulator leaves them (position p of the row is
+// hidden channel tr_hidden(p) of the 32-block), which only permutes the rows / columns of the gradient blocks.
+// The bias gradient is a product of its own on the 16x16x32 instruction: an operand of ones in row 0 for the even
+// 16-lane groups and in row 1 for the odd ones adds the lg values of hidden positions 0..15 and 16..31.
+struct MrCfg {
+    static constexpr int C = 32, H = 64, MH = 2, KC = 2;
+    static constexpr int RW = 2 * C * H + H;
+    static constexpr int F1_OFF = 0;                              // Wup^T rows   [mh][s]
+    static constexpr int F2_OFF = F1_OFF + MH * KC * 1024;        // Wdown rows   [mh][s]
+    static constexpr int F3_OFF = F2_OFF + MH * KC * 1024;        // Wup rows, hidden order of the accumulator
+    static constexpr int BH_OFF = F3_OFF + 2 * MH * 1024;         // bias
+    static constexpr int WV_OFF = (BH_OFF + H * 2 + 15) / 16 * 16;
+    static constexpr int TILE = 32 * 64;                          // one [32 voxels][32 values] fp16 tile
+    static constexpr int WV_BYTES = 5 * TILE;                     // per wavefront: x, g, hid, lg, dx
+    static constexpr int LOOP_BYTES = WV_OFF + kMlpWaves * WV_BYTES;
+    static constexpr int LDS_BYTES = LOOP_BYTES > RW * 4 ? LOOP_BYTES : RW * 4;
+};
+
+// hidden channel (inside its block of 32) stored at position p of a tile row
+__host__ __device__ constexpr int tr_hidden(int p) { return 16 * (p / 16) + 8 * ((p % 8) / 4) + 4 * ((p / 8) % 2) + p % 4; }
+
+typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 fp16x4_raw_t;
+__device__ __forceinline__ half4_t lds_read_tr16(const unsigned char* p)
+{
+    const auto q = (__attribute__((address_space(3))) fp16x4_raw_t*)(p);
+    return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4f16(q));
+}
+
+__global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_tr_kernel(
+    const half_t* __restrict__ x, const half_t* __restrict__ g, const half_t* __restrict__ Wup,
+    const half_t* __restrict__ Wdown, const half_t* __restrict__ bias, half_t* __restrict__ dx,
+    float* __restrict__ ws, int64_t V)
+{
+    using Cfg = MrCfg;
+    constexpr int C = Cfg::C, H = Cfg::H, MH = Cfg::MH, KC = Cfg::KC, TILE = Cfg::TILE;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
+    half_t* f1w = reinterpret_cast<half_t*>(smem + Cfg::F1_OFF);
+    half_t* f3w = reinterpret_cast<half_t*>(smem + Cfg::F3_OFF);
+    half_t* bsh = reinterpret_cast<half_t*>(smem + Cfg::BH_OFF);
+
+    const int t = threadIdx.x, lane = t % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(t / kWave);  // scalar: tile indices stay wavefront-uniform
+    const int il = lane % 32, hl = lane / 32;
+    const half8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // hidden channel (within a block of 32) that element j of reduction group `half` of lane half hl holds
+    auto hperm = [](int half, int hl_, int j) { return 16 * half + 8 * (j / 4) + 4 * hl_ + j % 4; };
+
+    for (int i = t; i < MH * KC * 512; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, s = (i / 512) % KC, mh = i / (512 * KC);
+        f1w[i] = Wup[(16 * s + 8 * (l / 32) + j) * H + 32 * mh + l % 32];
+    }
+    for (int i = t; i < MH * KC * 64; i += kMlpThreads) {
+        const int l = i % 64, s = (i / 64) % KC, mh = i / (64 * KC);
+        reinterpret_cast<half8_t*>(smem + Cfg::F2_OFF)[i] = load_c8(Wdown + (32 * mh + l % 32) * C + 16 * s + 8 * (l / 32));
+    }
+    for (int i = t; i < 2 * MH * 512; i += kMlpThreads) {
+        const int j = i % 8, l = (i / 8) % 64, f = i / 512;
+        f3w[i] = Wup[(l % 32) * H + 32 * (f / 2) + hperm(f % 2, l / 32, j)];
+    }
+    for (int i = t; i < H; i += kMlpThreads) bsh[i] = bias[i];
+    __syncthreads();
+
+    const half8_t* f1 = reinterpret_cast<const half8_t*>(smem + Cfg::F1_OFF) + lane;
+    const half8_t* f2 = reinterpret_cast<const half8_t*>(smem + Cfg::F2_OFF) + lane;
+    const half8_t* f3 = reinterpret_cast<const half8_t*>(smem + Cfg::F3_OFF) + lane;
+    unsigned char* mine = smem + Cfg::WV_OFF + wave * Cfg::WV_BYTES;
+    unsigned char* xt = mine;             // [32 voxels][32 channels]
+    unsigned char* gt = mine + TILE;
+    unsigned char* ht = mine + 2 * TILE;  // [32 voxels][32 hidden positions] of the current block
+    unsigned char* lt = mine + 3 * TILE;
+    unsigned char* dt = mine + 4 * TILE;  // [32 voxels][32 channels] of dx
+
+    // the lane's row: 16-byte chunks hl and 2 + hl
+    const int wsw = (il >> 1) & 3;
+    const int woff0 = il * 64 + ((hl ^ wsw) * 16), woff1 = il * 64 + (((2 + hl) ^ wsw) * 16);
+    // the fetched chunk: row lane / 4 (+ 16 for the second instruction: the same swizzle term), chunk lane % 4
+    const int foff = (lane / 4) * 64 + (((lane % 4) ^ ((lane >> 3) & 3)) * 16);
+    // transposing read of reduction half hf: lane (il, hl) receives position il of the voxels 16 hf + 8 hl + 0..7;
+    // inside its block of 16 lanes, lane s addresses row 8 hl + 4 r + s/4, positions 16 (block % 2) + 4 (s%4) ..
+    // (rows 16 hf + ...: the swizzle term (row / 2) % 4 does not depend on hf)
+    int toff[2];
+    {
+        const int s = lane % 16, blk = lane / 16;
+        const int pos = 16 * (blk % 2) + 4 * (s % 4);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int row = 8 * (blk / 2) + 4 * r + s / 4;
+            toff[r] = row * 64 + (((pos / 8) ^ ((row >> 1) & 3)) * 16) + (pos % 8) * 2;
+        }
+    }
+    auto read_T = [&](const unsigned char* tile, int hf) {
+        const half4_t a = lds_read_tr16(tile + hf * 1024 + toff[0]);
+        const half4_t b = lds_read_tr16(tile + hf * 1024 + toff[1]);
+        return half8_t{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    };
+    auto wave_sync = [] {  // LDS operations of one wavefront complete in issue order: only the compiler must not reorder
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    // bias gradient: ones in row 0 for the even 16-lane groups, in row 1 for the odd ones
+    const half_t one_h = (lane % 16) == ((lane / 16) % 2) ? (half_t)1 : (half_t)0;
+    const half8_t ones = {one_h, one_h, one_h, one_h, one_h, one_h, one_h, one_h};
+
+    float16_t wdn[MH], wup[MH];  // dWdown block: D[h][c];  dWup block: D[c][h]
+    float4_t bacc[MH];
+#pragma unroll
+    for (int mh = 0; mh < MH; ++mh) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wdn[mh][i] = wup[mh][i] = 0.0f;
+        bacc[mh] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    const int64_t ntiles = (V + 31) / 32;
+    const int64_t stride = (int64_t)gridDim.x * kMlpWaves;
+    half8_t xn[KC], gn[KC];
+    // one instruction fetches 16 whole rows (1 KB): lane -> 16-byte chunk lane % 4 of voxel 16 s + lane / 4
+    // (rows past V read the last voxel and are zeroed before use)
+    auto fetch = [&](int64_t tile) {
+#pragma unroll
+        for (int s = 0; s < KC; ++s) {
+            int64_t v = tile * 32 + 16 * s + lane / 4;
+            v = v < V ? v : V - 1;
+            xn[s] = load_c8_nt(x + v * C + (lane % 4) * 8);
+            gn[s] = load_c8_nt(g + v * C + (lane % 4) * 8);
+        }
+    };
+
+    // dx leaves one tile late: the wait for the operands of a tile then only covers stores issued a whole
+    // tile earlier (the memory counter retires loads and stores in issue order)
+    auto flush = [&](int64_t pv0, bool ragged) {
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {  // lane -> 16-byte chunk lane % 4 of row 16 pass + lane / 4
+            const int row = 16 * pass + lane / 4, cc = lane % 4;
+            if (!ragged || pv0 + row < V) {
+                const half8_t o = *reinterpret_cast<const half8_t*>(dt + row * 64 + ((cc ^ ((row >> 1) & 3)) * 16));
+                // rows 8..15 and 24..31 hold the two 8-byte halves of a chunk swapped
+                const bool sw = (row >> 3) & 1;
+                const half8_t w = {sw ? o[4] : o[0], sw ? o[5] : o[1], sw ? o[6] : o[2], sw ? o[7] : o[3],
+                                   sw ? o[0] : o[4], sw ? o[1] : o[5], sw ? o[2] : o[6], sw ? o[3] : o[7]};
+                store_c8_nt(dx + (pv0 + row) * C + cc * 8, w);
+            }
+        }
+        wave_sync();
+    };
+
+    const int64_t first = (int64_t)blockIdx.x * kMlpWaves + wave;
+    int64_t tile = first;
+    if (tile < ntiles) fetch(tile);
+    for (; tile < ntiles; tile += stride) {
+        const int64_t v0 = tile * 32;
+        half8_t xc[KC], gc[KC];
+#pragma unroll
+        for (int s = 0; s < KC; ++s) {
+            xc[s] = xn[s];
+            gc[s] = gn[s];
+        }
+        if (v0 + 32 > V) {  // ragged last tile (wavefront-uniform)
+#pragma unroll
+            for (int s = 0; s < KC; ++s) {
+                const bool ok = v0 + 16 * s + lane / 4 < V;
+                xc[s] = ok ? xc[s] : z8;
+                gc[s] = ok ? gc[s] : z8;
+            }
+        }
+        if (tile != first) flush(v0 - stride * 32, false);  // an earlier tile of this wavefront is never ragged
+        {
+            const int64_t nt = tile + stride;
+            fetch(nt < ntiles ? nt : tile);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // x and g into the tiles as fetched; back as the lane's own row (chunks hl and 2 + hl: the operands of the
+        // per-voxel products) and transposed
+        *reinterpret_cast<half8_t*>(xt + foff) = xc[0];
+        *reinterpret_cast<half8_t*>(xt + 1024 + foff) = xc[1];
+        *reinterpret_cast<half8_t*>(gt + foff) = gc[0];
+        *reinterpret_cast<half8_t*>(gt + 1024 + foff) = gc[1];
+        wave_sync();
+        xc[0] = *reinterpret_cast<const half8_t*>(xt + woff0);
+        xc[1] = *reinterpret_cast<const half8_t*>(xt + woff1);
+        gc[0] = *reinterpret_cast<const half8_t*>(gt + woff0);
+        gc[1] = *reinterpret_cast<const half8_t*>(gt + woff1);
+        half8_t xT[2], gT[2];  // lane = channel, registers = voxels 16 hf + 8 hl + 0..7
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            xT[hf] = read_T(xt, hf);
+            gT[hf] = read_T(gt, hf);
+        }
+
+        float16_t dacc;  // dx^T: D[c][v]
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dacc[i] = 0.0f;
+
+            // (measurement switch: -DKEROPS_MLP_MH=0 builds the kernel without its arithmetic, i.e. the time of its
+            // memory traffic alone: 0.56 ms at (1,32,350,350,128) against 0.61 ms with the arithmetic; two more tiles
+            // in flight per wavefront change neither, half as many wavefronts per compute unit bring the traffic
+            // alone to 0.52 ms and the whole kernel to 0.69 ms)
+#ifndef KEROPS_MLP_MH
+#define KEROPS_MLP_MH MH
+#endif
+#pragma unroll
+        for (int mh = 0; mh < KEROPS_MLP_MH; ++mh) {
+            float16_t up, dn;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) up[i] = dn[i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KC; ++s) {
+                up = __builtin_amdgcn_mfma_f32_32x32x16_f16(f1[(mh * KC + s) * 64], xc[s], up, 0, 0, 0);
+                dn = __builtin_amdgcn_mfma_f32_32x32x16_f16(f2[(mh * KC + s) * 64], gc[s], dn, 0, 0, 0);
+            }
+            // up[i], dn[i]: hidden channel 32 mh + 8 (i/4) + 4 hl + i%4 of voxel il
+            half8_t hv[2], lv[2];
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const half4_t b4 = *reinterpret_cast<const half4_t*>(bsh + 32 * mh + 8 * gq + 4 * hl);
+#pragma unroll
+                for (int jp = 0; jp < 2; ++jp) {
+                    const int i = 4 * gq + 2 * jp, e = 4 * (gq % 2) + 2 * jp;
+                    half2_t hid, lg;
+                    hid_lg_pair(up[i], up[i + 1], dn[i], dn[i + 1], half2_t{b4[2 * jp], b4[2 * jp + 1]}, hid, lg);
+                    hv[gq / 2][e] = hid[0];
+                    hv[gq / 2][e + 1] = hid[1];
+                    lv[gq / 2][e] = lg[0];
+                    lv[gq / 2][e + 1] = lg[1];
+                }
+            }
+            // rows past V hold x = g = 0: hid = relu(bias) there meets g = 0 in dWdown, lg = 0 everywhere else
+            dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(f3[(2 * mh) * 64], lv[0], dacc, 0, 0, 0);
+            dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(f3[(2 * mh + 1) * 64], lv[1], dacc, 0, 0, 0);
+
+            // hid and lg rows of the voxel (positions 8 (2 f + hl) + e) into the tiles, back transposed
+            wave_sync();  // (the reads of the previous block are issued)
+            *reinterpret_cast<half8_t*>(ht + woff0) = hv[0];
+            *reinterpret_cast<half8_t*>(ht + woff1) = hv[1];
+            *reinterpret_cast<half8_t*>(lt + woff0) = lv[0];
+            *reinterpret_cast<half8_t*>(lt + woff1) = lv[1];
+            wave_sync();
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const half8_t hT = read_T(ht, hf), lT = read_T(lt, hf);  // lane = hidden position il
+                wdn[mh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hT, gT[hf], wdn[mh], 0, 0, 0);
+                wup[mh] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xT[hf], lT, wup[mh], 0, 0, 0);
+                bacc[mh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, lT, bacc[mh], 0, 0, 0);
+            }
+        }
+
+        // ---- dx: row il of the wavefront's tile, 8 bytes (channels 8 gq + 4 hl + 0..3) at a time; the two halves
+        // of a chunk are swapped in every second group of eight rows so that the 16 lanes of a write phase hit 16
+        // different pairs of the 32 write banks ----
+#pragma unroll
+        for (int gq = 0; gq < C / 8; ++gq) {
+            half4_t o;
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)dacc[4 * gq + jj];
+            *reinterpret_cast<half4_t*>(dt + il * 64 + ((gq ^ wsw) * 16) + ((hl ^ ((il >> 3) & 1)) * 8)) = o;
+        }
+        wave_sync();
+    }
+    if (first < ntiles) flush((tile - stride) * 32, true);
+
+    // ---- the four wavefronts add their partials in LDS, wavefront 0 first: [dWup C*H][dWdown H*C][dbias H] ----
+    float* red = reinterpret_cast<float*>(smem);
+    __syncthreads();  // every wavefront is done with the fragments
+#pragma unroll 1
+    for (int w = 0; w < kMlpWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int mh = 0; mh < MH; ++mh) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int ri = 8 * (i / 4) + 4 * hl + i % 4;  // row of the block held in register i
+                    {  // dWdown[h = 32 mh + hidden of position ri][c = il]
+                        float* p = red + C * H + (32 * mh + tr_hidden(ri)) * C + il;
+                        *p = w == 0 ? wdn[mh][i] : *p + wdn[mh][i];
+                    }
+                    {  // dWup[c = ri][h = 32 mh + hidden of position il]
+                        float* p = red + ri * H + 32 * mh + tr_hidden(il);
+                        *p = w == 0 ? wup[mh][i] : *p + wup[mh][i];
+                    }
+                }
+                if (lane < 16) {  // rows 0 and 1 of the 16x16 block: hidden positions lane and 16 + lane
+#pragma unroll
+                    for (int r = 0; r < 2; ++r) {
+                        float* p = red + 2 * C * H + 32 * mh + tr_hidden(16 * r + lane);
+                        *p = w == 0 ? bacc[mh][r] : *p + bacc[mh][r];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = ws + (int64_t)blockIdx.x * Cfg::RW;
+    for (int i = t; i < Cfg::RW; i += kMlpThreads) out[i] = red[i];
+}
+
 // sums the rows of the partial buffer in a fixed order (16 columns per workgroup, 64 interleaved row slices with four
 // loads in flight, fixed tree in LDS; fp64) and scatters the three results
 __global__ __launch_bounds__(1024) void mlp_reduce_kernel(const float* __restrict__ ws, int nrows, int RW, int n_up,
@@ -889,8 +1205,21 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
         return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
     }
     KEROPS_MT_CASE(16)
+#ifdef KEROPS_MLP_BWD32_IDENTITY  // (comparison build: the identity-product transposes at C = 32 as well)
     KEROPS_MT_CASE(32)
+#endif
 #undef KEROPS_MT_CASE
+    if (C == 32) {
+        hipLaunchKernelGGL(lin_brelu_lin_bwd_tr_kernel, dim3(blocks), dim3(kMlpThreads), 0, s, (const half_t*)x,
+                           (const half_t*)g, (const half_t*)Wup, (const half_t*)Wdown, (const half_t*)bias, (half_t*)dx,
+                           ws, V);
+        int rc = check_launch("lin_brelu_lin_bwd");
+        if (rc != KEROPS_OK) return rc;
+        const int RW = MrCfg::RW;
+        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws, blocks, RW, 2 * 32 * 32,
+                           2 * 32 * 32, dWup, dWdown, dbias);
+        return check_launch("lin_brelu_lin_bwd_reduce");
+    }
 #define KEROPS_MB_CASE(CV)                                                                                        \
     if (C == CV) {                                                                                                \
         hipLaunchKernelGGL((lin_brelu_lin_bwd_kernel<CV>), dim3(blocks), dim3(kMlpThreads), 0, s,                \
