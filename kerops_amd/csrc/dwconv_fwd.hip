@@ -587,9 +587,14 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
     int boff[3];
 #pragma unroll
     for (int k = 0; k < 3; ++k) boff[k] = lds_swizzle<PB>(ra * PDP + pgrp + rr + k, cb);
-    // output tile: the halves of odd positions are swapped so that the four positions of a write spread over all banks
+    // output tile: LDS writes see 32 banks of 4 bytes (measured: 32 lanes of a dword write per clock), and half a
+    // wavefront writes 8 dwords at each of four consecutive positions; the positions' bytes are rotated so that those
+    // four runs fall into four different quarters of the 128 bytes of banks (no measurable change in time: the LDS
+    // is a third busy in this kernel)
     auto ot_swz = [](int pos, int cbyte) {
-        return PB == 128 ? pos * PB + ((cbyte + 64 * (pos & 1)) & 127) : pos * PB + cbyte;
+        return PB == 128  ? pos * PB + ((cbyte + 32 * (pos & 3)) & 127)
+               : PB == 64 ? pos * PB + ((cbyte + 32 * ((pos >> 1) & 1)) & 63)
+                          : pos * PB + cbyte;
     };
     int owr[RO];  // the lane's dword (two channels) of position pgrp + rr in the output rows ra .. ra+RO-1
 #pragma unroll
