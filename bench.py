@@ -107,6 +107,10 @@ def parse():
     ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the CPU legs (used under rocprofv3)')
     ap.add_argument('--no-extra-ops', action='store_true', help='time only the DWConv step')
     ap.add_argument('--no-clock-probe', action='store_true', help='skip the core-clock-under-load side figure')
+    ap.add_argument('--one-shape-per-kernel', action='store_true',
+                    help='counter runs: leave out the launches that run a kernel template at a second tensor size '
+                         '(stream ops and fused backward at the other channel counts, the C=128 convolution rows), so '
+                         'that per-kernel averages of a profiler are averages over one shape')
     return ap.parse_args()
 
 
@@ -406,6 +410,8 @@ def main():
                 ('DequantUint8Window', lambda: DequantUint8Window(q8c, torch.float16, 3.0), 3 * vc),
                 ('QuantInt8Sym', lambda: QuantInt8Sym(xc, amax), 3 * vc),
             ]
+            if args.one_shape_per_kernel:
+                cases = cases[:-1]  # (QuantInt8Sym runs at the config-5 shape below)
             rows = {}
             for name, fn, nb in cases:
                 ms_ = time_op(torch, fn, it, wm)[0]
@@ -422,6 +428,8 @@ def main():
                                  'dwconv_frac_hbm_peak': fwd['frac_hbm_peak'],
                                  'wgrad_frac_hbm_peak': wg['frac_hbm_peak']}
                 continue
+            if args.one_shape_per_kernel and c in (64, 128):  # (these two share their kernel templates)
+                continue
             x = g = None
             torch.cuda.empty_cache()
             x, g, wkc = make(c)
@@ -435,7 +443,8 @@ def main():
                              'wgrad_frac_hbm_peak': round(4 * V * c / wgm / 1e6 / HBM_PEAK_GBPS, 4),
                              'backward_fused_ms': round(bwm, 4),
                              'backward_fused_frac_hbm_peak': round(6 * V * c / bwm / 1e6 / HBM_PEAK_GBPS, 4)}
-            stream_table[str(c)] = stream_rows(x, g, c)
+            if not args.one_shape_per_kernel:
+                stream_table[str(c)] = stream_rows(x, g, c)
         table[str(C)]['backward_fused_ms'] = ops['DWConvBackward_fused']['ms']
         table[str(C)]['backward_fused_frac_hbm_peak'] = ops['DWConvBackward_fused']['frac_hbm_peak']
         ops['stream_ops_by_channels'] = {str(c): stream_table[str(c)] for c in (8, 16, 32, 64, 128) if str(c) in stream_table}
