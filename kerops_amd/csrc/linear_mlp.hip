@@ -802,8 +802,9 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
 // conversions of their results go.
 // LDS layout: measured on gfx950, reads see 64 banks of 4 bytes (32 lanes of an 8-byte read or 16 lanes of a 16-byte
 // read per clock), writes see 32 (16 lanes of an 8-byte write, 8 lanes of a 16-byte write per clock).  Chunk c of
-// row r sits in chunk slot c ^ ((r / 2) % 4): the eight rows of a write phase then cover the 128 bytes of write
-// banks once, and a read phase takes whole rows.
+// row r sits in chunk slot c ^ tr_slot(r) = c ^ ((r / 2) % 4) ^ ((r / 8) % 2): the eight rows of a write phase then
+// cover the 128 bytes of write banks once, the sixteen rows of a 16-byte read phase (the same chunk of each) the 256
+// of read banks once, and a transposing read phase takes four whole rows.
 // x and g are fetched as whole rows (one instruction = 16 voxels x 64 bytes = 1 KB of consecutive memory) into the
 // tiles; the lane's own row comes back from there as the operand of the per-voxel products.
 // The hidden channels of a tile row are stored in the order the accumulator leaves them (position p of the row is
@@ -824,6 +825,8 @@ struct MrCfg {
     static constexpr int LDS_BYTES = LOOP_BYTES > RW * 4 ? LOOP_BYTES : RW * 4;
 };
 
+// chunk-slot swizzle of tile row r (unchanged by r + 16)
+__host__ __device__ constexpr int tr_slot(int r) { return ((r >> 1) & 3) ^ ((r >> 3) & 1); }
 // hidden channel (inside its block of 32) stored at position p of a tile row
 __host__ __device__ constexpr int tr_hidden(int p) { return 16 * (p / 16) + 8 * ((p % 8) / 4) + 4 * ((p / 8) % 2) + p % 4; }
 
@@ -880,13 +883,13 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_tr_kernel(
     unsigned char* dt = mine + 4 * TILE;  // [32 voxels][32 channels] of dx
 
     // the lane's row: 16-byte chunks hl and 2 + hl
-    const int wsw = (il >> 1) & 3;
+    const int wsw = tr_slot(il);
     const int woff0 = il * 64 + ((hl ^ wsw) * 16), woff1 = il * 64 + (((2 + hl) ^ wsw) * 16);
     // the fetched chunk: row lane / 4 (+ 16 for the second instruction: the same swizzle term), chunk lane % 4
-    const int foff = (lane / 4) * 64 + (((lane % 4) ^ ((lane >> 3) & 3)) * 16);
+    const int foff = (lane / 4) * 64 + (((lane % 4) ^ tr_slot(lane / 4)) * 16);
     // transposing read of reduction half hf: lane (il, hl) receives position il of the voxels 16 hf + 8 hl + 0..7;
     // inside its block of 16 lanes, lane s addresses row 8 hl + 4 r + s/4, positions 16 (block % 2) + 4 (s%4) ..
-    // (rows 16 hf + ...: the swizzle term (row / 2) % 4 does not depend on hf)
+    // (rows 16 hf + ...: the swizzle term does not depend on hf)
     int toff[2];
     {
         const int s = lane % 16, blk = lane / 16;
@@ -894,7 +897,7 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_tr_kernel(
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const int row = 8 * (blk / 2) + 4 * r + s / 4;
-            toff[r] = row * 64 + (((pos / 8) ^ ((row >> 1) & 3)) * 16) + (pos % 8) * 2;
+            toff[r] = row * 64 + (((pos / 8) ^ tr_slot(row)) * 16) + (pos % 8) * 2;
         }
     }
     auto read_T = [&](const unsigned char* tile, int hf) {
@@ -942,7 +945,7 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_tr_kernel(
         for (int pass = 0; pass < 2; ++pass) {  // lane -> 16-byte chunk lane % 4 of row 16 pass + lane / 4
             const int row = 16 * pass + lane / 4, cc = lane % 4;
             if (!ragged || pv0 + row < V) {
-                const half8_t o = *reinterpret_cast<const half8_t*>(dt + row * 64 + ((cc ^ ((row >> 1) & 3)) * 16));
+                const half8_t o = *reinterpret_cast<const half8_t*>(dt + row * 64 + ((cc ^ tr_slot(row)) * 16));
                 // rows 8..15 and 24..31 hold the two 8-byte halves of a chunk swapped
                 const bool sw = (row >> 3) & 1;
                 const half8_t w = {sw ? o[4] : o[0], sw ? o[5] : o[1], sw ? o[6] : o[2], sw ? o[7] : o[3],
