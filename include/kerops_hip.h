@@ -98,9 +98,13 @@ int kerops_dwconv_stats_f16(const void* x, const void* wt, void* y, float* mean,
  *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]
  * gw is [3][3][3][C] fp32.  Deterministic: per-workgroup partials go to the
  * workspace and a second kernel adds them in a fixed order.
- * lane_channels selects the kernel family: 16 = matrix-core kernels (one 4x4x4
- * MFMA block per channel, 16 channels per instruction; the built-in choice),
- * 2 = vector kernels (two channels per lane, 2-way fp16 dot products).
+ * lane_channels selects the kernel family: 32 = matrix-core kernel (one 4x4x4
+ * MFMA block per channel) with planes loaded straight into LDS and 8-byte operand
+ * reads, on 8-row patches of 512 16-byte chunks (tile_w 8, tile_d 64 / 32 / 16 / 8 for
+ * C = 8 / 16 / 32 / 64 and more; the built-in choice) or 4-row patches of 256; 33 / 34 / 35 = the same with one / two /
+ * one x and two g planes in flight ahead of the arithmetic; 16 = matrix-core kernels
+ * staged through registers; 2 = vector kernels (two channels per lane, 2-way fp16
+ * dot products).
  * Replaces the zero-filled partial buffer, the `_DWConv_wgrad_cl3d_impl[grid](...)`
  * launches and the trailing `grad_w.sum(dim=(0, 1))`:
  * kerops/ops/conv/dwconv_wgrad.py:54-77 (kernel kerops/kernels/dw_conv.py:147-287). */
@@ -129,7 +133,9 @@ int kerops_dwconv_wgrad_noalloc_f16(const void* x, const void* g, float* gw, int
  *   dx[n,h,w,d,c] = sum_{kh,kw,kd} g[n,h-kh+1,w-kw+1,d-kd+1,c] * wt[kh,kw,kd,c]      (fp16, one rounding)
  *   gw[kh,kw,kd,c] = sum_{n,h,w,d} g[n,h,w,d,c] * x[n,h+kh-1,w+kw-1,d+kd-1,c]        (fp32, deterministic)
  * Every plane of g is staged once and feeds both products, which saves one of the two reads of g that
- * kerops_dwconv_fwd_f16(g, flipped wt) + kerops_dwconv_wgrad_f16 need.  C in {8,16,32,64,128}. */
+ * kerops_dwconv_fwd_f16(g, flipped wt) + kerops_dwconv_wgrad_f16 need.  C in {8,16,32,64,128}.
+ * The environment variable KEROPS_BWD_STAGING=registers (read at every call of either function) selects the
+ * earlier kernel that stages the planes through registers; dx is bit-identical, gw differs in the last bits. */
 int64_t kerops_dwconv_bwd_workspace_bytes(int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t h_chunk);
 int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* wt, void* dx, float* gw, void* workspace,
                           int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
