@@ -376,6 +376,87 @@ __device__ __forceinline__ void store_c8_nt(half_t* p, half8_t v)
     __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(p));
 }
 
+// ---- LDS tile for results that leave the accumulators in 8-byte pieces and LDS in 16-byte chunks ---------------
+// A 32x32x16 accumulator holds, per lane (row = lane % 32, half = lane / 32), groups of four consecutive output
+// channels: the 8-byte half `half` of the 16-byte chunk `chunk` of the row.  The rows leave LDS as 16-byte chunks,
+// lane c taking chunk c % CPR of row c / CPR, for coalesced stores.  Measured on gfx950, LDS writes see 32 banks of
+// 4 bytes (16 lanes of an 8-byte write per clock) and reads 64 (16 lanes of a 16-byte read per clock).  Rows are
+// dense (2 * COLS bytes), so the 16 lanes of a read phase take 256 consecutive bytes whatever the order inside a
+// row; inside a row the chunk slot and the half are flipped by bits of the row number, chosen so that the 16 rows
+// of a write phase (same chunk, same half) fall on 16 different bank pairs.
+template <int COLS>
+struct BounceTile {
+    static constexpr int CPR = COLS / 8, RB = 2 * COLS;     // chunks per row, bytes per row
+    static constexpr int RPW = RB >= 128 ? 1 : 128 / RB;    // rows per 128 bytes of write banks
+    static constexpr int SW = CPR < 8 ? CPR : 8;            // chunk slots that differ in their write banks
+    static constexpr int BYTES = 32 * RB;
+    static_assert(COLS == 16 || COLS == 32 || COLS == 64 || COLS == 128, "row widths of the built kernels");
+    // byte offset of the 8-byte piece (row, chunk, half)
+    __device__ static constexpr int piece(int row, int chunk, int half)
+    {
+        return row * RB + ((chunk ^ ((row / RPW) % SW)) * 16) + ((half ^ (((row / RPW) / SW) & 1)) * 8);
+    }
+    // byte offset of the 16-byte chunk (row, chunk); its two halves are swapped where halves_swapped(row)
+    __device__ static constexpr int chunk16(int row, int chunk) { return row * RB + ((chunk ^ ((row / RPW) % SW)) * 16); }
+    __device__ static constexpr bool halves_swapped(int row) { return (((row / RPW) / SW) & 1) != 0; }
+    __device__ static half8_t read(const unsigned char* tile, int row, int chunk)
+    {
+        const half8_t r = *reinterpret_cast<const half8_t*>(tile + chunk16(row, chunk));
+        const bool sw = halves_swapped(row);
+        return half8_t{sw ? r[4] : r[0], sw ? r[5] : r[1], sw ? r[6] : r[2], sw ? r[7] : r[3],
+                       sw ? r[0] : r[4], sw ? r[1] : r[5], sw ? r[2] : r[6], sw ? r[3] : r[7]};
+    }
+};
+
+// ---- LDS tile of dense [voxel][channel] fp16 rows that is written as 16-byte chunks, read as 16-byte chunks of
+// one voxel (matrix operands with the voxel per lane) and read transposed (operands with the channel per lane) -----
+// gfx950 reads LDS transposed: ds_read_b64_tr_b16 takes, in every block of 16 lanes, the 16 x 4 matrix M of 16-bit
+// values that the lanes address (lane s supplies the address of four consecutive values M[s][0..3]) and returns to
+// lane i the values M[4 j + i/4][i%4], j = 0..3.  With lane s pointing at row s/4, columns 4 (s%4) .. 4 (s%4) + 3
+// of a row-major tile, lane i receives column i of four consecutive rows: two such reads make the eight reduction
+// values (rows 16 s + 8 (lane/32) + 0..7) of a 32x32x16 operand whose lane index is the column.
+// Chunk c of row r sits in chunk slot c ^ slot(r).  slot(r) is chosen so that (measured bank structure: 64 banks
+// of 4 bytes for reads, 32 for writes) the 16 rows of a 16-byte read phase that takes the same chunk of each fall
+// on different banks, the four rows of a transposing read phase (64 bytes of each) likewise, and writes of whole
+// rows are conflict-free by construction.
+typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 fp16x4_raw_t;
+__device__ __forceinline__ half4_t lds_read_tr16(const unsigned char* p)
+{
+    const auto q = (__attribute__((address_space(3))) fp16x4_raw_t*)(p);
+    return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4f16(q));
+}
+template <int COLS>
+struct SwizzledRows {
+    static constexpr int CPR = COLS / 8, RB = 2 * COLS;
+    static_assert(COLS == 16 || COLS == 32 || COLS == 64 || COLS == 128, "row widths of the built kernels");
+    __device__ static constexpr int slot(int r)
+    {
+        return CPR == 2   ? ((r >> 3) & 1)
+               : CPR == 4 ? ((r >> 2) & 3)
+               : CPR == 8 ? ((((r >> 1) & 1) << 2) | ((r >> 2) & 3))
+                          : (((r & 3) << 2) | ((r >> 2) & 3));
+    }
+    __device__ static constexpr int chunk16(int row, int chunk) { return row * RB + ((chunk ^ slot(row)) * 16); }
+    // Per-lane byte offsets of the two transposing reads of reduction step 0 for the 32-column block `blk32`
+    // (columns 32 blk32 + lane % 32; a 16-column tile repeats its columns); step s adds s * 16 * RB.
+    __device__ static void tr_offsets(int lane, int blk32, int (&off)[2])
+    {
+        const int s = lane % 16, b16 = COLS >= 32 ? (lane / 16) % 2 : 0, hl = lane / 32;
+        const int col = 32 * blk32 + 16 * b16 + 4 * (s % 4);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int row = 8 * hl + 4 * r + s / 4;
+            off[r] = chunk16(row, col / 8) + (col % 8) * 2;
+        }
+    }
+    __device__ static half8_t read_tr(const unsigned char* tile, const int (&off)[2], int step)
+    {
+        const half4_t a = lds_read_tr16(tile + step * 16 * RB + off[0]);
+        const half4_t b = lds_read_tr16(tile + step * 16 * RB + off[1]);
+        return half8_t{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    }
+};
+
 // ---- wavefront reductions -----------------------------------------------------
 // Sum over the lanes of a wavefront whose index differs only in bits >= log2(stride_lo):
 // i.e. lanes l and l' are combined when l % stride_lo == l' % stride_lo.

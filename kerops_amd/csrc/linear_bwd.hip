@@ -34,7 +34,7 @@ struct LbCfg {
     static constexpr int MTI = (CIN + 31) / 32, MTO = (COUT + 31) / 32;  // 32-channel blocks
     static constexpr int KSO = COUT / 16;                                 // k steps of the dx product
     static constexpr int KSV = kLbTile / 16;                              // k steps (voxels) of the dW product
-    static constexpr int XP = CIN + 8, GP = COUT + 8, DP = CIN + 4;       // LDS row pitches in halves
+    static constexpr int XP = CIN, GP = COUT, DP = CIN;  // dense rows (halves); swizzled: SwizzledRows / BounceTile in common.hpp
     static constexpr int NBD = 2 * MTI;                                   // dx blocks (32 voxels x 32 channels) per tile
     static constexpr int NBW = MTI * MTO;                                 // dW blocks
     static constexpr int KSPL = NBW >= kLbWaves ? 1 : kLbWaves / NBW;     // voxel split when blocks are few
@@ -62,8 +62,10 @@ __global__ __launch_bounds__(kLbThreads) void relu_linear_bwd_kernel(const half_
     constexpr int XP = Cfg::XP, GP = Cfg::GP, DP = Cfg::DP, KSO = Cfg::KSO, KSV = Cfg::KSV;
     constexpr int NLX = Cfg::NLX, NLG = Cfg::NLG, BPW = Cfg::BPW, KSPL = Cfg::KSPL;
     __shared__ __attribute__((aligned(16))) unsigned char smem[Cfg::LDS_BYTES];
-    half_t* xs = reinterpret_cast<half_t*>(smem + Cfg::XS_OFF);
-    half_t* gs = reinterpret_cast<half_t*>(smem + Cfg::GS_OFF);
+    unsigned char* xs = smem + Cfg::XS_OFF;
+    unsigned char* gs = smem + Cfg::GS_OFF;
+    using XT = SwizzledRows<CIN>;
+    using GT = SwizzledRows<COUT>;
     half_t* ds = reinterpret_cast<half_t*>(smem + Cfg::DS_OFF);
     half8_t* wl = reinterpret_cast<half8_t*>(smem + Cfg::WL_OFF);
 
@@ -113,12 +115,12 @@ __global__ __launch_bounds__(kLbThreads) void relu_linear_bwd_kernel(const half_
 #pragma unroll
         for (int j = 0; j < NLX; ++j) {
             const int c = t + j * kLbThreads;
-            if (c < Cfg::NXC) *reinterpret_cast<half8_t*>(xs + (c / (CIN / 8)) * XP + (c % (CIN / 8)) * 8) = xpre[j];
+            if (c < Cfg::NXC) *reinterpret_cast<half8_t*>(xs + XT::chunk16(c / (CIN / 8), c % (CIN / 8))) = xpre[j];
         }
 #pragma unroll
         for (int j = 0; j < NLG; ++j) {
             const int c = t + j * kLbThreads;
-            if (c < Cfg::NGC) *reinterpret_cast<half8_t*>(gs + (c / (COUT / 8)) * GP + (c % (COUT / 8)) * 8) = gpre[j];
+            if (c < Cfg::NGC) *reinterpret_cast<half8_t*>(gs + GT::chunk16(c / (COUT / 8), c % (COUT / 8))) = gpre[j];
         }
         __syncthreads();
         if (tile + gridDim.x < ntiles) prefetch(tile + gridDim.x);
@@ -129,13 +131,14 @@ __global__ __launch_bounds__(kLbThreads) void relu_linear_bwd_kernel(const half_
             const int blk = wave + bd * kLbWaves;
             if (blk < Cfg::NBD) {  // wavefront-uniform
                 const int vt = blk % 2, mt = blk / 2;
-                const half_t* grow = gs + (32 * vt + il) * GP + 8 * hl;
+                // chunk 2 s + hl of the lane's voxel row: the swizzle is an XOR, so step s is the offset of step 0 ^ 32 s
+                const int grow = GT::chunk16(32 * vt + il, hl);
                 float16_t acc;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 #pragma unroll
                 for (int s = 0; s < KSO; ++s) {
-                    const half8_t bfrag = *reinterpret_cast<const half8_t*>(grow + 16 * s);
+                    const half8_t bfrag = *reinterpret_cast<const half8_t*>(gs + (grow ^ (32 * s)));
                     acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(wl[(mt * KSO + s) * 64 + lane], bfrag, acc, 0, 0, 0);
                 }
                 // acc[i]: input channel 32 mt + 8 (i/4) + 4 hl + i%4 of voxel 32 vt + il
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(kLbThreads) void relu_linear_bwd_kernel(const half_
                         half4_t o;
 #pragma unroll
                         for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)acc[4 * gq + jj];
-                        *reinterpret_cast<half4_t*>(ds + (32 * vt + il) * DP + ci) = o;
+                        *reinterpret_cast<half4_t*>(reinterpret_cast<unsigned char*>(ds) + BounceTile<CIN>::piece(32 * vt + il, 4 * mt + gq, hl)) = o;
                     }
                 }
             }
@@ -157,19 +160,14 @@ __global__ __launch_bounds__(kLbThreads) void relu_linear_bwd_kernel(const half_
         for (int bb = 0; bb < BPW; ++bb) {
             const int blk = wb0 + bb * kLbWaves;
             const int mi = blk / Cfg::MTO, ni = blk % Cfg::MTO;
-            const int ca = min(32 * mi + il, CIN - 1), cbb = min(32 * ni + il, COUT - 1);
+            int xoff[2], goff[2];  // transposing reads: lane = channel 32 mi + il / 32 ni + il, registers = 8 voxels
+            XT::tr_offsets(lane, mi, xoff);
+            GT::tr_offsets(lane, ni, goff);
 #pragma unroll
             for (int sp = 0; sp < KSV / KSPL; ++sp) {
                 const int s = kpart + sp * KSPL;
-                const half_t* xa = xs + (16 * s + 8 * hl) * XP + ca;
-                const half_t* gb = gs + (16 * s + 8 * hl) * GP + cbb;
-                half8_t af, bf;
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj) {
-                    const half_t xv = xa[jj * XP];
-                    af[jj] = xv > (half_t)0 ? xv : (half_t)0;
-                    bf[jj] = gb[jj * GP];
-                }
+                const half8_t af = __builtin_elementwise_max(XT::read_tr(xs, xoff, s), z8);  // relu(x), packed
+                const half8_t bf = GT::read_tr(gs, goff, s);
                 wacc[bb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, wacc[bb], 0, 0, 0);
             }
         }
@@ -181,10 +179,8 @@ __global__ __launch_bounds__(kLbThreads) void relu_linear_bwd_kernel(const half_
             const int c = t + j * kLbThreads;
             const int row = c / (CIN / 8), cc = c % (CIN / 8);
             if (c < Cfg::NXC && v0 + row < V) {
-                const half4_t lo = *reinterpret_cast<const half4_t*>(ds + row * DP + cc * 8);
-                const half4_t hi = *reinterpret_cast<const half4_t*>(ds + row * DP + cc * 8 + 4);
-                const half8_t xv = *reinterpret_cast<const half8_t*>(xs + row * XP + cc * 8);
-                half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const half8_t xv = *reinterpret_cast<const half8_t*>(xs + XT::chunk16(row, cc));
+                half8_t o = BounceTile<CIN>::read(reinterpret_cast<const unsigned char*>(ds), row, cc);
 #pragma unroll
                 for (int jj = 0; jj < 8; ++jj) o[jj] = xv[jj] > (half_t)0 ? o[jj] : (half_t)0;
                 store_c8_nt(dx + (v0 + row) * CIN + cc * 8, o);

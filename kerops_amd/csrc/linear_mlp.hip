@@ -29,7 +29,7 @@ struct MlpCfg {
     static constexpr int KS1 = C / 16;          // k steps of the first product
     static constexpr int MO = (C + 31) / 32;    // 32-row blocks of output channels
     static constexpr int KS2 = HID / 16;        // k steps of the second product: (mt, gp)
-    static constexpr int RH = C + 4;            // LDS row pitch of the output tile (halves)
+    static constexpr int RH = C;                // output tile: dense rows, swizzled (BounceTile in common.hpp)
     static constexpr int A1_OFF = 0;
     static constexpr int A2_OFF = A1_OFF + MT1 * KS1 * 64 * 16;
     static constexpr int B_OFF = A2_OFF + MO * KS2 * 64 * 16;
@@ -74,7 +74,8 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_add_kernel(const ha
 
     const half8_t* a1f = reinterpret_cast<const half8_t*>(a1) + lane;
     const half8_t* a2f = reinterpret_cast<const half8_t*>(a2) + lane;
-    half_t* my = reinterpret_cast<half_t*>(smem + Cfg::T_OFF) + wave * 32 * RH;
+    unsigned char* my = smem + Cfg::T_OFF + wave * 32 * RH * 2;
+    using Tile = BounceTile<C>;
 
     const int64_t ntiles = (V + 31) / 32;
     const int64_t tiles_per_round = (int64_t)gridDim.x * kMlpWaves;
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_add_kernel(const ha
                         half4_t o;
 #pragma unroll
                         for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)acc[4 * gq + jj];
-                        *reinterpret_cast<half4_t*>(my + vl * RH + co) = o;
+                        *reinterpret_cast<half4_t*>(my + Tile::piece(vl, 4 * mo + gq, hl)) = o;
                     }
                 }
             }
@@ -142,9 +143,7 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_add_kernel(const ha
                 const int c = c0 + lane;
                 const int row = c / (C / 8), cc = c % (C / 8);
                 if (c < 32 * C / 8 && v0 + row < V) {
-                    const half4_t lo = *reinterpret_cast<const half4_t*>(my + row * RH + cc * 8);
-                    const half4_t hi = *reinterpret_cast<const half4_t*>(my + row * RH + cc * 8 + 4);
-                    half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    half8_t o = Tile::read(my, row, cc);
                     const int64_t off = (v0 + row) * C + cc * 8;
                     const half8_t a8 = load_c8_nt(add + off);
 #pragma unroll
@@ -227,7 +226,7 @@ struct MbCfg {
     static constexpr int MH = H / 32, MO = (C + 31) / 32;  // 32-channel blocks of hidden / in-out channels
     static constexpr int KC = C / 16, KH = H / 16;         // k steps over C / over H
     static constexpr int KV = kMbTile / 16;                // k steps over the voxels of a tile
-    static constexpr int XP = C + 8, HP = H + 8, DP = C + 4;  // LDS row pitches in halves
+    static constexpr int XP = C + 8, HP = H + 8, DP = C;      // LDS row pitches in halves (the dx tile: dense rows, BounceTile)
     static constexpr int NBA = 2 * MH;                     // phase A blocks (vt, mh)
     static constexpr int NB6 = 2 * MO;                     // dx blocks (vt, mo)
     static constexpr int NU = 2 * MH * MO;                 // reduction blocks: (type, mh, mc)
@@ -403,7 +402,7 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_bwd_kernel(const ha
                         half4_t o;
 #pragma unroll
                         for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)acc[4 * gq + jj];
-                        *reinterpret_cast<half4_t*>(ds + row * DP + c) = o;
+                        *reinterpret_cast<half4_t*>(reinterpret_cast<unsigned char*>(ds) + BounceTile<C>::piece(row, 4 * mo + gq, hl)) = o;
                     }
                 }
             }
@@ -441,9 +440,7 @@ __global__ __launch_bounds__(kMlpThreads) void lin_brelu_lin_bwd_kernel(const ha
             const int c = t + j * kMlpThreads;
             const int row = c / (C / 8), cc = c % (C / 8);
             if (c < Cfg::NXC && v0 + row < V) {
-                const half4_t lo = *reinterpret_cast<const half4_t*>(ds + row * DP + cc * 8);
-                const half4_t hi = *reinterpret_cast<const half4_t*>(ds + row * DP + cc * 8 + 4);
-                const half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const half8_t o = BounceTile<C>::read(reinterpret_cast<const unsigned char*>(ds), row, cc);
                 store_c8_nt(dx + (v0 + row) * C + cc * 8, o);
             }
         }
@@ -498,7 +495,7 @@ struct MtCfg {
     static constexpr int H = 2 * C;
     static constexpr int MH = H / 32;   // 32-channel blocks of the hidden channels
     static constexpr int KC = C / 16;   // k steps over the in / out channels
-    static constexpr int DP = C + 4;    // row pitch of the dx tile (halves)
+    static constexpr int DP = C;        // row pitch of the dx tile (halves): dense rows, BounceTile in common.hpp
     static constexpr int RW = 2 * C * H + H;
     static constexpr int F1_OFF = 0;                              // Wup^T rows   [mh][s]
     static constexpr int F2_OFF = F1_OFF + MH * KC * 1024;        // Wdown rows   [mh][s]
@@ -596,7 +593,8 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
     const half8_t* f3 = reinterpret_cast<const half8_t*>(smem + Cfg::F3_OFF) + lane;
     const half8_t* ip = reinterpret_cast<const half8_t*>(smem + Cfg::IP_OFF) + lane;
     const half8_t* id = reinterpret_cast<const half8_t*>(smem + Cfg::ID_OFF) + lane;
-    half_t* my = reinterpret_cast<half_t*>(smem + Cfg::DS_OFF) + wave * 32 * DP;
+    unsigned char* my = smem + Cfg::DS_OFF + wave * 32 * DP * 2;
+    using Tile = BounceTile<C>;
 
     float16_t wdn[MH], wup[MH];  // dWdown block: D[h][c];  dWup block: D[c][h]
     float bacc[MH];
@@ -628,10 +626,7 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
             const int c = c0 + lane;
             const int row = c / (C / 8), cc = c % (C / 8);
             if (!ragged || pv0 + row < V) {
-                const half4_t lo = *reinterpret_cast<const half4_t*>(my + row * DP + cc * 8);
-                const half4_t hi = *reinterpret_cast<const half4_t*>(my + row * DP + cc * 8 + 4);
-                const half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                store_c8_nt(dx + (pv0 + row) * C + cc * 8, o);
+                store_c8_nt(dx + (pv0 + row) * C + cc * 8, Tile::read(my, row, cc));
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -746,7 +741,7 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_wave_kernel(
             half4_t o;
 #pragma unroll
             for (int jj = 0; jj < 4; ++jj) o[jj] = (half_t)dacc[4 * gq + jj];
-            *reinterpret_cast<half4_t*>(my + il * DP + 8 * gq + 4 * hl) = o;
+            *reinterpret_cast<half4_t*>(my + Tile::piece(il, gq, hl)) = o;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -830,12 +825,6 @@ __host__ __device__ constexpr int tr_slot(int r) { return ((r >> 1) & 3) ^ ((r >
 // hidden channel (inside its block of 32) stored at position p of a tile row
 __host__ __device__ constexpr int tr_hidden(int p) { return 16 * (p / 16) + 8 * ((p % 8) / 4) + 4 * ((p / 8) % 2) + p % 4; }
 
-typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 fp16x4_raw_t;
-__device__ __forceinline__ half4_t lds_read_tr16(const unsigned char* p)
-{
-    const auto q = (__attribute__((address_space(3))) fp16x4_raw_t*)(p);
-    return __builtin_bit_cast(half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4f16(q));
-}
 
 __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_tr_kernel(
     const half_t* __restrict__ x, const half_t* __restrict__ g, const half_t* __restrict__ Wup,

@@ -28,8 +28,7 @@ template <int CIN, int COUT>
 struct PwCfg {
     static constexpr int MT = (COUT + 31) / 32;      // 32-row blocks of output channels
     static constexpr int KS = CIN / 16;              // MFMA steps (k = 16 each) = 16-byte chunks a lane loads per voxel
-    static constexpr int ROW_HALVES = COUT + 4;      // LDS row pitch: +8 bytes staggers the banks
-    static constexpr int TILE_HALVES = 32 * ROW_HALVES;
+    static constexpr int TILE_HALVES = 32 * COUT;    // dense rows, swizzled: BounceTile in common.hpp
     static constexpr int OUT_CHUNKS = 32 * COUT / 8; // 16-byte chunks of one output tile
     static_assert(CIN % 16 == 0 && CIN <= 128, "CIN in {16,32,64,128}");
     static_assert(COUT % 8 == 0 && COUT <= 128, "COUT in {16,32,64,128}");
@@ -46,7 +45,8 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                                                                const float* __restrict__ shift = nullptr)
 {
     using Cfg = PwCfg<CIN, COUT>;
-    constexpr int MT = Cfg::MT, KS = Cfg::KS, RH = Cfg::ROW_HALVES;
+    constexpr int MT = Cfg::MT, KS = Cfg::KS;
+    using Tile = BounceTile<COUT>;
     __shared__ __attribute__((aligned(16))) half_t tile[kPwWaves][Cfg::TILE_HALVES];
     __shared__ __attribute__((aligned(16))) half_t wfrag[MT * KS * 64 * 8];
     __shared__ float red[kPwWaves];
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
     const int64_t ntiles = (V + 31) / 32;
     const int64_t tiles_per_round = (int64_t)gridDim.x * kPwWaves;
     const int64_t nrounds = (ntiles + tiles_per_round - 1) / tiles_per_round;
-    half_t* my = tile[wave];
+    unsigned char* my = reinterpret_cast<unsigned char*>(tile[wave]);
 
     // B fragments of a tile: this lane's voxel, chunks 2q+hl.  A tile index past the end reads the last voxel (the
     // loads are unconditional, the tile is then never used).
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                         half4_t o;
 #pragma unroll
                         for (int j = 0; j < 4; ++j) o[j] = (half_t)acc[mt][4 * gq + j];
-                        *reinterpret_cast<half4_t*>(my + vl * RH + co) = o;
+                        *reinterpret_cast<half4_t*>(my + Tile::piece(vl, 4 * mt + gq, hl)) = o;
                     }
                 }
         }
@@ -168,9 +168,7 @@ __global__ __launch_bounds__(kPwThreads) void pointwise_kernel(const half_t* __r
                 const int c = c0 + lane;
                 const int row = c / (COUT / 8), cc = c % (COUT / 8);
                 if (c < Cfg::OUT_CHUNKS && v0 + row < V) {
-                    const half4_t lo = *reinterpret_cast<const half4_t*>(my + row * RH + cc * 8);
-                    const half4_t hi = *reinterpret_cast<const half4_t*>(my + row * RH + cc * 8 + 4);
-                    half8_t o = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    half8_t o = Tile::read(my, row, cc);
                     const int64_t off = (v0 + row) * COUT + cc * 8;
                     if (HAS_ADD) {
                         const half8_t a8 = load_c8_nt(add + off);
