@@ -14,7 +14,8 @@
 //    (32 voxels x 32 input channels) block per wavefront; the fp32 result is rounded to fp16, bounced through
 //    an LDS tile and written back as 16-byte chunks with the (x > 0) mask applied from the staged x tile.
 //  * dW[ci, co] reduces over voxels, which is the slow axis of both operands in memory: the fragments
-//    "8 consecutive voxels of one channel" are gathered from the LDS tiles with 2-byte reads (the ReLU is
+//    "8 consecutive voxels of one channel" are gathered from the LDS tiles with transposing reads (two
+//    ds_read_b64_tr_b16 per fragment, see SwizzledRows in common.hpp; the ReLU is
 //    applied to the x fragment in registers).  The (32 x 32) output blocks are distributed over the
 //    wavefronts (with fewer than four blocks the wavefronts split the voxels instead) and accumulated in
 //    fp32 registers over all tiles of the workgroup; at the end every workgroup writes its partial
