@@ -8,6 +8,8 @@
 // lanes take consecutive (d_out, channel-group) chunks, so the two D-taps of a wavefront
 // together cover contiguous input memory.  The statistics use the unrounded fp32 pooled
 // values and the same deterministic two-pass reduction as the other per-channel sums.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace kerops {
@@ -135,7 +137,14 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_fwd_kernel(const ha
     block_channel_partials_any<2, V>(acc, p.CG, red, ws + (int64_t)blockIdx.x * 2 * p.CG * V);
 }
 
-template <int V, int U>
+// PERM (16-byte chunks, even D, whole wavefronts inside one pooled row, fewer than 64 channels): a wavefront's 64
+// results belong to 64 / CG consecutive pooled positions of one pooled row, so each of the four (h, w) rows of their
+// windows is one run of 128 consecutive output chunks in which every result appears twice (both D taps).  The
+// results are redistributed over the lanes (ds_bpermute: output chunk j of the run comes from lane (j / 2CG) CG +
+// j % CG) and every store instruction writes 1 KB of consecutive memory; stored straight from the lane that computed
+// them, an instruction would write every second voxel row, i.e. parts of 128-byte lines where a voxel row is
+// narrower than a line.
+template <int V, int U, bool PERM>
 __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_bwd_kernel(const half_t* __restrict__ inpgrad,
                                                                         const float* __restrict__ meangrad,
                                                                         const float* __restrict__ sqmeangrad,
@@ -153,7 +162,9 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_bwd_kernel(const ha
         mg[j] = __fdiv_rn(meangrad[cg0 * V + j], fMo);
         sg[j] = sqmeangrad[cg0 * V + j];
     }
-    auto one = [&](int64_t i, const hv& g, const hv& o) {
+    const int lane = threadIdx.x % kWave;
+    const int src0 = ((lane / (2 * p.CG)) * p.CG + lane % p.CG) * 4;  // PERM: byte index of the source lane, first run half
+    auto one = [&](int64_t i, const hv& g, const hv& o, auto whole_wave) {
         int64_t r = i / p.CG;
         const int dO = (int)(r % p.Do);
         r /= p.Do;
@@ -171,15 +182,39 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_bwd_kernel(const ha
             res[j] = (half_t)__fdiv_rn(t, cnt);
         }
         const int64_t base = n * sN + (2 * hO) * sH + (2 * wO) * sW + (2 * dO) * sD + cg0;
+        if constexpr (PERM && decltype(whole_wave)::value) {
+            // lane 0 holds the first pooled position of the run and channel group 0
+            const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)(uint64_t)base);
+            const uint32_t bhi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)base >> 32));
+            const int64_t run0 = (int64_t)(((uint64_t)bhi << 32) | blo);
+            constexpr int NDW = (int)(sizeof(hv) + 3) / 4;  // (4 dwords: this path is built for 16-byte chunks)
+            uint32_t rv[NDW] = {};
+            __builtin_memcpy(rv, &res, sizeof(hv));
 #pragma unroll
-        for (int a = 0; a < 2; ++a)
+            for (int e = 0; e < 2; ++e) {  // the two halves of the run
+                uint32_t pv[NDW];
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+                for (int q = 0; q < NDW; ++q) pv[q] = (uint32_t)__builtin_amdgcn_ds_bpermute(src0 + e * 128, (int)rv[q]);
+                hv out;
+                __builtin_memcpy(&out, pv, sizeof(hv));
 #pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
-                    if (ok) st_stream<V>(dx, base + a * sH + b * sW + e * sD, res);
-                }
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b)
+                        if ((a == 0 || h1) && (b == 0 || w1))  // wavefront-uniform
+                            st_stream<V>(dx, run0 + a * sH + b * sW + e * 64 + lane, out);
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const bool ok = (a == 0 || h1) && (b == 0 || w1) && (e == 0 || d1);
+                        if (ok) st_stream<V>(dx, base + a * sH + b * sW + e * sD, res);
+                    }
+        }
     };
     for (int64_t k = 0; k < wk.nfull; ++k) {
         const int64_t i = k * wk.step + wk.first;
@@ -190,9 +225,11 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_bwd_kernel(const ha
             o[u] = ld_stream<V>(output, i + u * wk.su);
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) one(i + u * wk.su, g[u], o[u]);
+        for (int u = 0; u < U; ++u) one(i + u * wk.su, g[u], o[u], std::true_type{});
     }
-    for (int64_t i = wk.tail; i < nchunks; i += wk.T) one(i, ld_stream<V>(inpgrad, i), ld_stream<V>(output, i));
+    // (the last, partly filled step: every lane stores its own result)
+    for (int64_t i = wk.tail; i < nchunks; i += wk.T)
+        one(i, ld_stream<V>(inpgrad, i), ld_stream<V>(output, i), std::false_type{});
 }
 
 // Launch shape (blocks, waves, segment) as for the flat stream kernels; segment counts output chunks per thread and
@@ -358,11 +395,18 @@ extern "C" int kerops_avgpool_ceil_stats_bwd_f16(const void* inpgrad, const floa
     }
     const float fMo = (float)((int64_t)N * p.Ho * p.Wo * p.Do);
     const int seg = sh.segment != 1;
+    // redistribute the results for whole-line stores where a voxel row is narrower than a 128-byte line
+    const bool perm = C >= 8 && C < 64 && D % 2 == 0 && ((int64_t)p.Do * p.CG) % kWave == 0;
 #define KEROPS_POOLB_GO(Uv)                                                                                          \
     KEROPS_DISPATCH_V(C, {                                                                                           \
-        hipLaunchKernelGGL((avgpool_bwd_kernel<V, Uv>), dim3(sh.blocks), dim3(sh.threads), 0, (hipStream_t)stream,   \
-                           (const half_t*)inpgrad, meangrad, sqmeangrad, (const half_t*)output, (half_t*)dx, p,      \
-                           nchunks, fMo, seg);                                                                       \
+        if (perm && V == 8)                                                                                          \
+            hipLaunchKernelGGL((avgpool_bwd_kernel<V, Uv, V == 8>), dim3(sh.blocks), dim3(sh.threads), 0,            \
+                               (hipStream_t)stream, (const half_t*)inpgrad, meangrad, sqmeangrad,                    \
+                               (const half_t*)output, (half_t*)dx, p, nchunks, fMo, seg);                            \
+        else                                                                                                         \
+            hipLaunchKernelGGL((avgpool_bwd_kernel<V, Uv, false>), dim3(sh.blocks), dim3(sh.threads), 0,             \
+                               (hipStream_t)stream, (const half_t*)inpgrad, meangrad, sqmeangrad,                    \
+                               (const half_t*)output, (half_t*)dx, p, nchunks, fMo, seg);                            \
     })
     if (sh.segment == 2) KEROPS_POOLB_GO(2);
     else KEROPS_POOLB_GO(1);

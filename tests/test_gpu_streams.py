@@ -149,7 +149,12 @@ def test_bn_block_end_to_end_vs_train_mode_batchnorm(golden):
     assert torch.allclose(mean.cpu().double(), torch.from_numpy(golden['stats_mean_f64']), atol=1e-6)
 
 
-@pytest.mark.parametrize('shape', SHAPES + [(1, 8, 1, 1, 1), (2, 16, 2, 3, 2), (1, 64, 13, 7, 128)])
+# (the last five: narrow voxel rows with an even D whose pooled rows hold whole wavefronts, the shapes on which the
+# backward redistributes its results over the lanes for whole-line stores; odd H and W put edge windows in every plane;
+# several launch steps and a partly filled last step)
+@pytest.mark.parametrize('shape', SHAPES + [(1, 8, 1, 1, 1), (2, 16, 2, 3, 2), (1, 64, 13, 7, 128), (1, 8, 5, 7, 128),
+                                            (2, 16, 3, 5, 64), (1, 32, 7, 3, 32), (1, 16, 37, 41, 128),
+                                            (3, 32, 21, 19, 64)])
 def test_avgpool_and_backward(shape):
     g = cpu_gen(3)
     c = shape[1]
