@@ -1104,7 +1104,7 @@ int dwconv_fwd_run(const void* x, const void* wt, void* y, const float* scale, c
         // measured best on MI355X at (1, C, 350, 350, 128)
         // (the matrix-core kernels)
         switch (cg) {
-            case 1: tile_w = 8; tile_d = 32; break;
+            case 1: tile_w = 8; tile_d = D > 32 ? 64 : 32; break;
             case 2: tile_w = 8; tile_d = 32; break;
             case 4: tile_w = 8; tile_d = 16; break;
             default: tile_w = 8; tile_d = 8; break;

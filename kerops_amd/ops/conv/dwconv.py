@@ -16,18 +16,19 @@ from .variants import FWD_VARIANTS
 _WAVES = {8: 4, 16: 8, 32: 8, 64: 8, 128: 8}
 _TILE_D = {8: 32, 16: 32, 32: 16, 64: 8, 128: 8}
 _TILE_W = {8: 8, 16: 8, 32: 8, 64: 8, 128: 8}
+# at 8 channels the patch is 8 x 64 (512 threads) when the volume is more than 32 deep
 # 16 = matrix-core kernels (16 channel blocks per MFMA); 2 / 4 = vector kernels (channels per lane)
 _LANE_C = {8: 16, 16: 16, 32: 16, 64: 16, 128: 16}
 
 
 @confexc(KeyError)
-def warps(channels):
-    return _WAVES[channels]
+def warps(channels, depth=None):
+    return 8 if channels == 8 and depth is not None and depth > 32 else _WAVES[channels]
 
 
 @confexc(KeyError)
-def dblock(channels):
-    return _TILE_D[channels]
+def dblock(channels, depth=None):
+    return 64 if channels == 8 and depth is not None and depth > 32 else _TILE_D[channels]
 
 
 @confexc(KeyError)
@@ -42,8 +43,8 @@ def lanec(channels):
 
 @configure(
     ACCTYPE='float32',
-    num_warps=lambda x: warps(x.shape[1]),
-    D_block=lambda x: dblock(x.shape[1]),
+    num_warps=lambda x: warps(x.shape[1], x.shape[4]),
+    D_block=lambda x: dblock(x.shape[1], x.shape[4]),
     W_block=lambda x: wtile(x.shape[1]),
     H_chunk=0,
     lane_channels=lambda x: lanec(x.shape[1]),
