@@ -63,8 +63,8 @@ extern "C" {
  * caller built against an older header can detect the mismatch before passing arguments
  * (kerops_hip_version() of the loaded library must equal the KEROPS_HIP_VERSION it was compiled
  * against).  100: first interface; 200: launch-shape knobs (waves, segment) on the stream entry points,
- * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16. */
-#define KEROPS_HIP_VERSION 200
+ * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16; 210: kerops_dwconv_wgrad_f16_out, kerops_dwconv_bwd_f16_out. */
+#define KEROPS_HIP_VERSION 210
 
 int kerops_hip_version(void);
 const char* kerops_last_error_string(void);
@@ -113,6 +113,13 @@ int64_t kerops_dwconv_wgrad_workspace_bytes(int32_t N, int32_t H, int32_t W, int
 int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, void* workspace, int64_t workspace_bytes,
                             int32_t N, int32_t H, int32_t W, int32_t D, int32_t C, int32_t tile_w, int32_t tile_d,
                             int32_t h_chunk, int32_t lane_channels, void* stream);
+/* kerops_dwconv_wgrad_f16 with the type of the result chosen by the caller: gw_dtype = KEROPS_DTYPE_F32 (gw is
+ * float[27*C], the same bits as kerops_dwconv_wgrad_f16) or KEROPS_DTYPE_F16 (gw is fp16[27*C]: the fp32 sum rounded
+ * once, to nearest even, by the reduction kernel).  The reference returns an fp16 [3,3,3,C] tensor
+ * (kerops/ops/conv/dwconv_wgrad.py:54,77-79); this entry point gives that type without a cast kernel after the call. */
+int kerops_dwconv_wgrad_f16_out(const void* x, const void* g, void* gw, int32_t gw_dtype, void* workspace,
+                                int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
+                                int32_t tile_w, int32_t tile_d, int32_t h_chunk, int32_t lane_channels, void* stream);
 
 /* kerops_dwconv_wgrad_f16 at its built-in launch shape for callers that cannot allocate: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
@@ -140,6 +147,11 @@ int64_t kerops_dwconv_bwd_workspace_bytes(int32_t N, int32_t H, int32_t W, int32
 int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* wt, void* dx, float* gw, void* workspace,
                           int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D, int32_t C,
                           int32_t h_chunk, void* stream);
+/* kerops_dwconv_bwd_f16 with gw written as gw_dtype (KEROPS_DTYPE_F32 or KEROPS_DTYPE_F16, rounded once), as in
+ * kerops_dwconv_wgrad_f16_out. */
+int kerops_dwconv_bwd_f16_out(const void* x, const void* g, const void* wt, void* dx, void* gw, int32_t gw_dtype,
+                              void* workspace, int64_t workspace_bytes, int32_t N, int32_t H, int32_t W, int32_t D,
+                              int32_t C, int32_t h_chunk, void* stream);
 
 /* Per-channel mean and mean of squares over M = numel / C voxels, fp32.
  * Replaces the zero-fill of mean/sqmean and the `_Stats_cl3d_impl[(grid,)](...)`

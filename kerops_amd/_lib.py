@@ -18,9 +18,11 @@ KEROPS_E_WORKSPACE = -3
 KEROPS_E_LAUNCH = -4
 
 # KEROPS_HIP_VERSION of include/kerops_hip.h that SIGNATURES below mirrors
-HEADER_VERSION = 200
+HEADER_VERSION = 210
 
 DTYPE_TAGS = {torch.float16: 0, torch.float32: 1, torch.bfloat16: 2}
+# result types the weight-gradient reduction kernel writes itself (kerops_dwconv_wgrad_f16_out, kerops_dwconv_bwd_f16_out)
+GW_DTYPES = {torch.float16: 0, torch.float32: 1}
 
 _p = ctypes.c_void_p
 _i32 = ctypes.c_int32
@@ -36,9 +38,13 @@ SIGNATURES = {
     'kerops_dwconv_stats_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_dwconv_bwd_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_dwconv_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _p]),
+    'kerops_dwconv_bwd_f16_out': (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32,
+                                                 _p]),
     'kerops_dwconv_wgrad_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_dwconv_wgrad_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32,
                                                _i32, _p]),
+    'kerops_dwconv_wgrad_f16_out': (ctypes.c_int, [_p, _p, _p, _i32, _p, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32,
+                                                   _i32, _i32, _p]),
     'kerops_dwconv_wgrad_noalloc_f16': (ctypes.c_int, [_p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p]),
     'kerops_stats_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'kerops_stats_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _p, _i64, _i32, _i32, _i32, _p]),

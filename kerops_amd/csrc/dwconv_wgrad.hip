@@ -1034,7 +1034,9 @@ __global__ __launch_bounds__(Cfg::NT, 4) void dwconv_bwd_split_kernel(const WgAr
 // d-patch) of width RW = slabs*27*SC floats.  A workgroup owns 16 columns, its 64 row slices sum interleaved rows
 // (four loads in flight), the slices are combined in LDS in a fixed order and the result is scattered to the
 // [27][C] layout.  One launch: at 128^3-class shapes a second small launch was 5 % of the whole op.
-__global__ __launch_bounds__(1024) void wgrad_reduce_kernel(const float* __restrict__ ws, float* __restrict__ gw,
+// OutT: fp32, or fp16 = the sum rounded once (what a cast of the fp32 result gives, without its launch).
+template <class OutT>
+__global__ __launch_bounds__(1024) void wgrad_reduce_kernel(const float* __restrict__ ws, OutT* __restrict__ gw,
                                                             int n_rows, int RW, int SC, int C)
 {
     __shared__ float part[64][17];
@@ -1060,7 +1062,7 @@ __global__ __launch_bounds__(1024) void wgrad_reduce_kernel(const float* __restr
     if (slice == 0 && col < RW) {
         const int slab = col / (27 * SC), rem = col % (27 * SC);
         const int tap = rem / SC, cs = rem % SC;
-        gw[tap * C + slab * SC + cs] = part[0][cl];
+        gw[tap * C + slab * SC + cs] = (OutT)part[0][cl];
     }
 }
 
@@ -1165,16 +1167,36 @@ static int64_t wgrad_ws_bytes(const WgPlan& p)
 }
 
 // the two reduction kernels over the per-workgroup partials [nblocks][27][SC] at the start of ws
-static int reduce_partials(float* ws, const WgPlan& p, int SC, int C, float* gw, hipStream_t stream)
+// where the reduced gradient goes: an fp32 [27][C] array, or an fp16 one (KEROPS_DTYPE_F16)
+struct GwOut {
+    void* p;
+    int dtype;
+    GwOut(float* f) : p(f), dtype(KEROPS_DTYPE_F32) {}
+    GwOut(void* q, int dt) : p(q), dtype(dt) {}
+};
+
+static int reduce_partials(float* ws, const WgPlan& p, int SC, int C, GwOut gw, hipStream_t stream)
 {
     const int n_rows = (int)(p.nblocks / p.n_slab);
     const int RW = p.n_slab * 27 * SC;
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, stream, ws, gw, n_rows, RW, SC, C);
+    if (gw.dtype == KEROPS_DTYPE_F16)
+        hipLaunchKernelGGL(wgrad_reduce_kernel<half_t>, dim3(ceil_div(RW, 16)), dim3(1024), 0, stream, ws, (half_t*)gw.p,
+                           n_rows, RW, SC, C);
+    else
+        hipLaunchKernelGGL(wgrad_reduce_kernel<float>, dim3(ceil_div(RW, 16)), dim3(1024), 0, stream, ws, (float*)gw.p,
+                           n_rows, RW, SC, C);
     return check_launch("dwconv_wgrad_reduce");
 }
 
+static int check_gw_dtype(const char* op, int32_t gw_dtype)
+{
+    if (gw_dtype == KEROPS_DTYPE_F32 || gw_dtype == KEROPS_DTYPE_F16) return KEROPS_OK;
+    set_error("%s: gw_dtype must be KEROPS_DTYPE_F32 or KEROPS_DTYPE_F16", op);
+    return KEROPS_E_BADARG;
+}
+
 template <class Cfg, class KernelT>
-static int launch_wgrad_cfg(KernelT kernel, const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
+static int launch_wgrad_cfg(KernelT kernel, const WgArgs& base, const WgPlan& p, GwOut gw, hipStream_t stream)
 {
     WgArgs a = base;
     a.n_wt = p.n_wt;
@@ -1195,14 +1217,14 @@ static int launch_wgrad_cfg(KernelT kernel, const WgArgs& base, const WgPlan& p,
 }
 
 template <int CG, int TW, int TD, int NT>
-static int launch_wgrad(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
+static int launch_wgrad(const WgArgs& base, const WgPlan& p, GwOut gw, hipStream_t stream)
 {
     using Cfg = WgCfg<CG, TW, TD, NT>;
     return launch_wgrad_cfg<Cfg>(dwconv_wgrad_kernel<Cfg>, base, p, gw, stream);
 }
 
 template <int CG, int TW, int TD, int NT>
-static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, float* gw, hipStream_t stream)
+static int launch_wgrad_mfma(const WgArgs& base, const WgPlan& p, GwOut gw, hipStream_t stream)
 {
     using Cfg = WmCfg<CG, TW, TD, NT>;
     if (base.stream_interior) return launch_wgrad_cfg<Cfg>(dwconv_wgrad_mfma_kernel<Cfg, true>, base, p, gw, stream);
@@ -1307,8 +1329,18 @@ extern "C" int kerops_dwconv_bwd_f16(const void* x, const void* g, const void* w
                                      void* workspace, int64_t workspace_bytes, int32_t N, int32_t H, int32_t W,
                                      int32_t D, int32_t C, int32_t h_chunk, void* stream)
 {
-    if (!x || !g || !wt || !dx || !gw || !aligned16(x) || !aligned16(g) || !aligned16(wt) || !aligned16(dx) ||
-        !aligned16(gw)) {
+    return kerops_dwconv_bwd_f16_out(x, g, wt, dx, gw, KEROPS_DTYPE_F32, workspace, workspace_bytes, N, H, W, D, C,
+                                     h_chunk, stream);
+}
+
+extern "C" int kerops_dwconv_bwd_f16_out(const void* x, const void* g, const void* wt, void* dx, void* gw_out,
+                                         int32_t gw_dtype, void* workspace, int64_t workspace_bytes, int32_t N,
+                                         int32_t H, int32_t W, int32_t D, int32_t C, int32_t h_chunk, void* stream)
+{
+    if (check_gw_dtype("dwconv_bwd", gw_dtype) != KEROPS_OK) return KEROPS_E_BADARG;
+    const GwOut gw(gw_out, gw_dtype);
+    if (!x || !g || !wt || !dx || !gw_out || !aligned16(x) || !aligned16(g) || !aligned16(wt) || !aligned16(dx) ||
+        !aligned16(gw_out)) {
         set_error("dwconv_bwd: null or misaligned pointer");
         return KEROPS_E_BADARG;
     }
@@ -1382,7 +1414,18 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
                                        int32_t tile_w, int32_t tile_d, int32_t h_chunk, int32_t lane_channels,
                                        void* stream)
 {
-    if (!x || !g || !gw || !aligned16(x) || !aligned16(g) || !aligned16(gw)) {
+    return kerops_dwconv_wgrad_f16_out(x, g, gw, KEROPS_DTYPE_F32, workspace, workspace_bytes, N, H, W, D, C, tile_w,
+                                       tile_d, h_chunk, lane_channels, stream);
+}
+
+extern "C" int kerops_dwconv_wgrad_f16_out(const void* x, const void* g, void* gw_out, int32_t gw_dtype,
+                                           void* workspace, int64_t workspace_bytes, int32_t N, int32_t H, int32_t W,
+                                           int32_t D, int32_t C, int32_t tile_w, int32_t tile_d, int32_t h_chunk,
+                                           int32_t lane_channels, void* stream)
+{
+    if (check_gw_dtype("dwconv_wgrad", gw_dtype) != KEROPS_OK) return KEROPS_E_BADARG;
+    const GwOut gw(gw_out, gw_dtype);
+    if (!x || !g || !gw_out || !aligned16(x) || !aligned16(g) || !aligned16(gw_out)) {
         set_error("dwconv_wgrad: null or misaligned pointer");
         return KEROPS_E_BADARG;
     }
@@ -1447,7 +1490,6 @@ extern "C" int kerops_dwconv_wgrad_f16(const void* x, const void* g, float* gw, 
         b.bal_r = p.bal_r;
         b.n_tiles = p.n_tiles;
         b.n_xcd = (uint32_t)p.n_xcd;
-    b.n_xcd = (uint32_t)p.n_xcd;
         const int depth = p.cl == 32 ? 0 : p.cl == 33 ? 11 : p.cl == 34 ? 22 : 12;
         if (launch_wgrad_dma(b, p.cg, p.tile_w, p.tile_d, depth, s) == 0) {
             rc = check_launch("dwconv_wgrad");

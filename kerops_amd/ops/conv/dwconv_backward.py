@@ -39,7 +39,10 @@ def DWConvBackward(x, grad, weight, *, H_chunk: ConfigurableArg, out_dtype: Conf
     ws_bytes = _lib.query('kerops_dwconv_bwd_workspace_bytes', bsize, H, W, D, channels, int(H_chunk))
     ws = _lib.workspace(ws_bytes, x.device)
     grad_x = torch.empty_like(x)
-    grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=torch.float32)
-    _lib.call('kerops_dwconv_bwd_f16', x.data_ptr(), grad.data_ptr(), weight.data_ptr(), grad_x.data_ptr(),
-              grad_w.data_ptr(), ws.data_ptr(), ws_bytes, bsize, H, W, D, channels, int(H_chunk), _lib.stream_of(x))
-    return grad_x, (grad_w if out_dtype == torch.float32 else grad_w.to(out_dtype))
+    # fp32 and fp16 results are written by the library's reduction kernel; any other type is cast from fp32
+    direct = out_dtype in _lib.GW_DTYPES
+    grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=out_dtype if direct else torch.float32)
+    _lib.call('kerops_dwconv_bwd_f16_out', x.data_ptr(), grad.data_ptr(), weight.data_ptr(), grad_x.data_ptr(),
+              grad_w.data_ptr(), _lib.GW_DTYPES[grad_w.dtype], ws.data_ptr(), ws_bytes, bsize, H, W, D, channels,
+              int(H_chunk), _lib.stream_of(x))
+    return grad_x, (grad_w if direct else grad_w.to(out_dtype))

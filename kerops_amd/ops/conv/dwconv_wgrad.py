@@ -3,7 +3,8 @@
 Host side of kerops_dwconv_wgrad_f16; same name, positional arguments and asserts as
 kerops/ops/conv/dwconv_wgrad.py:25-79 of the reference.  The reference stores fp16
 partials and returns an fp16 [3,3,3,C] tensor; here the sum is fp32 end to end and is
-cast once to `out_dtype` (fp16 by default so the result type matches the reference).
+rounded once to `out_dtype` (fp16 by default so the result type matches the reference;
+fp16 and fp32 are written by the reduction kernel itself).
 """
 import torch
 
@@ -100,10 +101,12 @@ def DWConvWGRAD(
     cfg = (w_block, d_block, int(H_chunk), lane_c)
     ws_bytes = _lib.query('kerops_dwconv_wgrad_workspace_bytes', bsize, H, W, D, channels, *cfg)
     ws = _lib.workspace(ws_bytes, x.device)
-    grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=torch.float32)
+    # fp32 and fp16 results are written by the library's reduction kernel; any other type is cast from fp32
+    direct = out_dtype in _lib.GW_DTYPES
+    grad_w = torch.empty([3, 3, 3, channels], device=x.device, dtype=out_dtype if direct else torch.float32)
 
     _lib.call(
-        'kerops_dwconv_wgrad_f16', x.data_ptr(), grad.data_ptr(), grad_w.data_ptr(), ws.data_ptr(), ws_bytes,
-        bsize, H, W, D, channels, *cfg, _lib.stream_of(x),
+        'kerops_dwconv_wgrad_f16_out', x.data_ptr(), grad.data_ptr(), grad_w.data_ptr(),
+        _lib.GW_DTYPES[grad_w.dtype], ws.data_ptr(), ws_bytes, bsize, H, W, D, channels, *cfg, _lib.stream_of(x),
     )
-    return grad_w if out_dtype == torch.float32 else grad_w.to(out_dtype)
+    return grad_w if direct else grad_w.to(out_dtype)

@@ -62,6 +62,10 @@ def test_dwconv_wgrad_matches_oracle(shape):
     # drop-in result type (fp16) and the reference's own criterion
     gw16 = DWConvWGRAD(x.to(DEV), grad.to(DEV)).cpu()
     assert gw16.dtype == torch.float16
+    # the fp16 result is written by the reduction kernel: the fp32 sum rounded once, as a cast of it rounds
+    assert torch.equal(gw16.view(torch.int16), gw32.to(torch.float16).view(torch.int16))
+    gwbf = DWConvWGRAD(x.to(DEV), grad.to(DEV), out_dtype=torch.bfloat16).cpu()  # any other type: cast from fp32
+    assert gwbf.dtype == torch.bfloat16 and torch.equal(gwbf.view(torch.int16), gw32.bfloat16().view(torch.int16))
     if ref.abs().max() < 6e4:
         assert weight_grad_similarity(ref.float(), gw16.float(), rtol_cos=1e-4, atol_cos=1e-4,
                                       rtol_len=1e-3 * shape[0], atol_len=1e-3)
@@ -355,6 +359,10 @@ def test_fused_backward_matches_oracle_and_separate_ops(c, shape_hc):
     # determinism
     dx3, gw3 = DWConvBackward(xd, gd, wd, H_chunk=hc, out_dtype=torch.float32)
     assert torch.equal(dx, dx3) and torch.equal(gw, gw3)
+    # default result type fp16, written by the reduction kernel = the fp32 sum rounded once
+    dx4, gw4 = DWConvBackward(xd, gd, wd, H_chunk=hc)
+    assert gw4.dtype == torch.float16 and torch.equal(dx, dx4)
+    assert torch.equal(gw4.view(torch.int16), gw.to(torch.float16).view(torch.int16))
 
 
 @pytest.mark.parametrize('c', [8, 64])
