@@ -63,7 +63,8 @@ extern "C" {
  * caller built against an older header can detect the mismatch before passing arguments
  * (kerops_hip_version() of the loaded library must equal the KEROPS_HIP_VERSION it was compiled
  * against).  100: first interface; 200: launch-shape knobs (waves, segment) on the stream entry points,
- * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16; 210: kerops_dwconv_wgrad_f16_out, kerops_dwconv_bwd_f16_out. */
+ * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16; 210: kerops_dwconv_wgrad_f16_out, kerops_dwconv_bwd_f16_out,
+ * scale output of kerops_quant_i8_sym_f16. */
 #define KEROPS_HIP_VERSION 210
 
 int kerops_hip_version(void);
@@ -253,10 +254,11 @@ int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, void* workspa
                       int32_t blocks, void* stream);
 
 /* q = clamp(rint_half_even(float(y) / (absmax/127)), -127, 127) as int8, with
- * absmax read from device memory; absmax == 0 gives q = 0.  No reference
+ * absmax read from device memory; absmax == 0 gives q = 0.  scale (device fp32, may be
+ * null) receives absmax/127, the factor that dequantises q.  No reference
  * counterpart: second pass of the symmetric int8 quantiser. */
-int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t numel, int32_t blocks,
-                            int32_t waves, int32_t segment, void* stream);
+int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, float* scale, int64_t numel,
+                            int32_t blocks, int32_t waves, int32_t segment, void* stream);
 
 /* Pointwise (1x1x1) channel mixing on MFMA:
  *   out[v, co] = fp16(sum_ci act(x[v, ci]) * Wm[ci, co]) (+ add[v, co], fp16 add)

@@ -65,7 +65,7 @@ SIGNATURES = {
     'kerops_dequant_u8_window': (ctypes.c_int, [_p, _p, _i32, _i64, _f32, _i32, _i32, _i32, _p]),
     'kerops_absmax_workspace_bytes': (_i64, [_i32]),
     'kerops_absmax_f16': (ctypes.c_int, [_p, _p, _i64, _p, _i64, _i32, _p]),
-    'kerops_quant_i8_sym_f16': (ctypes.c_int, [_p, _p, _p, _i64, _i32, _i32, _i32, _p]),
+    'kerops_quant_i8_sym_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p]),
     'kerops_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p]),
     'kerops_bnrelu_pointwise_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _p]),
     'kerops_lin_brelu_lin_add_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _p]),

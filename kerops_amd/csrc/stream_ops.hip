@@ -393,7 +393,8 @@ __device__ __forceinline__ uint32_t quant_i8_one(float v, float scale, float rsc
 template <int U>
 __global__ __launch_bounds__(kStreamMaxThreads) void quant_i8_kernel(const half_t* __restrict__ y,
                                                                      const float* __restrict__ absmax,
-                                                                     int8_t* __restrict__ q, int64_t numel,
+                                                                     int8_t* __restrict__ q,
+                                                                     float* __restrict__ scale_out, int64_t numel,
                                                                      int segments)
 {
     const float scale = __fdiv_rn(absmax[0], 127.0f);
@@ -427,6 +428,7 @@ __global__ __launch_bounds__(kStreamMaxThreads) void quant_i8_kernel(const half_
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         for (int64_t k = nunits * 8; k < numel; ++k)
             q[k] = zero ? (int8_t)0 : (int8_t)quant_i8_one((float)y[k], scale, rscale);
+        if (scale_out) scale_out[0] = scale;  // absmax / 127, correctly rounded: what the caller dequantises with
     }
 }
 
@@ -816,8 +818,8 @@ extern "C" int kerops_absmax_f16(const void* y, float* absmax, int64_t numel, vo
     return check_launch("absmax");
 }
 
-extern "C" int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, int64_t numel, int32_t blocks,
-                                       int32_t waves, int32_t segment, void* stream)
+extern "C" int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void* q, float* scale, int64_t numel,
+                                       int32_t blocks, int32_t waves, int32_t segment, void* stream)
 {
     StreamShape sh;
     int rc = check_flat("quant_i8_sym", kDefQuantI8, y, q, numel, numel / 8, blocks, waves, segment, &sh);
@@ -829,10 +831,10 @@ extern "C" int kerops_quant_i8_sym_f16(const void* y, const float* absmax, void*
     const int seg = sh.segment != 1;
     if (sh.unroll() == 8) {
         hipLaunchKernelGGL(quant_i8_kernel<8>, dim3(sh.blocks), dim3(sh.threads), 0, (hipStream_t)stream,
-                           (const half_t*)y, absmax, (int8_t*)q, numel, seg);
+                           (const half_t*)y, absmax, (int8_t*)q, scale, numel, seg);
     } else {
         hipLaunchKernelGGL(quant_i8_kernel<4>, dim3(sh.blocks), dim3(sh.threads), 0, (hipStream_t)stream,
-                           (const half_t*)y, absmax, (int8_t*)q, numel, seg);
+                           (const half_t*)y, absmax, (int8_t*)q, scale, numel, seg);
     }
     return check_launch("quant_i8_sym");
 }

@@ -86,6 +86,7 @@ def QuantInt8Sym(y, absmax=None, *, blocks: ConfigurableArg, num_warps: Configur
         absmax = AbsMax(y)
     assert absmax.dtype == torch.float32 and absmax.numel() == 1 and absmax.is_cuda
     q = torch.empty_like(y, dtype=torch.int8)
-    _lib.call('kerops_quant_i8_sym_f16', y.data_ptr(), absmax.data_ptr(), q.data_ptr(), y.numel(), int(blocks),
-              stream_waves(num_warps), int(segment), _lib.stream_of(y))
-    return q, absmax / 127.0
+    scale = torch.empty_like(absmax)  # absmax / 127, written by the quantising kernel
+    _lib.call('kerops_quant_i8_sym_f16', y.data_ptr(), absmax.data_ptr(), q.data_ptr(), scale.data_ptr(), y.numel(),
+              int(blocks), stream_waves(num_warps), int(segment), _lib.stream_of(y))
+    return q, scale

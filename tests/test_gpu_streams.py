@@ -393,8 +393,9 @@ def test_quant_i8_sym_bit_exact():
     # exhaustive over fp16 for a few explicit maxima, ties included
     for amax in (127.0, 1.0, 3.3, 65504.0, 6e-8, 0.001, 77.77, 1234.5, 2.0 ** -14):
         am = torch.tensor([amax], dtype=torch.float32, device=DEV)
-        q, _ = QuantInt8Sym(fin.to(DEV), am)
+        q, s = QuantInt8Sym(fin.to(DEV), am)
         assert torch.equal(q.cpu(), oracle.quant_i8_sym(fin, amax))
+        assert s.dtype == torch.float32 and s.shape == am.shape and torch.equal(s.cpu(), am.cpu() / 127.0)
     z, _ = QuantInt8Sym(torch.zeros(100, dtype=torch.float16, device=DEV))
     assert (z == 0).all()
 
