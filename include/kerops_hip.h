@@ -63,8 +63,8 @@ extern "C" {
  * caller built against an older header can detect the mismatch before passing arguments
  * (kerops_hip_version() of the loaded library must equal the KEROPS_HIP_VERSION it was compiled
  * against).  100: first interface; 200: launch-shape knobs (waves, segment) on the stream entry points,
- * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16; 210: kerops_dwconv_wgrad_f16_out, kerops_dwconv_bwd_f16_out,
- * scale output of kerops_quant_i8_sym_f16. */
+ * kerops_dwconv_wgrad_noalloc_f16, KEROPS_DTYPE_BF16; 210: the *_f16_out variants (weight gradients written as fp16 by the
+ * reduction kernels), scale output of kerops_quant_i8_sym_f16. */
 #define KEROPS_HIP_VERSION 210
 
 int kerops_hip_version(void);
@@ -288,6 +288,11 @@ int kerops_bnrelu_pointwise_f16(const void* x, const float* scale, const float* 
 int64_t kerops_relu_linear_bwd_workspace_bytes(int64_t V, int32_t Cin, int32_t Cout);
 int kerops_relu_linear_bwd_f16(const void* x, const void* g, const void* Wm, void* dx, float* dW, void* workspace,
                                int64_t workspace_bytes, int64_t V, int32_t Cin, int32_t Cout, void* stream);
+/* kerops_relu_linear_bwd_f16 with dW written as dw_dtype: KEROPS_DTYPE_F32, or KEROPS_DTYPE_F16 = the fp32 result
+ * rounded once by the reduction kernel (the reference returns fp16, kerops/ops/linear/relu_linear_backward.py:70). */
+int kerops_relu_linear_bwd_f16_out(const void* x, const void* g, const void* Wm, void* dx, void* dW, int32_t dw_dtype,
+                                   void* workspace, int64_t workspace_bytes, int64_t V, int32_t Cin, int32_t Cout,
+                                   void* stream);
 
 /* Inverted-bottleneck pointwise block on MFMA, the hidden activation stays in registers:
  *   hid = relu(fp16(x @ Wup) + bias);  out = fp16(hid @ Wdown) + add       (fp16 adds)
@@ -308,6 +313,12 @@ int64_t kerops_lin_brelu_lin_bwd_workspace_bytes(int64_t V, int32_t C);
 int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const void* Wup, const void* Wdown, const void* bias,
                                  void* dx, float* dWup, float* dWdown, float* dbias, void* workspace,
                                  int64_t workspace_bytes, int64_t V, int32_t C, void* stream);
+/* kerops_lin_brelu_lin_bwd_f16 with dWup, dWdown and dbias written as grad_dtype: KEROPS_DTYPE_F32, or
+ * KEROPS_DTYPE_F16 = the fp32 results rounded once by the reduction kernel (the reference returns fp16,
+ * kerops/ops/linear/linear_bias_relu_linear_backward.py:71-73). */
+int kerops_lin_brelu_lin_bwd_f16_out(const void* x, const void* g, const void* Wup, const void* Wdown, const void* bias,
+                                     void* dx, void* dWup, void* dWdown, void* dbias, int32_t grad_dtype,
+                                     void* workspace, int64_t workspace_bytes, int64_t V, int32_t C, void* stream);
 
 /* Fused depthwise-separable block (no single reference counterpart; composition
  * of DWConv, a folded inference BN, ReLU and the pointwise GEMM above):

@@ -21,7 +21,7 @@ KEROPS_E_LAUNCH = -4
 HEADER_VERSION = 210
 
 DTYPE_TAGS = {torch.float16: 0, torch.float32: 1, torch.bfloat16: 2}
-# result types the weight-gradient reduction kernel writes itself (kerops_dwconv_wgrad_f16_out, kerops_dwconv_bwd_f16_out)
+# result types the gradient reduction kernels write themselves (the *_f16_out entry points)
 GW_DTYPES = {torch.float16: 0, torch.float32: 1}
 
 _p = ctypes.c_void_p
@@ -71,8 +71,11 @@ SIGNATURES = {
     'kerops_lin_brelu_lin_add_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i32, _p]),
     'kerops_lin_brelu_lin_bwd_workspace_bytes': (_i64, [_i64, _i32]),
     'kerops_lin_brelu_lin_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _p]),
+    'kerops_lin_brelu_lin_bwd_f16_out': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i32,
+                                                        _p]),
     'kerops_relu_linear_bwd_workspace_bytes': (_i64, [_i64, _i32, _i32]),
     'kerops_relu_linear_bwd_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p]),
+    'kerops_relu_linear_bwd_f16_out': (ctypes.c_int, [_p, _p, _p, _p, _p, _i32, _p, _i64, _i64, _i32, _i32, _p]),
     'kerops_dwsep_block_workspace_bytes': (_i64, [_i32, _i32, _i32, _i32, _i32, _i32]),
     'kerops_dwsep_block_f16': (ctypes.c_int, [_p, _p, _p, _p, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _i32, _p,
                                               _i64, _p]),

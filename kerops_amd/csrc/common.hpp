@@ -671,5 +671,10 @@ __device__ __forceinline__ void block_channel_partials_any(float (&acc)[NACC][V]
 // columns [0, split) go to out0, the rest to out1.  (Kernel lives in core.hip.)
 void launch_reduce_rows(const float* ws, int nrows, int ncols, float* out0, float* out1, int split, double scale,
                         hipStream_t stream);
+// the same with the fp32 results rounded to fp16
+void launch_reduce_rows_f16(const float* ws, int nrows, int ncols, half_t* out0, half_t* out1, int split, double scale,
+                            hipStream_t stream);
+// result type of a gradient that a reduction kernel writes: fp32 or fp16
+inline bool grad_dtype_ok(int dtype) { return dtype == KEROPS_DTYPE_F32 || dtype == KEROPS_DTYPE_F16; }
 
 }  // namespace kerops

@@ -66,8 +66,10 @@ namespace kerops {
 // (columns below split) or out1.  A workgroup owns 16 columns; its 64 row slices take interleaved rows with four
 // loads in flight each (a single dependent chain over hundreds of rows took longer than the pass it finishes),
 // then the slices are combined by a fixed tree in LDS.
+// OutT: fp32, or fp16 = the fp32 result rounded once (what a cast of it gives, without the cast's launch).
+template <class OutT>
 __global__ __launch_bounds__(1024) void reduce_rows_kernel(const float* __restrict__ ws, int nrows, int ncols,
-                                                           float* __restrict__ out0, float* __restrict__ out1,
+                                                           OutT* __restrict__ out0, OutT* __restrict__ out1,
                                                            int split, double scale)
 {
     __shared__ double part[64][17];
@@ -96,9 +98,9 @@ __global__ __launch_bounds__(1024) void reduce_rows_kernel(const float* __restri
     if (sl == 0 && j < ncols) {
         const double v = part[0][lo] * scale;
         if (j < split) {
-            out0[j] = (float)v;
+            out0[j] = (OutT)(float)v;
         } else {
-            out1[j - split] = (float)v;
+            out1[j - split] = (OutT)(float)v;
         }
     }
 }
@@ -106,8 +108,15 @@ __global__ __launch_bounds__(1024) void reduce_rows_kernel(const float* __restri
 void launch_reduce_rows(const float* ws, int nrows, int ncols, float* out0, float* out1, int split, double scale,
                         hipStream_t stream)
 {
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3(ceil_div(ncols, 16)), dim3(1024), 0, stream, ws, nrows, ncols, out0,
-                       out1, split, scale);
+    hipLaunchKernelGGL(reduce_rows_kernel<float>, dim3(ceil_div(ncols, 16)), dim3(1024), 0, stream, ws, nrows, ncols,
+                       out0, out1, split, scale);
+}
+
+void launch_reduce_rows_f16(const float* ws, int nrows, int ncols, half_t* out0, half_t* out1, int split, double scale,
+                            hipStream_t stream)
+{
+    hipLaunchKernelGGL(reduce_rows_kernel<half_t>, dim3(ceil_div(ncols, 16)), dim3(1024), 0, stream, ws, nrows, ncols,
+                       out0, out1, split, scale);
 }
 
 }  // namespace kerops

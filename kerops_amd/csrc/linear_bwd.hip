@@ -212,15 +212,18 @@ static int lb_blocks(int64_t V)
 }
 
 template <int CIN, int COUT>
-static int launch_lb(const half_t* x, const half_t* g, const half_t* Wm, half_t* dx, float* dW, float* ws, int64_t V,
-                     hipStream_t s)
+static int launch_lb(const half_t* x, const half_t* g, const half_t* Wm, half_t* dx, void* dW, int dw_dtype, float* ws,
+                     int64_t V, hipStream_t s)
 {
     using Cfg = LbCfg<CIN, COUT>;
     const int blocks = lb_blocks(V);
     hipLaunchKernelGGL((relu_linear_bwd_kernel<CIN, COUT>), dim3(blocks), dim3(kLbThreads), 0, s, x, g, Wm, dx, ws, V);
     int rc = check_launch("relu_linear_bwd");
     if (rc != KEROPS_OK) return rc;
-    launch_reduce_rows(ws, blocks * Cfg::KSPL, CIN * COUT, dW, dW, CIN * COUT, 1.0, s);
+    if (dw_dtype == KEROPS_DTYPE_F16)
+        launch_reduce_rows_f16(ws, blocks * Cfg::KSPL, CIN * COUT, (half_t*)dW, (half_t*)dW, CIN * COUT, 1.0, s);
+    else
+        launch_reduce_rows(ws, blocks * Cfg::KSPL, CIN * COUT, (float*)dW, (float*)dW, CIN * COUT, 1.0, s);
     return check_launch("relu_linear_bwd_reduce");
 }
 
@@ -253,6 +256,18 @@ extern "C" int kerops_relu_linear_bwd_f16(const void* x, const void* g, const vo
                                           void* workspace, int64_t workspace_bytes, int64_t V, int32_t Cin,
                                           int32_t Cout, void* stream)
 {
+    return kerops_relu_linear_bwd_f16_out(x, g, Wm, dx, dW, KEROPS_DTYPE_F32, workspace, workspace_bytes, V, Cin, Cout,
+                                          stream);
+}
+
+extern "C" int kerops_relu_linear_bwd_f16_out(const void* x, const void* g, const void* Wm, void* dx, void* dW,
+                                              int32_t dw_dtype, void* workspace, int64_t workspace_bytes, int64_t V,
+                                              int32_t Cin, int32_t Cout, void* stream)
+{
+    if (!grad_dtype_ok(dw_dtype)) {
+        set_error("relu_linear_bwd: dw_dtype must be KEROPS_DTYPE_F32 or KEROPS_DTYPE_F16");
+        return KEROPS_E_BADARG;
+    }
     const int64_t need = kerops_relu_linear_bwd_workspace_bytes(V, Cin, Cout);
     if (need < 0) return (int)need;
     if (!x || !g || !Wm || !dx || !dW || !aligned16(x) || !aligned16(g) || !aligned16(Wm) || !aligned16(dx)) {
@@ -269,7 +284,7 @@ extern "C" int kerops_relu_linear_bwd_f16(const void* x, const void* g, const vo
     const half_t* wh = (const half_t*)Wm;
     hipStream_t s = (hipStream_t)stream;
 #define KEROPS_LB_CASE(CI, CO) \
-    if (Cin == CI && Cout == CO) return launch_lb<CI, CO>(xh, gh, wh, (half_t*)dx, dW, (float*)workspace, V, s);
+    if (Cin == CI && Cout == CO) return launch_lb<CI, CO>(xh, gh, wh, (half_t*)dx, dW, dw_dtype, (float*)workspace, V, s);
     KEROPS_LB_CASE(16, 16)
     KEROPS_LB_CASE(16, 32)
     KEROPS_LB_CASE(16, 64)

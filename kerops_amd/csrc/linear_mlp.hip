@@ -1097,9 +1097,11 @@ __global__ __launch_bounds__(kMlpThreads, 2) void lin_brelu_lin_bwd_tr_kernel(
 
 // sums the rows of the partial buffer in a fixed order (16 columns per workgroup, 64 interleaved row slices with four
 // loads in flight, fixed tree in LDS; fp64) and scatters the three results
+// (OutT: fp32, or fp16 = the fp32 results rounded once)
+template <class OutT>
 __global__ __launch_bounds__(1024) void mlp_reduce_kernel(const float* __restrict__ ws, int nrows, int RW, int n_up,
-                                                          int n_down, float* __restrict__ d_up,
-                                                          float* __restrict__ d_down, float* __restrict__ d_bias)
+                                                          int n_down, OutT* __restrict__ d_up,
+                                                          OutT* __restrict__ d_down, OutT* __restrict__ d_bias)
 {
     __shared__ double part[64][17];
     const int lo = threadIdx.x % 16, sl = threadIdx.x / 16;
@@ -1125,10 +1127,21 @@ __global__ __launch_bounds__(1024) void mlp_reduce_kernel(const float* __restric
     }
     if (sl == 0 && j < RW) {
         const double v = part[0][lo];
-        if (j < n_up) d_up[j] = (float)v;
-        else if (j < n_up + n_down) d_down[j - n_up] = (float)v;
-        else d_bias[j - n_up - n_down] = (float)v;
+        if (j < n_up) d_up[j] = (OutT)(float)v;
+        else if (j < n_up + n_down) d_down[j - n_up] = (OutT)(float)v;
+        else d_bias[j - n_up - n_down] = (OutT)(float)v;
     }
+}
+
+static void launch_mlp_reduce(const float* ws, int nrows, int RW, int n_up, int n_down, void* d_up, void* d_down,
+                              void* d_bias, int dtype, hipStream_t s)
+{
+    if (dtype == KEROPS_DTYPE_F16)
+        hipLaunchKernelGGL(mlp_reduce_kernel<half_t>, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws, nrows, RW, n_up,
+                           n_down, (half_t*)d_up, (half_t*)d_down, (half_t*)d_bias);
+    else
+        hipLaunchKernelGGL(mlp_reduce_kernel<float>, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws, nrows, RW, n_up,
+                           n_down, (float*)d_up, (float*)d_down, (float*)d_bias);
 }
 
 // workgroups and partial rows per workgroup
@@ -1169,6 +1182,19 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
                                             void* workspace, int64_t workspace_bytes, int64_t V, int32_t C,
                                             void* stream)
 {
+    return kerops_lin_brelu_lin_bwd_f16_out(x, g, Wup, Wdown, bias, dx, dWup, dWdown, dbias, KEROPS_DTYPE_F32, workspace,
+                                            workspace_bytes, V, C, stream);
+}
+
+extern "C" int kerops_lin_brelu_lin_bwd_f16_out(const void* x, const void* g, const void* Wup, const void* Wdown,
+                                                const void* bias, void* dx, void* dWup, void* dWdown, void* dbias,
+                                                int32_t grad_dtype, void* workspace, int64_t workspace_bytes, int64_t V,
+                                                int32_t C, void* stream)
+{
+    if (!grad_dtype_ok(grad_dtype)) {
+        set_error("lin_brelu_lin_bwd: grad_dtype must be KEROPS_DTYPE_F32 or KEROPS_DTYPE_F16");
+        return KEROPS_E_BADARG;
+    }
     const int64_t need = kerops_lin_brelu_lin_bwd_workspace_bytes(V, C);
     if (need < 0) return (int)need;
     if (!x || !g || !Wup || !Wdown || !bias || !dx || !dWup || !dWdown || !dbias || !aligned16(x) || !aligned16(g) ||
@@ -1192,8 +1218,7 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
         int rc = check_launch("lin_brelu_lin_bwd");                                                               \
         if (rc != KEROPS_OK) return rc;                                                                           \
         const int RW = MtCfg<CV>::RW;                                                                             \
-        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws, blocks, RW,           \
-                           2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);                                        \
+        launch_mlp_reduce(ws, blocks, RW, 2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias, grad_dtype, s);          \
         return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
     }
     KEROPS_MT_CASE(16)
@@ -1208,8 +1233,7 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
         int rc = check_launch("lin_brelu_lin_bwd");
         if (rc != KEROPS_OK) return rc;
         const int RW = MrCfg::RW;
-        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws, blocks, RW, 2 * 32 * 32,
-                           2 * 32 * 32, dWup, dWdown, dbias);
+        launch_mlp_reduce(ws, blocks, RW, 2 * 32 * 32, 2 * 32 * 32, dWup, dWdown, dbias, grad_dtype, s);
         return check_launch("lin_brelu_lin_bwd_reduce");
     }
 #define KEROPS_MB_CASE(CV)                                                                                        \
@@ -1220,8 +1244,8 @@ extern "C" int kerops_lin_brelu_lin_bwd_f16(const void* x, const void* g, const 
         int rc = check_launch("lin_brelu_lin_bwd");                                                               \
         if (rc != KEROPS_OK) return rc;                                                                           \
         const int RW = MbCfg<CV>::RW;                                                                             \
-        hipLaunchKernelGGL(mlp_reduce_kernel, dim3(ceil_div(RW, 16)), dim3(1024), 0, s, ws,                      \
-                           blocks * MbCfg<CV>::KSPL, RW, 2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias);          \
+        launch_mlp_reduce(ws, blocks * MbCfg<CV>::KSPL, RW, 2 * CV * CV, 2 * CV * CV, dWup, dWdown, dbias,        \
+                          grad_dtype, s);                                                                         \
         return check_launch("lin_brelu_lin_bwd_reduce");                                                          \
     }
     KEROPS_MB_CASE(64)

@@ -43,13 +43,16 @@ def LinBReLULinBackward(x, grad, weight_up, weight_down, bias, *, num_warps: Con
     ws_bytes = _lib.query('kerops_lin_brelu_lin_bwd_workspace_bytes', V, in_channels)
     ws = _lib.workspace(ws_bytes, x.device)
     x_grad = torch.empty_like(x)
-    f32 = dict(dtype=torch.float32, device=x.device)
-    up_grad = torch.empty([in_channels, hidden_channels], **f32)
-    down_grad = torch.empty([hidden_channels, in_channels], **f32)
-    bias_grad = torch.empty([hidden_channels], **f32)
-    _lib.call('kerops_lin_brelu_lin_bwd_f16', x.data_ptr(), grad.data_ptr(), weight_up.data_ptr(),
+    # fp32 and fp16 results are written by the library's reduction kernel; any other type is cast from fp32
+    direct = out_dtype in _lib.GW_DTYPES
+    res = dict(dtype=out_dtype if direct else torch.float32, device=x.device)
+    up_grad = torch.empty([in_channels, hidden_channels], **res)
+    down_grad = torch.empty([hidden_channels, in_channels], **res)
+    bias_grad = torch.empty([hidden_channels], **res)
+    _lib.call('kerops_lin_brelu_lin_bwd_f16_out', x.data_ptr(), grad.data_ptr(), weight_up.data_ptr(),
               weight_down.data_ptr(), bias.data_ptr(), x_grad.data_ptr(), up_grad.data_ptr(), down_grad.data_ptr(),
-              bias_grad.data_ptr(), ws.data_ptr(), ws_bytes, V, in_channels, _lib.stream_of(x))
-    if out_dtype != torch.float32:
+              bias_grad.data_ptr(), _lib.GW_DTYPES[res['dtype']], ws.data_ptr(), ws_bytes, V, in_channels,
+              _lib.stream_of(x))
+    if not direct:
         up_grad, down_grad, bias_grad = up_grad.to(out_dtype), down_grad.to(out_dtype), bias_grad.to(out_dtype)
     return x_grad, up_grad, down_grad, bias_grad

@@ -69,7 +69,11 @@ def ReLULinearBackward(
     ws_bytes = _lib.query('kerops_relu_linear_bwd_workspace_bytes', V, in_channels, out_channels)
     ws = _lib.workspace(ws_bytes, x.device)
     x_grad = torch.empty_like(x)
-    weight_grad = torch.empty([in_channels, out_channels], dtype=torch.float32, device=x.device)
-    _lib.call('kerops_relu_linear_bwd_f16', x.data_ptr(), grad.data_ptr(), weight.data_ptr(), x_grad.data_ptr(),
-              weight_grad.data_ptr(), ws.data_ptr(), ws_bytes, V, in_channels, out_channels, _lib.stream_of(x))
-    return x_grad, (weight_grad if out_dtype == torch.float32 else weight_grad.to(out_dtype))
+    # fp32 and fp16 results are written by the library's reduction kernel; any other type is cast from fp32
+    direct = out_dtype in _lib.GW_DTYPES
+    weight_grad = torch.empty([in_channels, out_channels], dtype=out_dtype if direct else torch.float32,
+                              device=x.device)
+    _lib.call('kerops_relu_linear_bwd_f16_out', x.data_ptr(), grad.data_ptr(), weight.data_ptr(), x_grad.data_ptr(),
+              weight_grad.data_ptr(), _lib.GW_DTYPES[weight_grad.dtype], ws.data_ptr(), ws_bytes, V, in_channels,
+              out_channels, _lib.stream_of(x))
+    return x_grad, (weight_grad if direct else weight_grad.to(out_dtype))

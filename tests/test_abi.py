@@ -58,6 +58,11 @@ def test_argument_validation_needs_no_device():
     assert rc == _lib.KEROPS_E_BADARG and 'gw_dtype' in _lib.last_error()
     rc = lib.kerops_dwconv_wgrad_f16_out(addr, addr, addr, 0, addr, 16, 1, 4, 4, 4, 64, 0, 0, 0, 0, None)
     assert rc == _lib.KEROPS_E_WORKSPACE
+    rc = lib.kerops_relu_linear_bwd_f16_out(addr, addr, addr, addr, addr, 2, addr, 1 << 30, 64, 32, 32, None)
+    assert rc == _lib.KEROPS_E_BADARG and 'dw_dtype' in _lib.last_error()
+    rc = lib.kerops_lin_brelu_lin_bwd_f16_out(addr, addr, addr, addr, addr, addr, addr, addr, addr, -1, addr, 1 << 30,
+                                              64, 32, None)
+    assert rc == _lib.KEROPS_E_BADARG and 'grad_dtype' in _lib.last_error()
     rc = lib.kerops_stats_f16(addr, addr, addr, 64, 1024, addr, 1 << 30, 0, 0, 0, None)
     assert rc == _lib.KEROPS_E_UNSUPPORTED_C
     rc = lib.kerops_stats_f16(addr, addr, addr, 64, 12, addr, 1 << 30, 0, 0, 0, None)

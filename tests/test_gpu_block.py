@@ -75,6 +75,10 @@ def test_relu_linear_backward_matches_oracle(cin, cout, spatial):
     grad = rand_cl3d(g, n, cout, h, w, d)
     Wm = rand_pw(g, cin, cout)
     dx, dw = ReLULinearBackward(x.to(DEV), grad.to(DEV), Wm.to(DEV), out_dtype=torch.float32)
+    # default result type fp16, written by the reduction kernel = the fp32 result rounded once; same dx
+    dx16, dw16 = ReLULinearBackward(x.to(DEV), grad.to(DEV), Wm.to(DEV))
+    assert dw16.dtype == torch.float16 and torch.equal(dx16, dx)
+    assert torch.equal(dw16.view(torch.int16), dw.to(torch.float16).view(torch.int16))
     dx, dw = dx.cpu(), dw.cpu()
     ref_dx, ref_dw = oracle.relu_linear_bwd(x, grad, Wm)
     assert dx.shape == x.shape and dx.stride() == x.stride() and dw.shape == (cin, cout)
@@ -165,6 +169,12 @@ def test_lin_brelu_lin_backward_matches_oracle(c, spatial):
     bias = (torch.randn(2 * c, generator=g) * 0.5).half()
     dev = [t_.to(DEV) for t_ in (x, grad, Wup, Wdown, bias)]
     dx, dup, ddn, db = (t_.cpu() for t_ in LinBReLULinBackward(*dev, out_dtype=torch.float32))
+    # default result type fp16, written by the reduction kernel = the fp32 results rounded once; same dx
+    got16 = [t_.cpu() for t_ in LinBReLULinBackward(*dev)]
+    assert torch.equal(got16[0], dx)
+    for h16, f32 in zip(got16[1:], (dup, ddn, db)):
+        assert h16.dtype == torch.float16 and h16.shape == f32.shape
+        assert torch.equal(h16.view(torch.int16), f32.to(torch.float16).view(torch.int16))
     rdx, rup, rdn, rdb = oracle.lin_brelu_lin_bwd(x, grad, Wup, Wdown, bias)
     assert dx.shape == x.shape and dx.stride() == x.stride()
     assert dup.shape == (c, 2 * c) and ddn.shape == (2 * c, c) and db.shape == (2 * c,)
