@@ -18,6 +18,19 @@ struct PoolDims {
     int N, H, W, D, Ho, Wo, Do, C, CG;
 };
 
+// acc + float(half SEL of the packed pair), one instruction (the mixed-precision fused multiply-add with the factor
+// 1.0: the product is exact, the sum is rounded once, i.e. the bits of a conversion followed by an addition)
+template <int SEL>
+__device__ __forceinline__ float add_half_of(uint32_t pair, float acc)
+{
+    float r;
+    if constexpr (SEL == 0)
+        asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pair), "v"(acc));
+    else
+        asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pair), "v"(acc));
+    return r;
+}
+
 // BNRELU: every voxel that exists is first mapped to fp16(max(x * bw[c] + bb[c], 0)), exactly what
 // bnrelu_fwd_kernel would have stored, so the fused op equals ApplyBNReLU followed by the pool bit for bit
 // while the full-size intermediate is neither written nor read.
@@ -90,6 +103,9 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_fwd_kernel(const ha
     };
     auto finish_window = [&](int64_t i, Window& wn) {
         if (BNRELU) {
+            hv zero;
+#pragma unroll
+            for (int j = 0; j < V; ++j) zero[j] = (half_t)0;
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -97,27 +113,61 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_fwd_kernel(const ha
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
                         const bool ok = (a == 0 || wn.h1) && (b == 0 || wn.w1) && (e == 0 || wn.d1);
+                        // fp16(max(v, 0)) = max(fp16(v), 0): rounding keeps the sign and the order, so the ReLU runs
+                        // on the rounded pairs (one packed instruction for two channels)
+                        // (fp16 of the fp32 result, as ApplyBNReLU stores it: two roundings)
+                        hv r;
 #pragma unroll
-                        for (int j = 0; j < V; ++j) {
-                            const half_t r =
-                                (half_t)fmaxf(__builtin_fmaf((float)wn.v[a][b][e][j], cw[j], cb[j]), 0.0f);
-                            wn.v[a][b][e][j] = ok ? r : (half_t)0;
-                        }
+                        for (int j = 0; j < V; ++j)
+                            r[j] = (half_t)as_fp32_value(__builtin_fmaf((float)wn.v[a][b][e][j], cw[j], cb[j]));
+                        if constexpr (V >= 2) r = __builtin_elementwise_max(r, zero);
+                        else r[0] = r[0] > (half_t)0 ? r[0] : (half_t)0;
+                        wn.v[a][b][e] = ok ? r : zero;
                     }
         }
-        const float cnt = (float)((wn.h1 ? 2 : 1) * (wn.w1 ? 2 : 1) * (wn.d1 ? 2 : 1));
+        // the window holds 2^k voxels, k = 0..3: the product with 2^-k (built from its exponent bits) is the
+        // correctly rounded quotient
+        const uint32_t k = (uint32_t)wn.h1 + (uint32_t)wn.w1 + (uint32_t)wn.d1;
+        const float inv = __builtin_bit_cast(float, (127u - k) << 23);
         hv o;
-#pragma unroll
-        for (int j = 0; j < V; ++j) {
-            float s = 0.0f;
+        if constexpr (V >= 2) {
+            // a (h, w) row: the two D taps of a channel are float(tap 0) + float(tap 1), the second conversion and the
+            // addition in one instruction
+            uint32_t wd[2][2][2][V / 2];
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
-                for (int b = 0; b < 2; ++b) s += (float)wn.v[a][b][0][j] + (float)wn.v[a][b][1][j];
-            const float m = __fdiv_rn(s, cnt);
-            o[j] = (half_t)m;
-            acc[0][j] += m;
-            acc[1][j] = __builtin_fmaf(m, m, acc[1][j]);
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) __builtin_memcpy(wd[a][b][e], &wn.v[a][b][e], V * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                float s = 0.0f;
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        const float t0 = (float)wn.v[a][b][0][j];
+                        s += (j % 2 == 0) ? add_half_of<0>(wd[a][b][1][j / 2], t0) : add_half_of<1>(wd[a][b][1][j / 2], t0);
+                    }
+                const float m = s * inv;
+                o[j] = (half_t)m;
+                acc[0][j] += m;
+                acc[1][j] = __builtin_fmaf(m, m, acc[1][j]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                float s = 0.0f;
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) s += (float)wn.v[a][b][0][j] + (float)wn.v[a][b][1][j];
+                const float m = s * inv;
+                o[j] = (half_t)m;
+                acc[0][j] += m;
+                acc[1][j] = __builtin_fmaf(m, m, acc[1][j]);
+            }
         }
         st_stream<V>(y, i, o);
     };

@@ -22,6 +22,16 @@ typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+// An fp32 result that is about to be rounded to fp16, made opaque to the compiler.  Where results are specified as
+// fp16(fp32 value) (two roundings, what the reference's kernels and the oracle compute), the product or fused
+// multiply-add must exist as an fp32 value first: left alone, the compiler may merge it with the conversion into
+// v_fma_mixlo_f16 / v_fma_mixhi_f16, which round the exact result once and differ in the last bit in rare cases.
+__device__ __forceinline__ float as_fp32_value(float f)
+{
+    asm("" : "+v"(f));
+    return f;
+}
 typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));

@@ -88,6 +88,23 @@ def test_bnrelu_and_backward(shape):
     assert close64(dW.flatten(), rdW, 1e-5) and close64(dB.flatten(), rdB, 1e-5)
 
 
+@pytest.mark.parametrize('c', [1, 2, 8, 64])
+def test_fp16_results_are_fp16_of_the_fp32_value(c):
+    """dx of ApplyBNReLUBackward is fp16(w * g computed in fp32), the pooled BN-ReLU values are fp16(fp32 fma): two
+    roundings, as the reference's kernels and the oracle compute them.  A mixed-precision instruction that rounds the
+    exact product once differs in about one value per 10^5; half a million values per case make that visible."""
+    g = cpu_gen(40 + c)
+    shape = (1, c, 32, 128, 128 // c) if c > 1 else (1, 1, 32, 128, 128)
+    x = rand_cl3d(g, *shape)
+    W = torch.randn(c, generator=g) * 1.7 + 0.3
+    B = torch.randn(c, generator=g)
+    grad = rand_cl3d(g, *shape)
+    dx = ApplyBNReLUBackward(x.to(DEV), W.to(DEV), B.to(DEV), grad.to(DEV))[0]
+    assert bits_equal(dx, oracle.bnrelu_bwd(x, W, B, grad)[0])
+    yp = ApplyBNReLUAvgPoolCeilStats(x.to(DEV), W.to(DEV), B.to(DEV))[0]
+    assert bits_equal(yp, oracle.avgpool_ceil_stats(oracle.bnrelu_fwd(x, W, B))[0])
+
+
 def _grid_sample(n, seed):
     """Deterministic sample of the reference's test grid (tests/conftest.py:4-36): channels {2,4,8,16,32}, batch
     1-4, extents from {2,3,7,13,16,32,37,53,111,128}; bounded in size."""
