@@ -179,7 +179,9 @@ __global__ __launch_bounds__(kStreamMaxThreads) void bnrelu_bwd_kernel(const hal
         for (int j = 0; j < V; ++j) {
             const float xf = (float)xv[j];
             const float gm = __fmul_rn((float)gv[j], (__fmul_rn(xf, w[j]) > nb[j]) ? 1.0f : 0.0f);  // keeps the sign of zero
-            o[j] = (half_t)as_fp32_value(__fmul_rn(w[j], gm));
+            // (one channel per lane: the compiler would otherwise round the exact product once; with two and more it
+            // converts pairs of fp32 products, and the opaque value only costs registers)
+            o[j] = (half_t)(V == 1 ? as_fp32_value(__fmul_rn(w[j], gm)) : __fmul_rn(w[j], gm));
             acc[0][j] = __builtin_fmaf(xf, gm, acc[0][j]);
             acc[1][j] += gm;
         }
