@@ -660,8 +660,15 @@ __device__ __forceinline__ void dwconv_fwd_mfma_segment(const FwdArgs& a, unsign
             *reinterpret_cast<half8_t*>(dst) = xpre[j];
         }
         __syncthreads();
-        flush_row(parity ^ 1);
+        // The loads of the next plane go out first and at raised wave priority, the stores of the finished plane
+        // after them at the normal one: the memory instructions of the wavefronts of a compute unit share one issue
+        // path, and loads queued behind other wavefronts' stores reach memory late (measured at C = 64: 0.703 ->
+        // 0.694 ms; the same order without the priority, or the priority without the order, changes nothing).
+        __builtin_amdgcn_s_setprio(3);
         prefetch(hp + AHEAD, xpre);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(0);
+        flush_row(parity ^ 1);
         __builtin_amdgcn_sched_barrier(0);  // the loads stay ahead of the arithmetic that hides their latency
         if (xin) {
 #pragma unroll
