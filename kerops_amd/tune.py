@@ -18,6 +18,7 @@ live table of `kerops_amd.settings.stream_table` under a key (a channel count, "
 stream ops read on every call.
 """
 import argparse
+import time
 import math
 
 import torch
@@ -27,9 +28,16 @@ from .ops.conv.variants import FWD_VARIANTS, WGRAD_VARIANTS, threads_per_workgro
 
 
 def _time(fn, iters, warmup):
+    # at least `warmup` launches and 30 ms of back-to-back launches: the core clock needs that long to settle after an
+    # idle gap, and a 0.1 ms kernel timed on the ramp loses to one timed after it
+    t0 = time.perf_counter()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    while time.perf_counter() - t0 < 0.03:
+        for _ in range(max(warmup, 5)):
+            fn()
+        torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
     for a, b in evs:
         a.record()
