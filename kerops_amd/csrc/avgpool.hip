@@ -288,8 +288,8 @@ __global__ __launch_bounds__(kStreamMaxThreads) void avgpool_bwd_kernel(const ha
 struct PoolDefault {
     int blocks, waves, segment;
 };
-constexpr PoolDefault kDefPoolFwd{256, 4, 2};
-constexpr PoolDefault kDefPoolFwdBnRelu{512, 4, 1};
+constexpr PoolDefault kDefPoolFwd{256, 4, 1};
+constexpr PoolDefault kDefPoolFwdBnRelu{256, 4, 2};
 constexpr PoolDefault kDefPoolBwd{256, 4, 1};
 constexpr int kMaxDefaultBlocks = 4096;  // workspace queries with blocks = 0 size for this many partials
 

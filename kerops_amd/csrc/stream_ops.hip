@@ -452,11 +452,11 @@ struct StreamDefault {
     int blocks, waves, segment;
 };
 constexpr StreamDefault kDefStats{256, 4, 8};
-constexpr StreamDefault kDefAddStats{256, 4, 1};
+constexpr StreamDefault kDefAddStats{1280, 16, 8};
 constexpr StreamDefault kDefStatsBwd{4096, 16, 4};
 constexpr StreamDefault kDefAddStatsBwd{512, 4, 4};
-constexpr StreamDefault kDefBnReluFwd{4096, 16, 4};
-constexpr StreamDefault kDefBnReluBwd{1280, 16, 4};
+constexpr StreamDefault kDefBnReluFwd{1280, 16, 4};
+constexpr StreamDefault kDefBnReluBwd{1536, 16, 4};
 constexpr StreamDefault kDefQuantU8{256, 4, 8};
 constexpr StreamDefault kDefDequantU8{512, 4, 4};
 constexpr StreamDefault kDefQuantI8{4096, 16, 4};
